@@ -1,0 +1,49 @@
+"""Compile the HIP sources in ``csrc/`` into ``libajq.so`` next to this file.
+
+Cross-compiles for gfx950 with hipcc; needs no GPU.  Run as
+``python -m ajllm_amd.build`` or call :func:`build_library`.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PACKAGE_DIR = Path(__file__).resolve().parent
+SOURCE = PACKAGE_DIR / "csrc" / "ajq.hip"
+LIBRARY = PACKAGE_DIR / "libajq.so"
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def build_library(verbose: bool = False) -> Path:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    tmp = LIBRARY.with_suffix(".so.tmp%d" % os.getpid())
+    cmd = [hipcc, *HIPCC_FLAGS, str(SOURCE), "-o", str(tmp)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    stderr = "\n".join(line for line in proc.stderr.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        tmp.unlink(missing_ok=True)
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{stderr}")
+    if stderr.strip() and verbose:
+        print(stderr, file=sys.stderr)
+    os.replace(tmp, LIBRARY)
+    return LIBRARY
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

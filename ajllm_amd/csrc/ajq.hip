@@ -1,0 +1,252 @@
+// C ABI of libajq.so: argument validation, launch geometry, error reporting.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "ajq_common.h"
+
+#include "quantize_kernels.h"
+#include "gemv_kernels.h"
+#include "gemm_kernels.h"
+
+using namespace ajq;
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(AJQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return AJQ_OK;
+}
+
+constexpr int kMaxGemvM = 16;
+constexpr size_t kGemvLdsBudget = 128 * 1024;  // bytes of LDS for the staged activations
+constexpr int kGemmMpadTo = 256;
+
+int round_up(int v, int to) { return (v + to - 1) / to * to; }
+
+// Largest K chunk (multiple of 128) whose M staged rows fit the LDS budget.
+int gemv_kchunk(int M, int K) {
+  long long per_k = 2LL * M;  // bytes per k column
+  long long fit = ((long long)kGemvLdsBudget - 16LL * M) / per_k;
+  fit = fit / 128 * 128;
+  if (fit < 128) fit = 128;
+  return (int)(fit < K ? fit : K);
+}
+
+template <typename Kernel>
+int allow_big_lds(Kernel kernel, size_t bytes) {
+  if (bytes <= 64 * 1024) return AJQ_OK;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) return fail(AJQ_ERR_HIP, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
+  return AJQ_OK;
+}
+
+int check_matmul_args(const char* name, const void* x, int M, int K, const void* wq, const void* aux, int N,
+                      const void* y, int out_dtype, int k_multiple) {
+  if (!x || !wq || !aux || !y) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (M < 1 || N < 1 || K < 1) return fail(AJQ_ERR_SHAPE, "%s: M, N, K must be positive (got %d, %d, %d)", name, M, N, K);
+  if (K % k_multiple != 0) return fail(AJQ_ERR_SHAPE, "%s: K=%d must be a multiple of %d", name, K, k_multiple);
+  if (N % kTileN != 0) return fail(AJQ_ERR_SHAPE, "%s: N=%d must be a multiple of %d", name, N, kTileN);
+  if (out_dtype != AJQ_OUT_BF16 && out_dtype != AJQ_OUT_F32)
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: out_dtype %d is neither AJQ_OUT_BF16 nor AJQ_OUT_F32", name, out_dtype);
+  if (!aligned16(x) || !aligned16(wq) || !aligned16(y))
+    return fail(AJQ_ERR_ALIGN, "%s: x, wq and y must be 16-byte aligned", name);
+  return AJQ_OK;
+}
+
+template <int BM, int BN, int WM, int WN, bool kW4>
+int launch_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                       const uint16_t* scales8, const float* gsum, int Mpad, int N, void* y, int out_f32,
+                       hipStream_t stream) {
+  constexpr int kThreads = (BM / WM) * (BN / WN) * 64;
+  const size_t lds = (size_t)2 * BM * (128 + 8) * 2;
+  auto kernel = dequant_gemm_kernel<BM, BN, WM, WN, kW4>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), lds, stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8, gsum, Mpad, N, y, out_f32);
+  return AJQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ajq_version(void) { return 1; }
+
+const char* ajq_last_error(void) { return g_error; }
+
+const char* ajq_status_string(int status) {
+  switch (status) {
+    case AJQ_OK: return "ok";
+    case AJQ_ERR_NULL: return "null pointer";
+    case AJQ_ERR_SHAPE: return "unsupported shape";
+    case AJQ_ERR_ALIGN: return "misaligned pointer";
+    case AJQ_ERR_UNSUPPORTED: return "unsupported option";
+    case AJQ_ERR_HIP: return "HIP runtime error";
+    case AJQ_ERR_WORKSPACE: return "workspace missing or too small";
+    default: return "unknown status";
+  }
+}
+
+int ajq_quantize_w8(const float* W, int N, int K, int8_t* q, uint16_t* scales, void* stream) {
+  if (!W || !q || !scales) return fail(AJQ_ERR_NULL, "ajq_quantize_w8: null pointer argument");
+  if (N < 1 || K < 4 || K % 4 != 0)
+    return fail(AJQ_ERR_SHAPE, "ajq_quantize_w8: need N >= 1 and K a positive multiple of 4 (got N=%d, K=%d)", N, K);
+  if (!aligned16(W) || (reinterpret_cast<uintptr_t>(q) & 3u))
+    return fail(AJQ_ERR_ALIGN, "ajq_quantize_w8: W must be 16-byte and q 4-byte aligned");
+  hipLaunchKernelGGL(quantize_w8_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, W, K, q, scales);
+  return check_launch("ajq_quantize_w8");
+}
+
+int ajq_quantize_w4_g128(const float* W, int N, int K, int32_t* qweight, uint16_t* scales, uint8_t* zeros,
+                         void* stream) {
+  if (!W || !qweight || !scales || !zeros) return fail(AJQ_ERR_NULL, "ajq_quantize_w4_g128: null pointer argument");
+  if (N < 1 || K < kGroup || K % kGroup != 0)
+    return fail(AJQ_ERR_SHAPE, "ajq_quantize_w4_g128: need N >= 1 and K a positive multiple of 128 (got N=%d, K=%d)", N, K);
+  if (!aligned16(W)) return fail(AJQ_ERR_ALIGN, "ajq_quantize_w4_g128: W must be 16-byte aligned");
+  const long long groups = (long long)N * (K / kGroup);
+  const long long blocks = (groups + 15) / 16;
+  if (blocks > 0x7FFFFFFFLL) return fail(AJQ_ERR_SHAPE, "ajq_quantize_w4_g128: too many groups");
+  hipLaunchKernelGGL(quantize_w4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, W, groups,
+                     qweight, scales, zeros);
+  return check_launch("ajq_quantize_w4_g128");
+}
+
+static int check_repack(const char* name, const void* a, const void* b, int N, int K, int kmul) {
+  if (!a || !b) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (N < kTileN || N % kTileN != 0 || K < kmul || K % kmul != 0)
+    return fail(AJQ_ERR_SHAPE, "%s: need N a multiple of 16 and K a multiple of %d (got N=%d, K=%d)", name, kmul, N, K);
+  return AJQ_OK;
+}
+
+int ajq_repack_w4(const int32_t* qweight, const uint16_t* scales, const uint8_t* zeros, int N, int K,
+                  uint32_t* wq, uint32_t* meta, void* stream) {
+  if (int s = check_repack("ajq_repack_w4", qweight, wq, N, K, kGroup)) return s;
+  if (!scales || !zeros || !meta) return fail(AJQ_ERR_NULL, "ajq_repack_w4: null pointer argument");
+  const long long words = (long long)N * (K / 8);
+  hipLaunchKernelGGL(repack_w4_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const uint32_t*>(qweight), N, K, wq);
+  const long long metas = (long long)N * (K / kGroup);
+  hipLaunchKernelGGL(repack_w4_meta_kernel, dim3((unsigned)((metas + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, scales, zeros, N, K / kGroup, meta);
+  return check_launch("ajq_repack_w4");
+}
+
+int ajq_unrepack_w4(const uint32_t* wq, const uint32_t* meta, int N, int K, int32_t* qweight, uint16_t* scales,
+                    uint8_t* zeros, void* stream) {
+  if (int s = check_repack("ajq_unrepack_w4", wq, qweight, N, K, kGroup)) return s;
+  if (!scales || !zeros || !meta) return fail(AJQ_ERR_NULL, "ajq_unrepack_w4: null pointer argument");
+  const long long words = (long long)N * (K / 8);
+  hipLaunchKernelGGL(unrepack_w4_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     wq, N, K, reinterpret_cast<uint32_t*>(qweight));
+  const long long metas = (long long)N * (K / kGroup);
+  hipLaunchKernelGGL(unrepack_w4_meta_kernel, dim3((unsigned)((metas + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, meta, N, K / kGroup, scales, zeros);
+  return check_launch("ajq_unrepack_w4");
+}
+
+int ajq_repack_w8(const int8_t* q, int N, int K, uint32_t* wq, void* stream) {
+  if (int s = check_repack("ajq_repack_w8", q, wq, N, K, kW8TileK)) return s;
+  if (reinterpret_cast<uintptr_t>(q) & 3u) return fail(AJQ_ERR_ALIGN, "ajq_repack_w8: q must be 4-byte aligned");
+  const long long words = (long long)N * (K / 4);
+  hipLaunchKernelGGL(repack_w8_kernel<false>, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, reinterpret_cast<const uint32_t*>(q), N, K, wq);
+  return check_launch("ajq_repack_w8");
+}
+
+int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream) {
+  if (int s = check_repack("ajq_unrepack_w8", wq, q, N, K, kW8TileK)) return s;
+  if (reinterpret_cast<uintptr_t>(q) & 3u) return fail(AJQ_ERR_ALIGN, "ajq_unrepack_w8: q must be 4-byte aligned");
+  const long long words = (long long)N * (K / 4);
+  hipLaunchKernelGGL(repack_w8_kernel<true>, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, wq, N, K, reinterpret_cast<uint32_t*>(q));
+  return check_launch("ajq_unrepack_w8");
+}
+
+// --------------------------------------------------------------- GEMV -----
+int ajq_w4a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                   int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemv", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  if (M > kMaxGemvM) return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemv: M=%d exceeds %d; use ajq_w4a16_gemm", M, kMaxGemvM);
+  constexpr int kWaves = 8;
+  const int kchunk = gemv_kchunk(M, K);
+  const size_t lds = (size_t)M * (kchunk + 8) * 2 + (size_t)kWaves * 64 * 16;
+  auto kernel = w4a16_gemv_kernel<kWaves>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, (hipStream_t)stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, N, y, out_dtype == AJQ_OUT_F32, kchunk);
+  return check_launch("ajq_w4a16_gemv");
+}
+
+int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                   int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemv", x, M, K, wq, scales, N, y, out_dtype, kW8TileK)) return s;
+  if (M > kMaxGemvM) return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemv: M=%d exceeds %d; use ajq_w8a16_gemm", M, kMaxGemvM);
+  constexpr int kWaves = 8;
+  const int kchunk = gemv_kchunk(M, K);
+  const size_t lds = (size_t)M * (kchunk + 8) * 2 + (size_t)kWaves * 64 * 16;
+  auto kernel = w8a16_gemv_kernel<kWaves>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, (hipStream_t)stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), scales, N, y, out_dtype == AJQ_OUT_F32, kchunk);
+  return check_launch("ajq_w8a16_gemv");
+}
+
+// --------------------------------------------------------------- GEMM -----
+size_t ajq_w4a16_gemm_workspace_bytes(int M, int K) {
+  if (M < 1 || K < kGroup) return 0;
+  return (size_t)(K / kGroup) * round_up(M, kGemmMpadTo) * sizeof(float);
+}
+
+int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                   int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemm", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
+  if (!workspace || workspace_bytes < need)
+    return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm: workspace must be 16-byte aligned");
+  const int Mpad = round_up(M, kGemmMpadTo);
+  float* gsum = reinterpret_cast<float*>(workspace);
+  const long long teams = (long long)M * (K / kGroup);
+  hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
+                     K, Mpad, gsum);
+  int s;
+  if (M <= 64)
+    s = launch_gemm<64, 64, 32, 32, true>(x, M, K, wq, meta, nullptr, gsum, Mpad, N, y, out_dtype == AJQ_OUT_F32,
+                                          (hipStream_t)stream);
+  else
+    s = launch_gemm<128, 128, 64, 64, true>(x, M, K, wq, meta, nullptr, gsum, Mpad, N, y,
+                                            out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
+  if (s) return s;
+  return check_launch("ajq_w4a16_gemm");
+}
+
+int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                   int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemm", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
+  int s;
+  if (M <= 64)
+    s = launch_gemm<64, 64, 32, 32, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,
+                                           out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
+  else
+    s = launch_gemm<128, 128, 64, 64, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,
+                                             out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
+  if (s) return s;
+  return check_launch("ajq_w8a16_gemm");
+}
+
+}  // extern "C"

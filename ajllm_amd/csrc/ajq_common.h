@@ -1,0 +1,67 @@
+// Shared device helpers for the gfx950 quantized-linear kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/ajq.h"
+
+namespace ajq {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kGroup = 128;      // int4 quantization group along K
+constexpr int kTileN = 16;       // rows of one private-layout tile
+constexpr int kW8TileK = 64;     // k extent of one private W8 tile
+
+// D[16x16] += A[16x32] * B[32x16], bf16 in, fp32 accumulate.
+// lane l supplies A[row l%16][k 8*(l/16)..+8) and B[k 8*(l/16)..+8)][col l%16];
+// it receives D[row 4*(l/16)+i][col l%16] in component i.
+__device__ __forceinline__ f32x4_t mfma16(u32x4_t a, u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// One private W4 dword (8 nibbles, weight e in nibble (e>>1)+4*(e&1)) -> 8 bf16
+// holding 128+q exactly: 0x4300 is bf16(128) and its ulp is 1.
+__device__ __forceinline__ u32x4_t w4_to_bf16_biased(uint32_t w) {
+  u32x4_t r;
+  r.x = (w & 0x000F000Fu) | 0x43004300u;
+  r.y = ((w >> 4) & 0x000F000Fu) | 0x43004300u;
+  r.z = ((w >> 8) & 0x000F000Fu) | 0x43004300u;
+  r.w = ((w >> 12) & 0x000F000Fu) | 0x43004300u;
+  return r;
+}
+
+// Four int8 (one dword, k order) -> two dwords of bf16 pairs, exact.
+__device__ __forceinline__ u32x2_t w8_to_bf16(uint32_t w) {
+  float f0 = (float)(int8_t)(w & 0xFF);
+  float f1 = (float)(int8_t)((w >> 8) & 0xFF);
+  float f2 = (float)(int8_t)((w >> 16) & 0xFF);
+  float f3 = (float)(int8_t)(w >> 24);
+  u32x2_t r;
+  // |q| <= 127 has at most 7 significant bits: the high half of the fp32 is the bf16.
+  r.x = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+  r.y = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+  return r;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
+  return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+// fp32 -> bf16 bits, round to nearest even (inputs are finite sums).
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7F800000u) == 0x7F800000u) {  // inf / nan: keep class
+    return (uint16_t)((u >> 16) | ((u & 0xFFFFu) ? 0x40u : 0u));
+  }
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+}  // namespace ajq

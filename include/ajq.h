@@ -1,0 +1,108 @@
+/*
+ * ajq -- MI355X (gfx950) quantized linear: quantize/pack, decode GEMV, prefill GEMM.
+ *
+ * C ABI of libajq.so.  Every pointer is a DEVICE pointer owned by the caller
+ * (in practice a PyTorch-ROCm tensor's data_ptr); the library never allocates,
+ * frees or keeps a pointer past the call.  Every compute entry point is
+ * asynchronous: it enqueues on `stream` (a hipStream_t, e.g.
+ * torch.cuda.current_stream().cuda_stream; NULL = the default stream) and
+ * returns without a host sync.  Return value: 0 on success, a negative
+ * ajq_status otherwise; ajq_last_error() gives the thread-local message.
+ *
+ * The reference project (Huangsj1/ajLLM) has exactly one linear operator,
+ *     Linear.forward:  inputs @ weight.transpose(-2, -1)
+ *     (src/ajllm/modeling/layers.py:9-33)
+ * and no quantized path, so there is no reference FFI to mirror; these entry
+ * points are what a quantized twin of that operator binds.  Each declaration
+ * names the reference call it stands behind.
+ *
+ * Canonical interchange tensors (what "bit-exact" compares):
+ *   W8 : q       int8   [N, K]       row-major
+ *        scales  fp16   [N]
+ *   W4 : qweight int32  [N, K/8]     word c of row n = sum_j q[n, 8c+j] << 4j
+ *        scales  fp16   [N, K/128]
+ *        zeros   uint8  [N, K/128]   values 0..15
+ * Kernel-private tensors (made by ajq_repack_*, restored bit-for-bit by
+ * ajq_unrepack_*):
+ *   W4 : wq   uint32 [N/16, K/128, 64, 4]   one 1 KiB tile = 16 rows x 128 k,
+ *             element (lane = 16*kc + nl, dword j) holds the 8 weights
+ *             n = 16*tile_n + nl, k = 128*g + 32*j + 8*kc + e (e = 0..7) with
+ *             weight e in nibble (e>>1) + 4*(e&1)
+ *        meta uint32 [N/16, K/128, 16]      fp16 scale bits | fp16(128+zero) << 16
+ *   W8 : wq   uint32 [N/16, K/64, 64, 4]    tile = 16 rows x 64 k; lane (kc, nl)
+ *             holds bytes k = 64*t + 32*j + 8*kc + e for j = 0,1 in k order
+ *             (dword 2j+0: e=0..3, dword 2j+1: e=4..7), int8 unchanged
+ */
+#ifndef AJQ_H
+#define AJQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ajq_status {
+  AJQ_OK = 0,
+  AJQ_ERR_NULL = -1,        /* a required pointer is NULL */
+  AJQ_ERR_SHAPE = -2,       /* N, K or M outside what the kernel supports */
+  AJQ_ERR_ALIGN = -3,       /* a pointer is not 16-byte aligned */
+  AJQ_ERR_UNSUPPORTED = -4, /* flag / dtype combination not implemented */
+  AJQ_ERR_HIP = -5,         /* the HIP runtime reported an error at launch */
+  AJQ_ERR_WORKSPACE = -6    /* workspace missing or too small */
+} ajq_status;
+
+/* output element type of the matmul entry points */
+#define AJQ_OUT_BF16 0
+#define AJQ_OUT_F32 1 /* same accumulation, final cast skipped (parity checks) */
+
+int ajq_version(void);
+const char* ajq_last_error(void);
+const char* ajq_status_string(int status);
+
+/* ---- quantize / pack (stands behind Linear.__init__'s fp32 weight[out, in],
+ *      src/ajllm/modeling/layers.py:19-30) -------------------------------- */
+
+/* W fp32 [N, K] -> q int8 [N, K], scales fp16 [N].  K % 4 == 0. */
+int ajq_quantize_w8(const float* W, int N, int K, int8_t* q, uint16_t* scales, void* stream);
+
+/* W fp32 [N, K] -> qweight int32 [N, K/8], scales fp16 [N, K/128],
+ * zeros uint8 [N, K/128].  K % 128 == 0. */
+int ajq_quantize_w4_g128(const float* W, int N, int K, int32_t* qweight, uint16_t* scales,
+                         uint8_t* zeros, void* stream);
+
+/* canonical -> kernel-private layout and back.  N % 16 == 0; K % 128 == 0 (W4),
+ * K % 64 == 0 (W8). */
+int ajq_repack_w4(const int32_t* qweight, const uint16_t* scales, const uint8_t* zeros, int N, int K,
+                  uint32_t* wq, uint32_t* meta, void* stream);
+int ajq_unrepack_w4(const uint32_t* wq, const uint32_t* meta, int N, int K, int32_t* qweight,
+                    uint16_t* scales, uint8_t* zeros, void* stream);
+int ajq_repack_w8(const int8_t* q, int N, int K, uint32_t* wq, void* stream);
+int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream);
+
+/* ---- fused dequantize-matmul (stands behind Linear.forward,
+ *      src/ajllm/modeling/layers.py:32-33: y[M, N] = x[M, K] @ W_hat[N, K]^T) ---
+ * x bf16 [M, K] row-major, y bf16 or fp32 [M, N] row-major (out_dtype).
+ * fp32 accumulation; scales applied in fp32; the bf16 cast is round-to-nearest-even.
+ */
+
+/* decode shapes, 1 <= M <= 16; HBM-bound */
+int ajq_w4a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                   void* y, int out_dtype, void* stream);
+int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                   void* y, int out_dtype, void* stream);
+
+/* prefill shapes, any M >= 1 (tuned for M >= 256); bf16 MFMA.
+ * The W4 GEMM needs a workspace of ajq_w4a16_gemm_workspace_bytes(M, K) bytes
+ * (per-row, per-group activation sums). */
+size_t ajq_w4a16_gemm_workspace_bytes(int M, int K);
+int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                   void* y, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
+int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                   void* y, int out_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AJQ_H */

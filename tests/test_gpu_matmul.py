@@ -1,0 +1,159 @@
+"""GPU dequant-GEMV / dequant-GEMM against the CPU oracle.
+
+Parity is judged on the fp32-output variant of each kernel (same accumulation,
+final cast skipped) against an fp64 evaluation of the oracle, with the north-star
+tolerances max-abs <= 1e-2 and relative Frobenius <= 2e-3.  The bf16 output is
+checked separately: it must be the round-to-nearest-even of the kernel's own fp32
+result, lie within half a bf16 ulp (plus the fp32 error just measured) of the
+oracle's fp64 value, and be inside the Frobenius bound.  (An output of magnitude
+>= 2 has a bf16 ulp of 2^-6 > 1e-2, so max-abs <= 1e-2 cannot be asked of any bf16
+output, the oracle's own included.)
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import qspec
+from tests.helpers import MAX_ABS_TOL, REL_FRO_TOL, bf16_rounding_excess, errors, make_activations, make_weight
+
+pytestmark = pytest.mark.gpu
+
+_cache: dict = {}
+
+
+def _quantized(scheme: str, n: int, k: int, seed: int, cuda):
+    """(oracle dequantized weight fp64 on CPU, private GPU tensors) for one seeded weight."""
+    key = (scheme, n, k, seed)
+    if key not in _cache:
+        from ajllm_amd import repack_w4, repack_w8
+
+        w = make_weight(n, k, seed).numpy()
+        if scheme == "w4":
+            q, s, z = qspec.quantize_w4_g128(w)
+            qw = qspec.pack_int4(q)
+            w_hat = torch.from_numpy(qspec.dequantize_w4(qw, s, z))
+            wq, meta = repack_w4(torch.from_numpy(qw).to(cuda), torch.from_numpy(s).to(cuda), torch.from_numpy(z).to(cuda))
+        else:
+            q, s = qspec.quantize_w8(w)
+            w_hat = torch.from_numpy(qspec.dequantize_w8(q, s))
+            wq, meta = repack_w8(torch.from_numpy(q).to(cuda)), torch.from_numpy(s).to(cuda)
+        _cache.clear()  # keep one weight resident at a time
+        _cache[key] = (w_hat, wq, meta)
+    return _cache[key]
+
+
+def _run(scheme, x, wq, meta, out_dtype, kernel):
+    from ajllm_amd import w4a16_matmul, w8a16_matmul
+
+    fn = w4a16_matmul if scheme == "w4" else w8a16_matmul
+    return fn(x, wq, meta, out_dtype, kernel=kernel)
+
+
+def _check(scheme, kernel, m, n, k, seed, cuda, outliers=False, max_rows=None):
+    w_hat, wq, meta = _quantized(scheme, n, k, seed, cuda)
+    x = make_activations(m, k, seed + 100, outliers)
+    xg = x.to(cuda)
+    y32 = _run(scheme, xg, wq, meta, torch.float32, kernel)
+    y16 = _run(scheme, xg, wq, meta, torch.bfloat16, kernel)
+    torch.cuda.synchronize()
+    assert y32.shape == (m, n) and y16.shape == (m, n)
+    rows = torch.arange(m)
+    if max_rows is not None and m > max_rows:
+        rows = torch.randperm(m, generator=torch.Generator().manual_seed(seed))[:max_rows].sort().values
+    want64 = qspec.quant_linear(x[rows], w_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    max_abs, rel_fro = errors(y32.cpu()[rows], want64)
+    assert max_abs <= MAX_ABS_TOL and rel_fro <= REL_FRO_TOL, (max_abs, rel_fro)
+    # the kernel's fp32 result is far inside the tolerance: fp32 accumulation noise only
+    assert max_abs <= 2e-3, max_abs
+    got16 = y16.cpu()[rows]
+    assert bf16_rounding_excess(got16, want64, max_abs) <= 0
+    assert errors(got16, want64)[1] <= REL_FRO_TOL
+    # bf16 output is the rounding of the fp32 output
+    assert torch.equal(y16.cpu(), y32.cpu().to(torch.bfloat16))
+    return y32
+
+
+GEMV_SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336)]  # (N, K)
+
+
+@pytest.mark.parametrize("n,k", GEMV_SHAPES)
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_w4a16_gemv(cuda, m, n, k):
+    _check("w4", "gemv", m, n, k, seed=11, cuda=cuda)
+
+
+@pytest.mark.parametrize("n,k", GEMV_SHAPES)
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_w8a16_gemv(cuda, m, n, k):
+    _check("w8", "gemv", m, n, k, seed=12, cuda=cuda)
+
+
+@pytest.mark.parametrize("m", [2, 3, 7, 13])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemv_ragged_m_and_small_shapes(cuda, scheme, m):
+    _check(scheme, "gemv", m, 48, 384, seed=13, cuda=cuda)
+    _check(scheme, "gemv", m, 2048, 5632, seed=14, cuda=cuda)
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemv_is_deterministic(cuda, scheme):
+    w_hat, wq, meta = _quantized(scheme, 4096, 4096, 11 if scheme == "w4" else 12, cuda)
+    x = make_activations(4, 4096, 5).to(cuda)
+    first = _run(scheme, x, wq, meta, torch.float32, "gemv")
+    for _ in range(10):
+        assert torch.equal(_run(scheme, x, wq, meta, torch.float32, "gemv"), first)
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_one_hot_activation_reads_back_dequantized_weights(cuda, scheme):
+    """x = e_k picks column k of W_hat: every entry must be the exact fp32 dequantized weight."""
+    n, k = 64, 512
+    w_hat, wq, meta = _quantized(scheme, n, k, 21, cuda)
+    cols = [0, 1, 7, 8, 127, 128, 255, 300, 511, 37, 64, 65, 190, 256, 383, 448]
+    x = torch.zeros((16, k), dtype=torch.bfloat16)
+    for i, c in enumerate(cols):
+        x[i, c] = 1.0
+    for kernel in ("gemv", "gemm"):
+        y = _run(scheme, x.to(cuda), wq, meta, torch.float32, kernel).cpu()
+        assert torch.equal(y, w_hat[:, cols].t().contiguous()), kernel
+
+
+GEMM_CASES = [(256, 4096, 4096), (2048, 4096, 4096), (256, 14336, 4096), (2048, 14336, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_CASES)
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_prefill_gemm(cuda, scheme, m, n, k):
+    _check(scheme, "gemm", m, n, k, seed=31, cuda=cuda, outliers=True, max_rows=256)
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+@pytest.mark.parametrize("n", [4096, 14336])
+def test_prefill_gemm_m8192(cuda, scheme, n):
+    _check(scheme, "gemm", 8192, n, 4096, seed=32, cuda=cuda, outliers=True, max_rows=128)
+
+
+@pytest.mark.parametrize("m", [1, 17, 63, 65, 100, 129, 300])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemm_ragged_m(cuda, scheme, m):
+    _check(scheme, "gemm", m, 272, 640, seed=33, cuda=cuda, outliers=True)
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemv_and_gemm_agree(cuda, scheme):
+    w_hat, wq, meta = _quantized(scheme, 2048, 2048, 41, cuda)
+    x = make_activations(16, 2048, 6).to(cuda)
+    a = _run(scheme, x, wq, meta, torch.float32, "gemv")
+    b = _run(scheme, x, wq, meta, torch.float32, "gemm")
+    assert errors(a, b)[0] <= 1e-4
+
+
+def test_linearity_at_full_size(cuda):
+    """Size-independent property: the kernel is linear in x (checked in fp32 output)."""
+    w_hat, wq, meta = _quantized("w4", 14336, 4096, 31, cuda)
+    x1 = make_activations(512, 4096, 1).to(cuda)
+    x2 = (x1.float() * 2).to(torch.bfloat16)  # exact doubling in bf16
+    y1 = _run("w4", x1, wq, meta, torch.float32, "gemm")
+    y2 = _run("w4", x2, wq, meta, torch.float32, "gemm")
+    assert errors(y2, 2 * y1)[0] <= 1e-3
