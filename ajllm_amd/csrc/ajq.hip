@@ -45,12 +45,19 @@ int gemv_kchunk(int M, int K) {
   return (int)(fit < K ? fit : K);
 }
 
+// Kernels that stage more than 64 KiB in LDS must be opted in once per process
+// (and per device); the largest size granted so far is remembered per kernel.
 template <typename Kernel>
 int allow_big_lds(Kernel kernel, size_t bytes) {
+  static thread_local size_t granted[16] = {0};
   if (bytes <= 64 * 1024) return AJQ_OK;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = 0;
+  if (bytes <= granted[dev]) return AJQ_OK;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
   if (e != hipSuccess) return fail(AJQ_ERR_HIP, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
+  granted[dev] = bytes;
   return AJQ_OK;
 }
 

@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Default run (what the driver calls: ``python bench.py --gpus 1 --steps K --warmup W``):
+
+* timed region: the W4A16-g128 decode GEMV at the headline shape K = N = 4096, M = 1.
+  One *step* is one pass over ``--copies`` distinct weight matrices (default 64, 559 MB of
+  packed weights, larger than the 256 MB Infinity Cache plus the L2s, so every launch
+  streams its weights from HBM).  The launches of a step are recorded once into a HIP
+  graph and replayed, so the host's launch cost is not part of the measurement.  Timing is
+  by HIP events on the launch stream around exactly K steps.
+* after it (not part of ``value``): the M = 2048 prefill GEMMs (W4 and W8, K = N = 4096) in
+  TFLOP/s against the bf16 dense MFMA peak, and the CPU baseline: the oracle's quantized
+  linear timed on this box's host cores for the same GEMV shape.
+
+``--sweep`` adds the rest of the decode sweep (three shapes x M in {1, 4, 16}, W4 and W8)
+and all prefill shapes; ``--decode`` adds the end-to-end decode tokens/s of the 12-layer
+model.  One JSON line is printed on stdout; everything else goes to stderr.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor peak
+
+
+def log(*args) -> None:
+    print(*args, file=sys.stderr, flush=True)
+
+
+# ------------------------------------------------------------------ algorithmic work
+def w4_gemv_bytes(m: int, n: int, k: int) -> float:
+    """packed nibbles + fp16 scales + 4-bit zero-points + bf16 activations in and out"""
+    return n * k / 2 + 2 * n * k / 128 + 0.5 * n * k / 128 + 2 * m * k + 2 * m * n
+
+
+def w8_gemv_bytes(m: int, n: int, k: int) -> float:
+    return n * k + 2 * n + 2 * m * k + 2 * m * n
+
+
+def gemm_flops(m: int, n: int, k: int) -> float:
+    return 2.0 * m * n * k
+
+
+# ------------------------------------------------------------------ synthetic inputs
+def make_w4(n: int, k: int, copies: int, device, seed: int):
+    """``copies`` distinct private W4 weights.  Weights ~ N(0, 0.02) are quantized on the GPU."""
+    from ajllm_amd import quantize_w4_g128, repack_w4
+
+    out = []
+    g = torch.Generator(device=device).manual_seed(seed)
+    for _ in range(copies):
+        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+        out.append(repack_w4(*quantize_w4_g128(w)))
+    return out
+
+
+def make_w8(n: int, k: int, copies: int, device, seed: int):
+    from ajllm_amd import quantize_w8, repack_w8
+
+    out = []
+    g = torch.Generator(device=device).manual_seed(seed)
+    for _ in range(copies):
+        w = torch.randn((n, k), generator=g, device=device, dtype=torch.float32) * 0.02
+        q, s = quantize_w8(w)
+        out.append((repack_w8(q), s))
+    return out
+
+
+def make_x(m: int, k: int, device, seed: int, outliers: bool = False) -> torch.Tensor:
+    g = torch.Generator(device=device).manual_seed(seed)
+    x = torch.randn((m, k), generator=g, device=device, dtype=torch.float32)
+    if outliers:
+        mask = torch.rand((m, k), generator=g, device=device) < 0.001
+        x = torch.where(mask, x * 20.0, x)
+    return x.to(torch.bfloat16)
+
+
+# ------------------------------------------------------------------ timing
+def time_graph_steps(step_fn, steps: int, warmup: int) -> float:
+    """Record ``step_fn`` (kernel launches on the current stream) into a HIP graph, replay it
+    ``warmup`` times untimed, then time exactly ``steps`` replays with HIP events on the same
+    stream.  Returns seconds for the ``steps`` replays."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        step_fn()  # eager once: sets function attributes, fills caches
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            step_fn()
+        for _ in range(warmup):
+            graph.replay()
+        stream.synchronize()
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record(stream)
+        for _ in range(steps):
+            graph.replay()
+        stop.record(stream)
+        stop.synchronize()
+        torch.cuda.synchronize()
+    return start.elapsed_time(stop) / 1e3
+
+
+def bench_gemv(scheme: str, m: int, n: int, k: int, copies: int, steps: int, warmup: int, device) -> dict:
+    from ajllm_amd import w4a16_matmul, w8a16_matmul
+
+    weights = make_w4(n, k, copies, device, 1234) if scheme == "w4" else make_w8(n, k, copies, device, 1234)
+    x = make_x(m, k, device, 99)
+    fn = w4a16_matmul if scheme == "w4" else w8a16_matmul
+    nbytes = w4_gemv_bytes(m, n, k) if scheme == "w4" else w8_gemv_bytes(m, n, k)
+    outs = []
+
+    def step():
+        outs.clear()
+        for a, b in weights:
+            outs.append(fn(x, a, b, torch.bfloat16, kernel="gemv"))
+
+    seconds = time_graph_steps(step, steps, warmup)
+    launches = steps * copies
+    us = seconds / launches * 1e6
+    gbs = nbytes / (seconds / launches) / 1e9
+    return {"scheme": scheme, "M": m, "N": n, "K": k, "launches": launches, "us_per_launch": us,
+            "bytes_per_launch": nbytes, "GB/s": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+            "ms_per_step": seconds / steps * 1e3}
+
+
+def bench_gemm(scheme: str, m: int, n: int, k: int, steps: int, warmup: int, device, copies: int = 4) -> dict:
+    from ajllm_amd import w4a16_matmul, w8a16_matmul
+
+    weights = make_w4(n, k, copies, device, 4321) if scheme == "w4" else make_w8(n, k, copies, device, 4321)
+    x = make_x(m, k, device, 98, outliers=True)
+    fn = w4a16_matmul if scheme == "w4" else w8a16_matmul
+    outs = []
+
+    def step():
+        outs.clear()
+        for a, b in weights:
+            outs.append(fn(x, a, b, torch.bfloat16, kernel="gemm"))
+
+    seconds = time_graph_steps(step, steps, warmup)
+    launches = steps * copies
+    us = seconds / launches * 1e6
+    tflops = gemm_flops(m, n, k) / (seconds / launches) / 1e12
+    return {"scheme": scheme, "M": m, "N": n, "K": k, "launches": launches, "us_per_launch": us,
+            "TFLOP/s": tflops, "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS}
+
+
+# ------------------------------------------------------------------ CPU baseline
+def cpu_baseline(m: int, n: int, k: int, budget_s: float = 15.0) -> dict:
+    """The oracle's quantized linear (dequantize -> matmul, fp32) on the host cores, same shape
+    and seeded inputs as the timed GEMV.  The reference project has no quantized CPU path (its
+    only linear is the dense ``x @ W.T`` of src/ajllm/modeling/layers.py:32-33, also timed here),
+    so ``kind`` is "port"."""
+    from oracle import qspec
+
+    threads = min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(1234)
+    w = torch.randn((n, k), generator=g, dtype=torch.float32) * 0.02
+    layer = qspec.QuantLinearRef.from_weight(w, "w4a16_g128", cache_dequant=False)
+    x = torch.randn((m, k), generator=torch.Generator().manual_seed(99)).to(torch.bfloat16)
+    nbytes = w4_gemv_bytes(m, n, k)
+
+    def timed(fn, reps_cap=20):
+        fn()
+        times = []
+        t_end = time.perf_counter() + budget_s / 3
+        while len(times) < reps_cap and (time.perf_counter() < t_end or len(times) < 3):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    t_deq, n_deq = timed(lambda: layer(x))
+    layer.cache_dequant = True
+    layer.dequantized()
+    t_pre, n_pre = timed(lambda: layer(x))
+    w_bf16 = w.to(torch.bfloat16)
+    t_dense, n_dense = timed(lambda: x @ w_bf16.t())
+    return {
+        "value": nbytes / t_deq / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"oracle QuantLinearRef (dequantize every call, fp32 matmul), W4A16-g128 M={m} N={n} K={k}, "
+                  f"median of {n_deq} calls; same algorithmic bytes as the GPU figure",
+        "predequantized_GB/s": nbytes / t_pre / 1e9,
+        "dense_bf16_x_at_wT_GB/s": nbytes / t_dense / 1e9,
+        "ms_per_call": t_deq * 1e3, "host_cpu_count": os.cpu_count(),
+    }
+
+
+# ------------------------------------------------------------------ main
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--copies", type=int, default=64, help="distinct weight matrices per step")
+    ap.add_argument("--sweep", action="store_true", help="also time the full decode and prefill sweeps")
+    ap.add_argument("--decode", action="store_true", help="also time end-to-end greedy decode")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="timed region only")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on exactly one GPU (the quantized linear is a single-GPU "
+            f"path; no collectives exist). --gpus {args.gpus} is not supported.")
+        return 2
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible")
+        return 2
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    from ajllm_amd import _lib
+
+    _lib.load()
+    m, n, k = 1, 4096, 4096
+    head = bench_gemv("w4", m, n, k, args.copies, args.steps, args.warmup, device)
+    log("headline", json.dumps(head))
+    extras: dict = {}
+    if not args.no_extras:
+        gemm = []
+        for scheme in ("w4", "w8"):
+            r = bench_gemm(scheme, 2048, 4096, 4096, steps=10, warmup=3, device=device)
+            log("gemm", json.dumps(r))
+            gemm.append(r)
+        extras["prefill_gemm"] = gemm
+    if args.sweep:
+        sweep = []
+        for scheme in ("w4", "w8"):
+            for (sn, sk) in ((4096, 4096), (14336, 4096), (4096, 14336)):
+                copies = args.copies if sn * sk < 2**25 else max(12, args.copies // 3)
+                for sm in (1, 4, 16):
+                    r = bench_gemv(scheme, sm, sn, sk, copies, max(5, args.steps // 5), 2, device)
+                    log("sweep", json.dumps(r))
+                    sweep.append(r)
+        extras["decode_sweep"] = sweep
+        gemm = []
+        for scheme in ("w4", "w8"):
+            for sm in (256, 2048, 8192):
+                for sn in (4096, 14336):
+                    r = bench_gemm(scheme, sm, sn, 4096, steps=5, warmup=2, device=device, copies=2)
+                    log("gemm", json.dumps(r))
+                    gemm.append(r)
+        extras["prefill_sweep"] = gemm
+    if args.decode:
+        from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
+
+        extras["decode"] = bench_decode(device, log)
+    cpu = None if args.no_cpu else cpu_baseline(m, n, k)
+    if cpu:
+        log("cpu_baseline", json.dumps(cpu))
+
+    line = {
+        "metric": "W4A16 dequant-GEMV GB/s",
+        "value": head["GB/s"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 activations x uint4 weights, fp32 accumulate",
+        "data": "synthetic (seeded N(0,0.02) weights quantized on the GPU, N(0,1) bf16 activations)",
+        "config": {
+            "workload": "W4A16-g128 decode GEMV, K=N=4096, M=1 (decode sweep headline shape)",
+            "launches_per_step": args.copies,
+            "distinct_weight_bytes": args.copies * (n * k // 2 + n * k // 128 * 4),
+            "launch": "HIP graph replay of one step",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": head["GB/s"],
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": head["frac_hbm_peak"],
+            "traffic": None,
+            "kernel": "w4a16_gemv_kernel",
+            "algorithmic_bytes_per_launch": head["bytes_per_launch"],
+            "avg_launch_us": head["us_per_launch"],
+        },
+        "cpu_baseline": cpu,
+        "peaks": {"hbm_GB/s": HBM_PEAK_GBS, "mfma_bf16_TFLOP/s": MFMA_BF16_PEAK_TFLOPS},
+    }
+    line.update(extras)
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
