@@ -31,19 +31,9 @@ int check_launch(const char* what) {
 }
 
 constexpr int kMaxGemvM = 16;
-constexpr size_t kGemvLdsBudget = 128 * 1024;  // bytes of LDS for the staged activations
 constexpr int kGemmMpadTo = 256;
 
 int round_up(int v, int to) { return (v + to - 1) / to * to; }
-
-// Largest K chunk (multiple of 128) whose M staged rows fit the LDS budget.
-int gemv_kchunk(int M, int K) {
-  long long per_k = 2LL * M;  // bytes per k column
-  long long fit = ((long long)kGemvLdsBudget - 16LL * M) / per_k;
-  fit = fit / 128 * 128;
-  if (fit < 128) fit = 128;
-  return (int)(fit < K ? fit : K);
-}
 
 // Kernels that stage more than 64 KiB in LDS must be opted in once per process
 // (and per device); the largest size granted so far is remembered per kernel.
@@ -184,32 +174,54 @@ int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream) {
   return check_launch("ajq_unrepack_w8");
 }
 
+}  // extern "C"
+
 // --------------------------------------------------------------- GEMV -----
+namespace {
+
+template <int kWaves, int TPW, int MROWS, bool kW4>
+int launch_gemv_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                    const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  constexpr size_t lds = gemv_lds_bytes(kWaves, TPW, MROWS);
+  static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
+  auto kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8, N, y, out_f32);
+  return AJQ_OK;
+}
+
+// Row bound MROWS is the next power of two >= M; the slice a wave stages shrinks
+// (TPW 4 -> 2, twice the waves) when 16 rows would not fit the LDS otherwise.
+template <bool kW4>
+int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  if (M <= 1) return launch_gemv_cfg<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 2) return launch_gemv_cfg<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 4) return launch_gemv_cfg<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 8) return launch_gemv_cfg<8, 4, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_gemv_cfg<16, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
 int ajq_w4a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
                    int out_dtype, void* stream) {
   if (int s = check_matmul_args("ajq_w4a16_gemv", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
   if (M > kMaxGemvM) return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemv: M=%d exceeds %d; use ajq_w4a16_gemm", M, kMaxGemvM);
-  constexpr int kWaves = 8;
-  const int kchunk = gemv_kchunk(M, K);
-  const size_t lds = (size_t)M * (kchunk + 8) * 2 + (size_t)kWaves * 64 * 16;
-  auto kernel = w4a16_gemv_kernel<kWaves>;
-  if (int s = allow_big_lds(kernel, lds)) return s;
-  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, (hipStream_t)stream, x, M, K,
-                     reinterpret_cast<const u32x4_t*>(wq), meta, N, y, out_dtype == AJQ_OUT_F32, kchunk);
+  if (int s = launch_gemv<true>(x, M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
+    return s;
   return check_launch("ajq_w4a16_gemv");
 }
 
 int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
                    int out_dtype, void* stream) {
-  if (int s = check_matmul_args("ajq_w8a16_gemv", x, M, K, wq, scales, N, y, out_dtype, kW8TileK)) return s;
+  if (int s = check_matmul_args("ajq_w8a16_gemv", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
   if (M > kMaxGemvM) return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemv: M=%d exceeds %d; use ajq_w8a16_gemm", M, kMaxGemvM);
-  constexpr int kWaves = 8;
-  const int kchunk = gemv_kchunk(M, K);
-  const size_t lds = (size_t)M * (kchunk + 8) * 2 + (size_t)kWaves * 64 * 16;
-  auto kernel = w8a16_gemv_kernel<kWaves>;
-  if (int s = allow_big_lds(kernel, lds)) return s;
-  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, (hipStream_t)stream, x, M, K,
-                     reinterpret_cast<const u32x4_t*>(wq), scales, N, y, out_dtype == AJQ_OUT_F32, kchunk);
+  if (int s = launch_gemv<false>(x, M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
+    return s;
   return check_launch("ajq_w8a16_gemv");
 }
 

@@ -1,52 +1,173 @@
 // Decode dequant-GEMV, 1 <= M <= 16:  y[M, N] = x[M, K] @ W_hat[N, K]^T.
 //
-// HBM-bound.  One workgroup owns one 16-row tile of N and all of K; its waves
-// take the 1 KiB weight tiles of that row block round-robin, so a wave's load
-// instruction reads one contiguous KiB (64 lanes x 16 B) and the workgroup as a
-// whole streams one contiguous region.  Weights go global -> registers ->
-// in-register unpack to bf16 -> MFMA B operand; they never touch LDS.  The
-// activations are staged once per workgroup in LDS (row-major, rows padded by
-// 16 B so the 16 rows of an A fragment fall in distinct banks) and are the
-// MFMA A operand with rows >= M zero.  Partial sums of the waves are combined
-// through LDS in a fixed order (no atomics: results are run-to-run identical).
+// HBM-bound and short (a 4096 x 4096 int4 matrix is 8.7 MB, about a microsecond
+// of HBM time), so the kernel is built to have every byte in flight as early as
+// possible and to do its arithmetic while the bytes arrive:
+//  * one workgroup owns one 16-row tile of N and all of K; wave w owns a
+//    contiguous run of 128-wide k groups, i.e. a contiguous run of 1 KiB private
+//    weight tiles, and loads each with one 128-bit load per lane (a wave-wide
+//    load instruction reads one contiguous KiB), non-temporal, issued up front;
+//  * weights go global -> registers -> in-register unpack (3 shifts + 4
+//    v_and_or_b32 per 8 nibbles) -> MFMA B operand; they never touch LDS;
+//  * each wave stages only ITS k-slice of the activations in a wave-private LDS
+//    region (rows padded by 16 B: the 16 rows of an A fragment fall in distinct
+//    banks) and reads it back as MFMA A fragments, so there is no workgroup
+//    barrier before the arithmetic; rows >= M of the A operand repeat row M-1 and
+//    their outputs are never stored;
+//  * group sums of the activations (needed for the zero-point term) come from a
+//    second MFMA against an all-ones B operand, which lands them in exactly the
+//    accumulator layout that needs them;
+//  * the waves' partial sums meet once, through LDS, in a fixed order: no
+//    atomics, results are run-to-run identical.
 #pragma once
 #include "ajq_common.h"
 
 namespace ajq {
 
-constexpr int kPrefetch = 4;  // weight tiles a wave keeps in flight per batch
-
-struct GemvSmem {
-  // x chunk: M rows x (kchunk + 8) bf16, then the cross-wave reduction area
-  __device__ static uint16_t* x(void* base) { return reinterpret_cast<uint16_t*>(base); }
-};
-
-template <int kWaves>
-__device__ __forceinline__ void stage_x_chunk(const uint16_t* __restrict__ x, int M, int K, int c0,
-                                              int clen, uint16_t* xs, int stride) {
-  const int vec_per_row = clen >> 3;
-  const int total = M * vec_per_row;
-  for (int v = threadIdx.x; v < total; v += kWaves * 64) {
-    const int m = v / vec_per_row;
-    const int c = v - m * vec_per_row;
-    const u32x4_t val = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + c0 + 8 * c);
-    *reinterpret_cast<u32x4_t*>(xs + m * stride + 8 * c) = val;
-  }
+__device__ __forceinline__ uint32_t and_or_b32(uint32_t a, uint32_t mask_sgpr, uint32_t magic_vgpr) {
+  uint32_t r;
+  // VOP3 on gfx9 takes no literal: the mask rides in an SGPR, the magic in a VGPR
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask_sgpr), "v"(magic_vgpr));
+  return r;
 }
 
-template <int kWaves>
-__device__ __forceinline__ void reduce_and_store(f32x4_t acc, float* red, int M, int N, int nt, void* y,
-                                                 int out_f32, const float* chan_scale) {
+// private W4 dword -> 8 bf16 holding 128+q (see w4_to_bf16_biased), 7 VALU ops
+__device__ __forceinline__ u32x4_t w4_unpack(uint32_t w, uint32_t mask, uint32_t magic) {
+  u32x4_t r;
+  r.x = and_or_b32(w, mask, magic);
+  r.y = and_or_b32(w >> 4, mask, magic);
+  r.z = and_or_b32(w >> 8, mask, magic);
+  r.w = and_or_b32(w >> 12, mask, magic);
+  return r;
+}
+
+// kWaves waves per workgroup; a wave works through its k groups TPW at a time;
+// MROWS >= M is the compile-time row bound that sizes the activation slice.
+template <int kWaves, int TPW, int MROWS, bool kW4>
+__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
+    const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
+    const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
+    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
+    int N, void* __restrict__ y, int out_f32) {
+  constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
+  constexpr int kStride = kSlice + 8;      // padded LDS row, bf16 elements
+  constexpr int kVecPerRow = kSlice / 8;   // 16-byte vectors per slice row
+  constexpr int kXLoads = (MROWS * kVecPerRow + 63) / 64;
+  constexpr int kLoadsPerGroup = kW4 ? 1 : 2;  // 1 KiB tiles per 128 k
+
+  extern __shared__ u32x4_t smem_raw[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nl = lane & 15, kc = lane >> 4;
+  const int nt = blockIdx.x;
+  const int G = K >> 7;
+  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * (MROWS * kStride);
+  float* red = reinterpret_cast<float*>(reinterpret_cast<uint16_t*>(smem_raw) + kWaves * (MROWS * kStride));
+
+  const int per_wave = (G + kWaves - 1) / kWaves;
+  const int g_begin = wave * per_wave;
+  const int g_end = min(G, g_begin + per_wave);
+
+  const u32x4_t* wtile = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
+  const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
+
+  u32x4_t xv[kXLoads];
+  u32x4_t wv[TPW][kLoadsPerGroup];
+  uint32_t mv[TPW];
+
+  auto load_x = [&](int g0) {  // activations of groups [g0, g0 + TPW) -> registers
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = lane + 64 * i;
+      const int m = v / kVecPerRow, c = v % kVecPerRow;
+      if (m < M && g0 * kGroup + 8 * c < K)
+        xv[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g0 * kGroup + 8 * c);
+    }
+  };
+  auto load_w = [&](int g0) {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      if (g0 + p < g_end) {
+#pragma unroll
+        for (int h = 0; h < kLoadsPerGroup; ++h)
+          wv[p][h] = __builtin_nontemporal_load(wtile + ((size_t)(g0 + p) * kLoadsPerGroup + h) * 64);
+        if (kW4) mv[p] = mtile[(size_t)(g0 + p) * 16];
+      }
+    }
+  };
+
+  const uint32_t mask = 0x000F000Fu;
+  uint32_t magic = 0x43004300u;
+  asm volatile("" : "+v"(magic));  // keep it in a VGPR for v_and_or_b32
+  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  const int row = min(nl, M - 1);
+  const uint16_t* xrow = xs + row * kStride + 8 * kc;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+  if (g_begin < g_end) {
+    load_x(g_begin);
+    load_w(g_begin);
+  }
+  for (int g0 = g_begin; g0 < g_end; g0 += TPW) {
+    // slice of this batch -> wave-private LDS (LDS ops of one wave execute in order,
+    // so the reads of the previous batch are already done)
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = lane + 64 * i;
+      const int m = v / kVecPerRow, c = v % kVecPerRow;
+      if (m < M && g0 * kGroup + 8 * c < K) *reinterpret_cast<u32x4_t*>(xs + m * kStride + 8 * c) = xv[i];
+    }
+    // registers of this batch
+    u32x4_t wc[TPW][kLoadsPerGroup];
+    uint32_t mc[TPW];
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h) wc[p][h] = wv[p][h];
+      mc[p] = mv[p];
+    }
+    if (g0 + TPW < g_end) {  // next batch in flight while this one is computed
+      load_x(g0 + TPW);
+      load_w(g0 + TPW);
+    }
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      if (g0 + p < g_end) {
+        if (kW4) {
+          f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+            const u32x4_t b = w4_unpack(wc[p][0][j], mask, magic);
+            part = mfma16(a, b, part);
+            asum = mfma16(a, ones, asum);
+          }
+          const float s = f16_bits_to_f32(mc[p] & 0xFFFFu);
+          const float zc = f16_bits_to_f32(mc[p] >> 16);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] += s * (part[i] - zc * asum[i]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+            const u32x2_t lo = w8_to_bf16(wc[p][j >> 1][2 * (j & 1)]);
+            const u32x2_t hi = w8_to_bf16(wc[p][j >> 1][2 * (j & 1) + 1]);
+            acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- the waves' partial sums meet in LDS; wave 0 adds them in wave order
   reinterpret_cast<f32x4_t*>(red)[wave * 64 + lane] = acc;
   __syncthreads();
   if (wave != 0) return;
   f32x4_t sum = reinterpret_cast<f32x4_t*>(red)[lane];
 #pragma unroll
   for (int w = 1; w < kWaves; ++w) sum += reinterpret_cast<f32x4_t*>(red)[w * 64 + lane];
-  const int nl = lane & 15, kc = lane >> 4;
   const int n = nt * kTileN + nl;
-  const float cs = chan_scale ? chan_scale[0] : 1.0f;
+  float cs = 1.0f;
+  if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int m = 4 * kc + i;
@@ -60,161 +181,9 @@ __device__ __forceinline__ void reduce_and_store(f32x4_t acc, float* red, int M,
   }
 }
 
-// ------------------------------------------------------------------ W4 ----
-template <int kWaves>
-__global__ __launch_bounds__(kWaves * 64) void w4a16_gemv_kernel(
-    const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
-    const uint32_t* __restrict__ meta, int N, void* __restrict__ y, int out_f32, int kchunk) {
-  extern __shared__ u32x4_t smem_raw[];
-  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw);
-  const int stride = kchunk + 8;
-  float* red = reinterpret_cast<float*>(xs + (size_t)M * stride);
-
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nl = lane & 15, kc = lane >> 4;
-  const int nt = blockIdx.x;
-  const int G = K >> 7;
-  const u32x4_t* wtile = wq + (size_t)nt * G * 64 + lane;
-  const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
-  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  const bool row_live = nl < M;
-
-  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-
-  for (int c0 = 0; c0 < K; c0 += kchunk) {
-    const int clen = min(kchunk, K - c0);
-    const int g_lo = c0 >> 7, g_hi = (c0 + clen) >> 7;
-    // first group of this wave inside the chunk
-    int g = g_lo + ((wave - g_lo) % kWaves + kWaves) % kWaves;
-
-    u32x4_t wcur[kPrefetch];
-    uint32_t mcur[kPrefetch];
-#pragma unroll
-    for (int p = 0; p < kPrefetch; ++p) {
-      const int gp = g + p * kWaves;
-      if (gp < g_hi) {
-        wcur[p] = wtile[(size_t)gp * 64];
-        mcur[p] = mtile[(size_t)gp * 16];
-      }
-    }
-    __syncthreads();  // everyone is done reading the previous chunk
-    stage_x_chunk<kWaves>(x, M, K, c0, clen, xs, stride);
-    __syncthreads();
-
-    while (g < g_hi) {
-      u32x4_t wnxt[kPrefetch];
-      uint32_t mnxt[kPrefetch];
-      const int gn = g + kPrefetch * kWaves;
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) {
-        const int gp = gn + p * kWaves;
-        if (gp < g_hi) {
-          wnxt[p] = wtile[(size_t)gp * 64];
-          mnxt[p] = mtile[(size_t)gp * 16];
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) {
-        const int gp = g + p * kWaves;
-        if (gp < g_hi) {
-          const uint16_t* xrow = xs + nl * stride + (gp * kGroup - c0) + 8 * kc;
-          f32x4_t tmp = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            u32x4_t a = zero4;
-            if (row_live) a = *reinterpret_cast<const u32x4_t*>(xrow + 32 * j);
-            const u32x4_t b = w4_to_bf16_biased(wcur[p][j]);
-            tmp = mfma16(a, b, tmp);
-            asum = mfma16(a, ones, asum);
-          }
-          const float s = f16_bits_to_f32(mcur[p] & 0xFFFFu);
-          const float zc = f16_bits_to_f32(mcur[p] >> 16);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] += s * (tmp[i] - zc * asum[i]);
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) {
-        wcur[p] = wnxt[p];
-        mcur[p] = mnxt[p];
-      }
-      g = gn;
-    }
-  }
-  reduce_and_store<kWaves>(acc, red, M, N, nt, y, out_f32, nullptr);
+// LDS bytes of one workgroup of dequant_gemv_kernel<kWaves, TPW, MROWS, *>
+constexpr size_t gemv_lds_bytes(int waves, int tpw, int mrows) {
+  return (size_t)waves * mrows * (tpw * kGroup + 8) * 2 + (size_t)waves * 64 * 16;
 }
-
-// ------------------------------------------------------------------ W8 ----
-template <int kWaves>
-__global__ __launch_bounds__(kWaves * 64) void w8a16_gemv_kernel(
-    const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
-    const uint16_t* __restrict__ scales, int N, void* __restrict__ y, int out_f32, int kchunk) {
-  extern __shared__ u32x4_t smem_raw[];
-  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw);
-  const int stride = kchunk + 8;
-  float* red = reinterpret_cast<float*>(xs + (size_t)M * stride);
-
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int nl = lane & 15, kc = lane >> 4;
-  const int nt = blockIdx.x;
-  const int T = K >> 6;  // 64-wide tiles along K
-  const u32x4_t* wtile = wq + (size_t)nt * T * 64 + lane;
-  const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-  const bool row_live = nl < M;
-
-  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-
-  for (int c0 = 0; c0 < K; c0 += kchunk) {
-    const int clen = min(kchunk, K - c0);
-    const int t_lo = c0 >> 6, t_hi = (c0 + clen) >> 6;
-    int t = t_lo + ((wave - t_lo) % kWaves + kWaves) % kWaves;
-
-    u32x4_t wcur[kPrefetch];
-#pragma unroll
-    for (int p = 0; p < kPrefetch; ++p) {
-      const int tp = t + p * kWaves;
-      if (tp < t_hi) wcur[p] = wtile[(size_t)tp * 64];
-    }
-    __syncthreads();
-    stage_x_chunk<kWaves>(x, M, K, c0, clen, xs, stride);
-    __syncthreads();
-
-    while (t < t_hi) {
-      u32x4_t wnxt[kPrefetch];
-      const int tn = t + kPrefetch * kWaves;
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) {
-        const int tp = tn + p * kWaves;
-        if (tp < t_hi) wnxt[p] = wtile[(size_t)tp * 64];
-      }
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) {
-        const int tp = t + p * kWaves;
-        if (tp < t_hi) {
-          const uint16_t* xrow = xs + nl * stride + (tp * kW8TileK - c0) + 8 * kc;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            u32x4_t a = zero4;
-            if (row_live) a = *reinterpret_cast<const u32x4_t*>(xrow + 32 * j);
-            const u32x2_t lo = w8_to_bf16(wcur[p][2 * j]);
-            const u32x2_t hi = w8_to_bf16(wcur[p][2 * j + 1]);
-            const u32x4_t b = {lo.x, lo.y, hi.x, hi.y};
-            acc = mfma16(a, b, acc);
-          }
-        }
-      }
-#pragma unroll
-      for (int p = 0; p < kPrefetch; ++p) wcur[p] = wnxt[p];
-      t = tn;
-    }
-  }
-  // per-output-channel scale, applied once after the cross-wave sum
-  __shared__ float chan_scale_s[16];
-  if (threadIdx.x < 16) chan_scale_s[threadIdx.x] = f16_bits_to_f32(scales[nt * kTileN + threadIdx.x]);
-  // reduce_and_store's barrier orders the write above before its reads
-  reduce_and_store<kWaves>(acc, red, M, N, nt, y, out_f32, &chan_scale_s[nl]);
-}
-
 
 }  // namespace ajq

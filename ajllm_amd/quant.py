@@ -116,8 +116,8 @@ def repack_w8(q: torch.Tensor) -> torch.Tensor:
     """int8 [N, K] -> wq int32 [N16/16, K/64, 64, 4] (rows zero-padded to a multiple of 16)."""
     _require_cuda(q)
     n, k = q.shape
-    if k % 64 != 0:
-        raise ValueError(f"K={k} must be a multiple of 64 for w8a16")
+    if k % GROUP != 0:
+        raise ValueError(f"K={k} must be a multiple of {GROUP} for w8a16")
     n16 = (n + TILE_N - 1) // TILE_N * TILE_N
     q = _pad_rows(q, n16)
     wq = torch.empty((n16 // TILE_N, k // 64, 64, 4), dtype=torch.int32, device=q.device)
@@ -200,8 +200,6 @@ def w8a16_matmul(
     lib = _lib.load()
     use_gemv = (m <= GEMV_MAX_M) if kernel == "auto" else (kernel == "gemv")
     fn = lib.ajq_w8a16_gemv if use_gemv else lib.ajq_w8a16_gemm
-    if not use_gemv and k % GROUP != 0:
-        raise ValueError(f"K={k} must be a multiple of {GROUP} for the W8 GEMM")
     with torch.cuda.device(x.device):
         status = fn(x.data_ptr(), m, k, wq.data_ptr(), scales.data_ptr(), n16, y.data_ptr(), flag, _stream())
     _lib.check(status, "w8a16_matmul")

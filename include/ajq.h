@@ -72,8 +72,8 @@ int ajq_quantize_w8(const float* W, int N, int K, int8_t* q, uint16_t* scales, v
 int ajq_quantize_w4_g128(const float* W, int N, int K, int32_t* qweight, uint16_t* scales,
                          uint8_t* zeros, void* stream);
 
-/* canonical -> kernel-private layout and back.  N % 16 == 0; K % 128 == 0 (W4),
- * K % 64 == 0 (W8). */
+/* canonical -> kernel-private layout and back.  N % 16 == 0; K % 128 == 0 for W4,
+ * K % 64 == 0 for W8 (the W8 matmuls below additionally need K % 128 == 0). */
 int ajq_repack_w4(const int32_t* qweight, const uint16_t* scales, const uint8_t* zeros, int N, int K,
                   uint32_t* wq, uint32_t* meta, void* stream);
 int ajq_unrepack_w4(const uint32_t* wq, const uint32_t* meta, int N, int K, int32_t* qweight,
