@@ -191,16 +191,17 @@ int launch_gemv_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const u
   return AJQ_OK;
 }
 
-// Row bound MROWS is the next power of two >= M; the slice a wave stages shrinks
-// (TPW 4 -> 2, twice the waves) when 16 rows would not fit the LDS otherwise.
+// Row bound MROWS is the next power of two >= M; above 4 rows a wave stages two
+// k groups at a time instead of four, which keeps the two register sets of the
+// ping-pong inside the VGPR budget and the slices inside 80 KiB of LDS.
 template <bool kW4>
 int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                 const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   if (M <= 1) return launch_gemv_cfg<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 2) return launch_gemv_cfg<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 4) return launch_gemv_cfg<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  if (M <= 8) return launch_gemv_cfg<8, 4, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  return launch_gemv_cfg<16, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 8) return launch_gemv_cfg<8, 2, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_gemv_cfg<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
 }  // namespace

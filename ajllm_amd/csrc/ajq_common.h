@@ -37,14 +37,16 @@ __device__ __forceinline__ u32x4_t w4_to_bf16_biased(uint32_t w) {
   return r;
 }
 
-// Four int8 (one dword, k order) -> two dwords of bf16 pairs, exact.
+// Four int8 (one dword, k order) -> two dwords of bf16 pairs, exact: one SDWA
+// convert per byte (sign-extending byte select), one v_perm_b32 per pair.
+// |q| <= 127 has at most 7 significant bits, so the high half of the fp32 IS the bf16.
 __device__ __forceinline__ u32x2_t w8_to_bf16(uint32_t w) {
-  float f0 = (float)(int8_t)(w & 0xFF);
-  float f1 = (float)(int8_t)((w >> 8) & 0xFF);
-  float f2 = (float)(int8_t)((w >> 16) & 0xFF);
-  float f3 = (float)(int8_t)(w >> 24);
+  float f0, f1, f2, f3;
+  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(f0) : "v"(w));
+  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(f1) : "v"(w));
+  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(f2) : "v"(w));
+  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(f3) : "v"(w));
   u32x2_t r;
-  // |q| <= 127 has at most 7 significant bits: the high half of the fp32 is the bf16.
   r.x = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
   r.y = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
   return r;

@@ -41,6 +41,15 @@ __device__ __forceinline__ u32x4_t w4_unpack(uint32_t w, uint32_t mask, uint32_t
   return r;
 }
 
+// One batch of a wave: TPW consecutive k groups, their weights, meta words and the
+// matching slice of the activations, all in registers.
+template <int TPW, int kXLoads, int kLoadsPerGroup>
+struct GemvBatch {
+  u32x4_t x[kXLoads];
+  u32x4_t w[TPW][kLoadsPerGroup];
+  uint32_t m[TPW];
+};
+
 // kWaves waves per workgroup; a wave works through its k groups TPW at a time;
 // MROWS >= M is the compile-time row bound that sizes the activation slice.
 template <int kWaves, int TPW, int MROWS, bool kW4>
@@ -52,11 +61,14 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
   constexpr int kStride = kSlice + 8;      // padded LDS row, bf16 elements
   constexpr int kVecPerRow = kSlice / 8;   // 16-byte vectors per slice row
-  constexpr int kXLoads = (MROWS * kVecPerRow + 63) / 64;
+  constexpr int kVecs = MROWS * kVecPerRow;
+  constexpr int kXLoads = (kVecs + 63) / 64;
   constexpr int kLoadsPerGroup = kW4 ? 1 : 2;  // 1 KiB tiles per 128 k
+  using Batch = GemvBatch<TPW, kXLoads, kLoadsPerGroup>;
 
   extern __shared__ u32x4_t smem_raw[];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: scalar branches
   const int nl = lane & 15, kc = lane >> 4;
   const int nt = blockIdx.x;
   const int G = K >> 7;
@@ -70,28 +82,24 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   const u32x4_t* wtile = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
   const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
 
-  u32x4_t xv[kXLoads];
-  u32x4_t wv[TPW][kLoadsPerGroup];
-  uint32_t mv[TPW];
-
-  auto load_x = [&](int g0) {  // activations of groups [g0, g0 + TPW) -> registers
+  // Every load below is unconditional (addresses are clamped into the wave's own
+  // range instead), so the number of loads in flight is static and the compiler
+  // can wait for exactly the tile it is about to use.
+  auto load = [&](Batch& b, int g0) {
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
-      const int v = lane + 64 * i;
-      const int m = v / kVecPerRow, c = v % kVecPerRow;
-      if (m < M && g0 * kGroup + 8 * c < K)
-        xv[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g0 * kGroup + 8 * c);
+      const int v = min(lane + 64 * i, kVecs - 1);
+      const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
+      const int k = min(g0 * kGroup + 8 * c, K - 8);
+      b.x[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + k);
     }
-  };
-  auto load_w = [&](int g0) {
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
-      if (g0 + p < g_end) {
+      const int g = min(g0 + p, g_end - 1);
 #pragma unroll
-        for (int h = 0; h < kLoadsPerGroup; ++h)
-          wv[p][h] = __builtin_nontemporal_load(wtile + ((size_t)(g0 + p) * kLoadsPerGroup + h) * 64);
-        if (kW4) mv[p] = mtile[(size_t)(g0 + p) * 16];
-      }
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
+      if (kW4) b.m[p] = mtile[(size_t)g * 16];
     }
   };
 
@@ -103,31 +111,14 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   const uint16_t* xrow = xs + row * kStride + 8 * kc;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
-  if (g_begin < g_end) {
-    load_x(g_begin);
-    load_w(g_begin);
-  }
-  for (int g0 = g_begin; g0 < g_end; g0 += TPW) {
-    // slice of this batch -> wave-private LDS (LDS ops of one wave execute in order,
-    // so the reads of the previous batch are already done)
+  auto compute = [&](Batch& b, int g0) {
+    // slice of this batch -> wave-private LDS.  LDS operations of one wave execute
+    // in order, so the reads of the previous batch are already done.
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = lane + 64 * i;
-      const int m = v / kVecPerRow, c = v % kVecPerRow;
-      if (m < M && g0 * kGroup + 8 * c < K) *reinterpret_cast<u32x4_t*>(xs + m * kStride + 8 * c) = xv[i];
-    }
-    // registers of this batch
-    u32x4_t wc[TPW][kLoadsPerGroup];
-    uint32_t mc[TPW];
-#pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-#pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h) wc[p][h] = wv[p][h];
-      mc[p] = mv[p];
-    }
-    if (g0 + TPW < g_end) {  // next batch in flight while this one is computed
-      load_x(g0 + TPW);
-      load_w(g0 + TPW);
+      if ((i + 1) * 64 <= kVecs || v < kVecs)
+        *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = b.x[i];
     }
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
@@ -137,24 +128,37 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-            const u32x4_t b = w4_unpack(wc[p][0][j], mask, magic);
-            part = mfma16(a, b, part);
+            const u32x4_t bw = w4_unpack(b.w[p][0][j], mask, magic);
+            part = mfma16(a, bw, part);
             asum = mfma16(a, ones, asum);
           }
-          const float s = f16_bits_to_f32(mc[p] & 0xFFFFu);
-          const float zc = f16_bits_to_f32(mc[p] >> 16);
+          const float s = f16_bits_to_f32(b.m[p] & 0xFFFFu);
+          const float zc = f16_bits_to_f32(b.m[p] >> 16);
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[i] += s * (part[i] - zc * asum[i]);
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-            const u32x2_t lo = w8_to_bf16(wc[p][j >> 1][2 * (j & 1)]);
-            const u32x2_t hi = w8_to_bf16(wc[p][j >> 1][2 * (j & 1) + 1]);
+            const u32x2_t lo = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1)]);
+            const u32x2_t hi = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1) + 1]);
             acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);
           }
         }
       }
+    }
+  };
+
+  // two register sets, ping-pong: the next batch is in flight while one is computed
+  if (g_begin < g_end) {
+    Batch b0, b1;
+    load(b0, g_begin);
+    for (int g0 = g_begin; g0 < g_end; g0 += 2 * TPW) {
+      const bool has1 = g0 + TPW < g_end;
+      if (has1) load(b1, g0 + TPW);
+      compute(b0, g0);
+      if (g0 + 2 * TPW < g_end) load(b0, g0 + 2 * TPW);
+      if (has1) compute(b1, g0 + TPW);
     }
   }
 

@@ -1,0 +1,87 @@
+"""The C-ABI library loads without a GPU, exports every symbol the header declares, and its
+argument validation (which runs before any HIP call) reports errors the way the header says."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from ajllm_amd import _lib
+
+HEADER = Path(__file__).resolve().parents[1] / "include" / "ajq.h"
+
+
+def _declared_functions() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(ajq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert len(names) >= 14
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in ajq.h but not exported by libajq.so"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.ajq_version() >= 1
+    assert lib.ajq_status_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert lib.ajq_status_string(code) not in (b"", b"unknown status")
+    assert lib.ajq_status_string(-99) == b"unknown status"
+
+
+def test_null_pointers_are_rejected_before_any_gpu_work():
+    lib = _lib.load()
+    assert lib.ajq_quantize_w8(None, 16, 128, None, None, None) == -1
+    assert lib.ajq_quantize_w4_g128(None, 16, 128, None, None, None, None) == -1
+    assert lib.ajq_w4a16_gemv(None, 1, 128, None, None, 16, None, 0, None) == -1
+    assert b"null" in lib.ajq_last_error()
+    with pytest.raises(ValueError):
+        _lib.check(-1, "probe")
+
+
+def test_shape_alignment_and_option_errors():
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096 + 16)
+    base = (ctypes.addressof(buf) + 15) & ~15  # host memory: only its address is inspected
+    p = ctypes.c_void_p(base)
+    odd = ctypes.c_void_p(base + 4)
+    assert lib.ajq_quantize_w4_g128(p, 16, 100, p, p, p, None) == -2      # K not a multiple of 128
+    assert lib.ajq_quantize_w8(p, 0, 128, p, p, None) == -2
+    assert lib.ajq_repack_w4(p, p, p, 10, 128, p, p, None) == -2            # N not a multiple of 16
+    assert lib.ajq_w4a16_gemv(p, 17, 128, p, p, 16, p, 0, None) == -2       # M beyond the GEMV range
+    assert b"M=17" in lib.ajq_last_error()
+    assert lib.ajq_w4a16_gemv(p, 1, 128, p, p, 16, p, 7, None) == -4        # unknown out_dtype
+    assert lib.ajq_w4a16_gemv(odd, 1, 128, p, p, 16, p, 0, None) == -3      # misaligned x
+    assert lib.ajq_w8a16_gemm(p, 1, 192, p, p, 16, p, 0, None) == -2
+    need = lib.ajq_w4a16_gemm_workspace_bytes(300, 512)
+    assert need == 4 * 512 * 4                                              # G=4 groups x 512 padded rows x fp32
+    assert lib.ajq_w4a16_gemm(p, 300, 512, p, p, 16, p, 0, None, 0, None) == -6
+    assert lib.ajq_w4a16_gemm(p, 300, 512, p, p, 16, p, 0, p, need - 1, None) == -6
+    with pytest.raises(ValueError):
+        _lib.check(-6, "probe")
+    with pytest.raises(RuntimeError):
+        _lib.check(-5, "probe")
+
+
+def test_python_layer_refuses_cpu_tensors():
+    """There is no CPU fallback: the host API raises instead of computing elsewhere."""
+    import torch
+
+    from ajllm_amd import QuantLinear, quantize_w4_g128, w4a16_matmul
+
+    with pytest.raises(ValueError):
+        quantize_w4_g128(torch.zeros(16, 128))
+    with pytest.raises(ValueError):
+        QuantLinear.from_weight(torch.zeros(16, 128))
+    with pytest.raises(ValueError):
+        QuantLinear(128, 16, scheme="w2")
+    with pytest.raises(RuntimeError):
+        QuantLinear(128, 16)(torch.zeros(1, 128))
+    assert w4a16_matmul.__module__ == "ajllm_amd.quant"
