@@ -188,4 +188,7 @@ class QuantLinearRef(torch.nn.Module):
         return w
 
     def forward(self, inputs: torch.Tensor) -> torch.Tensor:
-        return quant_linear(inputs, self.dequantized())
+        # "A16": the activations the matmul sees are bf16; other input dtypes are rounded to
+        # bf16 first and the fp32-accumulated result is returned in the input's dtype.
+        x = inputs if inputs.dtype == torch.bfloat16 else inputs.to(torch.bfloat16)
+        return quant_linear(x, self.dequantized(), out_dtype=inputs.dtype)

@@ -46,3 +46,32 @@ def bf16_rounding_excess(got16: torch.Tensor, want: torch.Tensor, eps: float) ->
 # north-star tolerances for floating-point outputs
 MAX_ABS_TOL = 1e-2
 REL_FRO_TOL = 2e-3
+
+
+def compare_greedy(tokens_got: torch.Tensor, tokens_ref: torch.Tensor, margins_ref: torch.Tensor,
+                   prompt_len: int, noise: float) -> dict:
+    """Compare two greedy decodes of the same prompts.
+
+    Rows are compared up to their first differing token.  A first difference is *attributable*
+    when the reference's top-1 minus top-2 logit at that step is below ``noise`` (the two runs
+    may then legitimately pick different tokens: their logits differ by accumulation-order
+    noise); everything after it is a different context and says nothing.  Returns counts and the
+    smallest margin met on the compared prefix."""
+    got, ref = tokens_got.cpu(), tokens_ref.cpu()
+    rows = ref.shape[0]
+    identical_rows, attributable, unexplained = 0, [], []
+    min_margin = float("inf")
+    for b in range(rows):
+        diff = (got[b, prompt_len:] != ref[b, prompt_len:]).nonzero()
+        first = int(diff[0]) if len(diff) else None
+        upto = first if first is not None else ref.shape[1] - prompt_len
+        if upto:
+            min_margin = min(min_margin, float(margins_ref[b, :upto].min()))
+        if first is None:
+            identical_rows += 1
+        elif float(margins_ref[b, first]) < noise:
+            attributable.append((b, first, float(margins_ref[b, first])))
+        else:
+            unexplained.append((b, first, float(margins_ref[b, first])))
+    return {"rows": rows, "identical_rows": identical_rows, "attributable": attributable,
+            "unexplained": unexplained, "min_margin_on_compared_prefix": min_margin}
