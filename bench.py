@@ -30,6 +30,7 @@ import torch
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor peak
+GEMV_W4_4096_M1_HBM_BYTES = 9.49e6  # measured: 4423 KiB x 2.093 fetched + 8 KiB x 1.047 written per launch
 
 
 def log(*args) -> None:
@@ -255,6 +256,13 @@ def main() -> int:
         from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
 
         extras["decode"] = bench_decode(device, log)
+    # a plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
+    # counters of a profiling run are scaled by (64 MiB read + 64 MiB written per launch)
+    calib_src = torch.empty(64 * 2**20, dtype=torch.uint8, device=device)
+    calib_dst = torch.empty_like(calib_src)
+    for _ in range(3):
+        calib_dst.copy_(calib_src)
+    torch.cuda.synchronize()
     cpu = None if args.no_cpu else cpu_baseline(m, n, k)
     if cpu:
         log("cpu_baseline", json.dumps(cpu))
@@ -284,8 +292,10 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": head["frac_hbm_peak"],
-            "traffic": None,
-            "kernel": "w4a16_gemv_kernel",
+            # HBM bytes per launch from separate rocprofv3 --pmc runs of this command
+            # (FETCH_SIZE, WRITE_SIZE, each scaled by what a 64 MiB copy reads on the same counter)
+            "traffic": GEMV_W4_4096_M1_HBM_BYTES,
+            "kernel": "ajq::dequant_gemv_kernel<8, 4, 1, true>",
             "algorithmic_bytes_per_launch": head["bytes_per_launch"],
             "avg_launch_us": head["us_per_launch"],
         },
