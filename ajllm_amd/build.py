@@ -24,6 +24,9 @@ HIPCC_FLAGS = [
     "-shared",
     # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # kernel arguments arrive in SGPRs with the wave instead of by a scalar load
+    # at its start (the short GEMV kernels issue their first loads that much sooner)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 
 

@@ -179,16 +179,26 @@ int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream) {
 // --------------------------------------------------------------- GEMV -----
 namespace {
 
-template <int kWaves, int TPW, int MROWS, bool kW4>
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
 int launch_gemv_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                     const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   constexpr size_t lds = gemv_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4>;
+  auto kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4, kSingle>;
   if (int s = allow_big_lds(kernel, lds)) return s;
-  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, x, M, K,
-                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8, N, y, out_f32);
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M | (out_f32 << 8), N, y, scales8);
   return AJQ_OK;
+}
+
+// One wave stages TPW k groups at a time; K == kWaves * TPW * 128 takes the
+// straight-line variant of the kernel.
+template <int kWaves, int TPW, int MROWS, bool kW4>
+int launch_gemv_rows(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                     const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  if (K == kWaves * TPW * kGroup)
+    return launch_gemv_cfg<kWaves, TPW, MROWS, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_gemv_cfg<kWaves, TPW, MROWS, kW4, false>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
 // Row bound MROWS is the next power of two >= M; above 4 rows a wave stages two
@@ -197,11 +207,11 @@ int launch_gemv_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const u
 template <bool kW4>
 int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                 const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
-  if (M <= 1) return launch_gemv_cfg<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  if (M <= 2) return launch_gemv_cfg<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  if (M <= 4) return launch_gemv_cfg<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  if (M <= 8) return launch_gemv_cfg<8, 2, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  return launch_gemv_cfg<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 1) return launch_gemv_rows<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 2) return launch_gemv_rows<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 4) return launch_gemv_rows<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 8) return launch_gemv_rows<8, 2, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_gemv_rows<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
 }  // namespace

@@ -56,14 +56,9 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t bits16) {
   return __half2float(__ushort_as_half((unsigned short)bits16));
 }
 
-// fp32 -> bf16 bits, round to nearest even (inputs are finite sums).
+// fp32 -> bf16 bits, round to nearest even (one v_cvt_pk_bf16_f32; NaN stays NaN).
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7F800000u) == 0x7F800000u) {  // inf / nan: keep class
-    return (uint16_t)((u >> 16) | ((u & 0xFFFFu) ? 0x40u : 0u));
-  }
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 }  // namespace ajq

@@ -1,22 +1,26 @@
 // Decode dequant-GEMV, 1 <= M <= 16:  y[M, N] = x[M, K] @ W_hat[N, K]^T.
 //
-// HBM-bound and short (a 4096 x 4096 int4 matrix is 8.7 MB, about a microsecond
-// of HBM time), so the kernel is built to have every byte in flight as early as
-// possible and to do its arithmetic while the bytes arrive:
+// HBM-bound and short: a 4096 x 4096 int4 matrix is 8.7 MB, which the memory
+// system delivers in well under two microseconds, and a wave's tiles (contiguous
+// KiB) land together in one burst.  What the kernel can influence is how soon
+// its loads are in flight and how little work is left once the weights are
+// there, so it is laid out around that:
 //  * one workgroup owns one 16-row tile of N and all of K; wave w owns a
 //    contiguous run of 128-wide k groups, i.e. a contiguous run of 1 KiB private
 //    weight tiles, and loads each with one 128-bit load per lane (a wave-wide
-//    load instruction reads one contiguous KiB), non-temporal, issued up front;
+//    load instruction reads one contiguous KiB), non-temporal;
+//  * a wave issues its weight loads before anything else (vector loads complete
+//    in issue order, and every load instruction of the eight waves shares the
+//    CU's one address path, so whatever is issued first delays the HBM requests);
+//    then ITS k-slice of the activations, which it stages in a wave-private LDS
+//    region (rows padded by 16 B; no workgroup barrier) and reads back as MFMA A
+//    fragments, and the meta words;
+//  * the per-group activation sums the zero-point term needs come from a second
+//    MFMA against an all-ones B operand, which lands them in exactly the
+//    accumulator layout that uses them;
 //  * weights go global -> registers -> in-register unpack (3 shifts + 4
-//    v_and_or_b32 per 8 nibbles) -> MFMA B operand; they never touch LDS;
-//  * each wave stages only ITS k-slice of the activations in a wave-private LDS
-//    region (rows padded by 16 B: the 16 rows of an A fragment fall in distinct
-//    banks) and reads it back as MFMA A fragments, so there is no workgroup
-//    barrier before the arithmetic; rows >= M of the A operand repeat row M-1 and
-//    their outputs are never stored;
-//  * group sums of the activations (needed for the zero-point term) come from a
-//    second MFMA against an all-ones B operand, which lands them in exactly the
-//    accumulator layout that needs them;
+//    v_and_or_b32 per 8 nibbles) -> MFMA B operand; they never touch LDS.  Rows
+//    >= M of the A operand repeat row M-1 and their outputs are never stored;
 //  * the waves' partial sums meet once, through LDS, in a fixed order: no
 //    atomics, results are run-to-run identical.
 #pragma once
@@ -45,25 +49,32 @@ __device__ __forceinline__ u32x4_t w4_unpack(uint32_t w, uint32_t mask, uint32_t
 // matching slice of the activations, all in registers.
 template <int TPW, int kXLoads, int kLoadsPerGroup>
 struct GemvBatch {
-  u32x4_t x[kXLoads];
   u32x4_t w[TPW][kLoadsPerGroup];
+  u32x4_t x[kXLoads];
   uint32_t m[TPW];
 };
 
 // kWaves waves per workgroup; a wave works through its k groups TPW at a time;
 // MROWS >= M is the compile-time row bound that sizes the activation slice.
-template <int kWaves, int TPW, int MROWS, bool kW4>
+// kSingle: K == kWaves * TPW * 128, every wave has exactly one full batch (no
+// loop, no clamped addresses, no tail tests).
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
-    const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
+    const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
-    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
-    int N, void* __restrict__ y, int out_f32) {
+    const uint16_t* __restrict__ x, int K,
+    int m_flags,  // M | out_f32 << 8 (one word: the leading arguments arrive preloaded in SGPRs)
+    int N, void* __restrict__ y,
+    const uint16_t* __restrict__ scales8) {  // W8: fp16 [N]; W4: unused
+  const int M = m_flags & 0xFF;
+  const bool out_f32 = (m_flags >> 8) != 0;
   constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
   constexpr int kStride = kSlice + 8;      // padded LDS row, bf16 elements
   constexpr int kVecPerRow = kSlice / 8;   // 16-byte vectors per slice row
   constexpr int kVecs = MROWS * kVecPerRow;
   constexpr int kXLoads = (kVecs + 63) / 64;
   constexpr int kLoadsPerGroup = kW4 ? 1 : 2;  // 1 KiB tiles per 128 k
+  constexpr int kRowQuads = (MROWS + 3) / 4;   // lane quarters (kc) that hold live output rows
   using Batch = GemvBatch<TPW, kXLoads, kLoadsPerGroup>;
 
   extern __shared__ u32x4_t smem_raw[];
@@ -75,32 +86,41 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * (MROWS * kStride);
   float* red = reinterpret_cast<float*>(reinterpret_cast<uint16_t*>(smem_raw) + kWaves * (MROWS * kStride));
 
-  const int per_wave = (G + kWaves - 1) / kWaves;
+  const int per_wave = kSingle ? TPW : (G + kWaves - 1) / kWaves;
   const int g_begin = wave * per_wave;
-  const int g_end = min(G, g_begin + per_wave);
+  const int g_end = kSingle ? g_begin + TPW : min(G, g_begin + per_wave);
 
   const u32x4_t* wtile = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
   const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
 
   // Every load below is unconditional (addresses are clamped into the wave's own
   // range instead), so the number of loads in flight is static and the compiler
-  // can wait for exactly the tile it is about to use.
+  // can wait for exactly the operand it is about to use.
   auto load = [&](Batch& b, int g0) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      const int g = kSingle ? g0 + p : min(g0 + p, g_end - 1);
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
+    }
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = min(lane + 64 * i, kVecs - 1);
       const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
-      const int k = min(g0 * kGroup + 8 * c, K - 8);
+      const int k = kSingle ? g0 * kGroup + 8 * c : min(g0 * kGroup + 8 * c, K - 8);
       b.x[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + k);
     }
+    if (kW4) {
 #pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      const int g = min(g0 + p, g_end - 1);
-#pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h)
-        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
-      if (kW4) b.m[p] = mtile[(size_t)g * 16];
+      for (int p = 0; p < TPW; ++p)
+        b.m[p] = mtile[(size_t)(kSingle ? g0 + p : min(g0 + p, g_end - 1)) * 16];
     }
+    // the whole batch is in flight before anything else happens: left alone, the
+    // instruction scheduler sinks loads towards their first use and turns one
+    // memory round trip into several
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   const uint32_t mask = 0x000F000Fu;
@@ -112,6 +132,19 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](Batch& b, int g0) {
+    // The meta words are the last loads of the batch and their conversion is its
+    // first use: a wave's tiles arrive together, so waiting for all of the batch
+    // here costs nothing, and it keeps the scheduler from sinking those loads
+    // below an earlier wait (a second memory round trip).
+    float sc[TPW], zc[TPW];
+    if (kW4) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) {
+        sc[p] = f16_bits_to_f32(b.m[p] & 0xFFFFu);
+        zc[p] = f16_bits_to_f32(b.m[p] >> 16);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     // slice of this batch -> wave-private LDS.  LDS operations of one wave execute
     // in order, so the reads of the previous batch are already done.
 #pragma unroll
@@ -120,23 +153,28 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
       if ((i + 1) * 64 <= kVecs || v < kVecs)
         *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = b.x[i];
     }
+    if (kW4) {
 #pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      if (g0 + p < g_end) {
-        if (kW4) {
+      for (int p = 0; p < TPW; ++p) {
+        if (kSingle || g0 + p < g_end) {
+          // the group's activation sums (for the zero-point term) come from a second
+          // MFMA against an all-ones B operand: same layout as the accumulator
           f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-            const u32x4_t bw = w4_unpack(b.w[p][0][j], mask, magic);
-            part = mfma16(a, bw, part);
+            part = mfma16(a, w4_unpack(b.w[p][0][j], mask, magic), part);
             asum = mfma16(a, ones, asum);
           }
-          const float s = f16_bits_to_f32(b.m[p] & 0xFFFFu);
-          const float zc = f16_bits_to_f32(b.m[p] >> 16);
+          // (128+q) and (128+z) cancel in fp32 before the scale is applied
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[i] += s * (part[i] - zc * asum[i]);
-        } else {
+          for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) {
+        if (kSingle || g0 + p < g_end) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
@@ -150,7 +188,11 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   };
 
   // two register sets, ping-pong: the next batch is in flight while one is computed
-  if (g_begin < g_end) {
+  if (kSingle) {
+    Batch b0;
+    load(b0, g_begin);
+    compute(b0, g_begin);
+  } else if (g_begin < g_end) {
     Batch b0, b1;
     load(b0, g_begin);
     for (int g0 = g_begin; g0 < g_end; g0 += 2 * TPW) {
@@ -162,18 +204,31 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
     }
   }
 
-  // ---- the waves' partial sums meet in LDS; wave 0 adds them in wave order
-  reinterpret_cast<f32x4_t*>(red)[wave * 64 + lane] = acc;
-  __syncthreads();
-  if (wave != 0) return;
-  f32x4_t sum = reinterpret_cast<f32x4_t*>(red)[lane];
+  // ---- the waves' partial sums meet in LDS; wave 0 adds them in wave order.
+  // Only the lane quarters that hold rows < MROWS take part.
+  // (the empty asm pins the accumulator here: otherwise the compiler sinks the
+  // epilogue arithmetic, and the loads that feed it, into the conditional store)
+  asm volatile("" : "+v"(acc));
+  constexpr int kLive = MROWS < 4 ? MROWS : 4;  // accumulator components that hold rows < MROWS
+  typedef float live_t __attribute__((ext_vector_type(kLive == 3 ? 4 : kLive)));
+  live_t* redv = reinterpret_cast<live_t*>(red);
+  live_t mine;
 #pragma unroll
-  for (int w = 1; w < kWaves; ++w) sum += reinterpret_cast<f32x4_t*>(red)[w * 64 + lane];
+  for (int i = 0; i < kLive; ++i) mine[i] = acc[i];
+  if (kc < kRowQuads) redv[wave * (16 * kRowQuads) + lane] = mine;
+  __syncthreads();
+  if (wave != 0 || kc >= kRowQuads) return;
+  live_t part[kWaves];
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) part[w] = redv[w * (16 * kRowQuads) + lane];
+  live_t sum = part[0];
+#pragma unroll
+  for (int w = 1; w < kWaves; ++w) sum += part[w];
   const int n = nt * kTileN + nl;
   float cs = 1.0f;
   if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < kLive; ++i) {
     const int m = 4 * kc + i;
     if (m < M) {
       const float v = sum[i] * cs;
