@@ -78,6 +78,27 @@ int launch_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
   return AJQ_OK;
 }
 
+// 256 x 128 tiles on 32x32x16 MFMA; M >= 256 (the last row tile is shifted, not masked)
+template <int MT, bool kW4>
+int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                   const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
+  auto kernel = dequant_gemm256_kernel<MT, kW4>;
+  if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
+  const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
+                     reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
+  return AJQ_OK;
+}
+
+constexpr int kGemm256MinM = 256;
+#ifndef AJQ_G2_MT_W4
+#define AJQ_G2_MT_W4 2
+#endif
+#ifndef AJQ_G2_MT_W8
+#define AJQ_G2_MT_W8 4
+#endif
+
 }  // namespace
 
 extern "C" {
@@ -239,7 +260,8 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 // --------------------------------------------------------------- GEMM -----
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K) {
   if (M < 1 || K < kGroup) return 0;
-  return (size_t)(K / kGroup) * round_up(M, kGemmMpadTo) * sizeof(float);
+  // covers both layouts: fp32 [G][Mpad] (small M) and 16-byte pieces [G][M] (M >= 256)
+  return (size_t)(K / kGroup) * round_up(M, kGemmMpadTo) * 16;
 }
 
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
@@ -249,9 +271,19 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   if (!workspace || workspace_bytes < need)
     return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm: workspace must be 16-byte aligned");
+  const long long teams = (long long)M * (K / kGroup);
+  if (M >= kGemm256MinM) {
+    if ((long long)M * K * 2 >= (1LL << 32))
+      return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+    hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
+                       K, reinterpret_cast<u32x4_t*>(workspace));
+    if (int s = launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_dtype == AJQ_OUT_F32,
+                                     (hipStream_t)stream))
+      return s;
+    return check_launch("ajq_w4a16_gemm");
+  }
   const int Mpad = round_up(M, kGemmMpadTo);
   float* gsum = reinterpret_cast<float*>(workspace);
-  const long long teams = (long long)M * (K / kGroup);
   hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
                      K, Mpad, gsum);
   int s;
@@ -268,6 +300,14 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
                    int out_dtype, void* stream) {
   if (int s = check_matmul_args("ajq_w8a16_gemm", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
+  if (M >= kGemm256MinM) {
+    if ((long long)M * K * 2 >= (1LL << 32))
+      return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+    if (int s = launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_dtype == AJQ_OUT_F32,
+                                      (hipStream_t)stream))
+      return s;
+    return check_launch("ajq_w8a16_gemm");
+  }
   int s;
   if (M <= 64)
     s = launch_gemm<64, 64, 32, 32, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,

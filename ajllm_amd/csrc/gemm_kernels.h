@@ -215,4 +215,268 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void dequant_gemm_kerne
 }
 
 
+
+// ===========================================================================
+// Large-M prefill GEMM (M >= 256): 256 x 128 output tile per workgroup, 4 waves
+// (2 x 2), wave tile 128 x 64 on v_mfma_f32_32x32x16_bf16.
+//
+//  * Activations go global -> LDS directly (global_load_lds_dwordx4, no register
+//    staging).  One k-block of the tile is 256 rows x 256 B, exactly 64 KiB, rows
+//    unpadded; the 16-byte chunk c of row r sits in slot c ^ (r & 15) of its row,
+//    so the 32 rows of an A fragment read fall in distinct banks.  A wave-wide
+//    load fills 1 KiB of LDS (4 rows) from 4 row segments of 256 B.
+//  * W4 zero-point: the per-row group sums, split into three bf16 pieces by
+//    group_sum3_kernel, ride in a 4 KiB side buffer; a ninth MFMA k-step per
+//    group multiplies them by -(128+z) (exact in bf16), so the fp32 partial sum of
+//    a group already is  sum_k a[m,k] * (q[n,k] - z[n,g]),  and what is left for
+//    the VALU is one FMA per accumulator element and group (acc += s * part).
+//  * Weights: every wave loads the private tiles of its own 64 columns straight
+//    into registers and unpacks them once per k-block into B fragments that hold
+//    exact small integers (128+q, or q for int8).
+//  * A wave walks its four 32-row blocks in turn: A fragments are read from LDS
+//    just in time and each feeds the two 32-column blocks of the wave.
+//  * The last row tile is shifted up to end at row M (M >= 256), so no row is
+//    clamped or masked; rows it shares with its neighbour are computed twice
+//    with identical results.
+// ===========================================================================
+
+// gs3[g][m] = 16 bytes: bf16 pieces h, m, l with h + m + l == the sum of the 128
+// activations of group g in row m to fp32 precision, then five zeros.
+__global__ __launch_bounds__(256) void group_sum3_kernel(const uint16_t* __restrict__ x, int M, int K,
+                                                         u32x4_t* __restrict__ gs3) {
+  const int G = K >> 7;
+  const long long team = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
+  if (team >= (long long)M * G) return;
+  const int sub = threadIdx.x & 15;
+  const int m = (int)(team / G), g = (int)(team % G);
+  const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g * kGroup + sub * 8);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    s += __uint_as_float(v[i] << 16);
+    s += __uint_as_float(v[i] & 0xFFFF0000u);
+  }
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
+  if (sub == 0) {
+    // truncation keeps every remainder exactly representable
+    const uint32_t hb = __float_as_uint(s) & 0xFFFF0000u;
+    const float r1 = s - __uint_as_float(hb);
+    const uint32_t mb = __float_as_uint(r1) & 0xFFFF0000u;
+    const float r2 = r1 - __uint_as_float(mb);
+    const uint32_t lb = (uint32_t)f32_to_bf16_rne(r2);
+    gs3[(size_t)g * M + m] = u32x4_t{(hb >> 16) | mb, lb, 0u, 0u};
+  }
+}
+
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void global_void_t;
+
+constexpr int kG2BM = 256, kG2BN = 128;
+constexpr int kG2TileBytes = kG2BM * 256;                         // 64 KiB: one k-block of activations
+constexpr int kG2SideBytes = kG2BM * 16;                          // 4 KiB: group-sum pieces
+constexpr size_t kG2LdsBytes = 2 * (size_t)(kG2TileBytes + kG2SideBytes);
+
+// MT = 32-row blocks per wave: 4 -> 4 waves (2 x 2, wave tile 128 x 64), 2 -> 8 waves
+// (4 x 2, wave tile 64 x 64, two waves per SIMD).
+template <int MT, bool kW4>
+__global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
+    const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
+    const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
+    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
+    const u32x4_t* __restrict__ gs3,       // W4: [K/128][M] group-sum pieces; W8: unused
+    int N, void* __restrict__ y, int out_f32) {
+  constexpr int kSteps = kW4 ? 9 : 8;       // MFMA k-steps per 128-k block
+  constexpr int kRawPerNt = kW4 ? 2 : 4;    // 128-bit weight loads per lane, 32 columns and k-block
+
+  extern __shared__ u32x4_t smem_raw[];
+  char* lds = reinterpret_cast<char*>(smem_raw);  // [2][64 KiB] tiles, then [2][4 KiB] side buffers
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  constexpr int kWaves = 16 / MT;          // 4 or 8
+  constexpr int kWaveRows = 32 * MT;       // rows of the tile one wave computes
+  constexpr int kLoadRows = kG2BM / kWaves;  // rows of the tile one wave loads
+  const int wm = wave >> 1, wn = wave & 1;
+  const int col = lane & 31, kh = lane >> 5;
+
+  // column-major walk over output tiles: consecutive workgroups share a column block of W
+  const int tiles_m = (M + kG2BM - 1) / kG2BM;
+  const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+  const int m0 = min(tile_m * kG2BM, M - kG2BM), n0 = tile_n * kG2BN;
+  const int G = K >> 7;
+  const int ntiles16 = N / kTileN;
+
+  // ---- activations.  Wave w fills kLoadRows rows of the tile with wave-wide loads
+  // of 4 rows each; lane (row_in = l >> 4, slot = l & 15) of load q fetches chunk
+  // slot ^ ((4q + row_in) & 15) of its row, which depends on q only through q & 3.
+  const int row_in = lane >> 4, slot = lane & 15;
+  uint32_t a_voff[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)((slot ^ (4 * v + row_in)) * 16);
+  const char* a_base = reinterpret_cast<const char*>(x) + (size_t)(m0 + kLoadRows * wave) * K * 2;
+  auto load_a = [&](int kb, int buf) {
+    char* dst = lds + buf * kG2TileBytes + wave * (kLoadRows * 256);
+    const char* src = a_base + (size_t)kb * 256;
+#pragma unroll
+    for (int q = 0; q < kLoadRows / 4; ++q)
+      __builtin_amdgcn_global_load_lds((global_void_t*)(src + (size_t)q * 4 * K * 2 + a_voff[q & 3]),
+                                       (lds_void_t*)(dst + q * 1024), 16, 0, 0);
+    if (kW4 && wave < 4)
+      __builtin_amdgcn_global_load_lds((global_void_t*)(gs3 + (size_t)kb * M + m0 + 64 * wave + lane),
+                                       (lds_void_t*)(lds + 2 * kG2TileBytes + buf * kG2SideBytes + wave * 1024),
+                                       16, 0, 0);
+  };
+
+  // ---- weights: lane (col, kh) of a 32-column block reads, from the 16-row private
+  // tile that holds its column, the 16 bytes of tile lanes (kc = kh) and (kc = kh + 2):
+  // dword j of the first is k-step 2j, of the second k-step 2j + 1.
+  u32x4_t raw[2][kRawPerNt];
+  uint32_t mraw[2];
+  auto load_b = [&](int kb) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int nt16 = min((n0 + wn * 64 + t * 32 + col) / kTileN, ntiles16 - 1);
+      const int nl = col & 15;
+      if (kW4) {
+        const u32x4_t* tile = wq + ((size_t)nt16 * G + kb) * 64;
+        raw[t][0] = tile[kh * 16 + nl];
+        raw[t][1] = tile[(kh + 2) * 16 + nl];
+        mraw[t] = meta[((size_t)nt16 * G + kb) * 16 + nl];
+      } else {
+        const u32x4_t* tile = wq + ((size_t)nt16 * (2 * G) + 2 * kb) * 64;
+        raw[t][0] = tile[kh * 16 + nl];
+        raw[t][1] = tile[(kh + 2) * 16 + nl];
+        raw[t][2] = tile[64 + kh * 16 + nl];
+        raw[t][3] = tile[64 + (kh + 2) * 16 + nl];
+      }
+    }
+  };
+
+  f32x16_t acc[MT][2];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
+
+  // ---- A fragment addresses: row r = kWaveRows wm + 32 i + col, chunk 2s + kh sits in slot
+  // (2s + kh) ^ (r & 15) = ((s ^ (col >> 1 & 7)) << 1) | (kh ^ (col & 1)).  The two tile
+  // buffers are 64 KiB apart, so one XOR flips all of them.
+  uint32_t a_off[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s)
+    a_off[s] = (uint32_t)((wm * kWaveRows + col) * 256 + (((s ^ ((col >> 1) & 7)) << 5) | ((kh ^ (col & 1)) << 4)));
+  uint32_t g_off = (uint32_t)(2 * kG2TileBytes + (wm * kWaveRows + col) * 16);
+
+  load_a(0, 0);
+  load_b(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  const uint32_t mask = 0x000F000Fu;
+  uint32_t magic = 0x43004300u;
+  asm volatile("" : "+v"(magic));
+
+  for (int kb = 0; kb < G; ++kb) {
+    const bool has_next = kb + 1 < G;
+    if (has_next) load_a(kb + 1, (kb + 1) & 1);
+
+    // ---- unpack this block's weights into B fragments
+    u32x4_t bf[2][kSteps];
+    float sc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      if (kW4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          bf[t][2 * j] = w4_unpack(raw[t][0][j], mask, magic);
+          bf[t][2 * j + 1] = w4_unpack(raw[t][1][j], mask, magic);
+        }
+        // ninth step: -(128 + z) against the three pieces of the group sum (lanes kh = 0 only)
+        const uint32_t z = (mraw[t] >> 19) & 0xFu;  // fp16(128 + z): z sits in mantissa bits 3..6
+        const uint32_t nz = kh == 0 ? (0xC300u | z) : 0u;
+        bf[t][8] = u32x4_t{nz | (nz << 16), nz, 0u, 0u};
+        sc[t] = f16_bits_to_f32(mraw[t] & 0xFFFFu);
+      } else {
+        // W8 tile tau (64 k), load h (kc = kh + 2h): dwords (2j, 2j+1) are k-step 4 tau + 2j + h
+#pragma unroll
+        for (int tau = 0; tau < 2; ++tau)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const u32x2_t lo = w8_to_bf16(raw[t][2 * tau + h][2 * j]);
+              const u32x2_t hi = w8_to_bf16(raw[t][2 * tau + h][2 * j + 1]);
+              bf[t][4 * tau + 2 * j + h] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
+      }
+    }
+    if (has_next) load_b(kb + 1);
+
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      if (kW4) {
+        f32x16_t part[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) part[t][r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+          const uint32_t off = (s < 8 ? a_off[s < 8 ? s : 0] + i * 32 * 256 : g_off + i * 32 * 16);
+          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(lds + off);
+#pragma unroll
+          for (int t = 0; t < 2; ++t) part[t] = mfma32(a, bf[t][s], part[t]);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][t][r] += sc[t] * part[t][r];
+      } else {
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(lds + a_off[s] + i * 32 * 256);
+#pragma unroll
+          for (int t = 0; t < 2; ++t) acc[i][t] = mfma32(a, bf[t][s], acc[i][t]);
+        }
+      }
+    }
+    // flip to the other tile / side buffer
+#pragma unroll
+    for (int s = 0; s < 8; ++s) a_off[s] ^= (uint32_t)kG2TileBytes;
+    g_off ^= (uint32_t)kG2SideBytes;
+    // the next tile must have landed and every wave must be done with this one
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulator register r of lane (col, kh) is row (r & 3) + 8 * (r >> 2) + 4 * kh
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int n = n0 + wn * 64 + t * 32 + col;
+    if (n >= N) continue;
+    float cs = 1.0f;
+    if (!kW4) cs = f16_bits_to_f32(scales8[n]);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        const float v = acc[i][t][r] * cs;
+        if (out_f32)
+          reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
+        else
+          reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+      }
+    }
+  }
+}
+
 }  // namespace ajq
