@@ -278,9 +278,19 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void global_void_t;
 
 constexpr int kG2BM = 256, kG2BN = 128;
-constexpr int kG2TileBytes = kG2BM * 256;                         // 64 KiB: one k-block of activations
-constexpr int kG2SideBytes = kG2BM * 16;                          // 4 KiB: group-sum pieces
-constexpr size_t kG2LdsBytes = 2 * (size_t)(kG2TileBytes + kG2SideBytes);
+constexpr int kG2TileBytes = kG2BM * 256;  // 64 KiB: one k-block of activations
+// LDS map (bytes).  Buffers of a pair differ in one address bit, so one XOR flips a
+// read offset from one to the other.
+//   [0, 128 Ki)            two activation tiles
+//   W4: [128 Ki, 136 Ki)   two 4 KiB side buffers (group-sum pieces)
+//       136 Ki, 152 Ki     two 8 KiB weight buffers (8 private tiles each)
+//       144 Ki, +512       two 512 B meta buffers
+//   W8: 128 Ki, 144 Ki     two 16 KiB weight buffers (16 private tiles each)
+constexpr int kG2SideBase = 2 * kG2TileBytes, kG2SideBytes = 4096;
+constexpr int kG2W4Base = kG2SideBase + 2 * kG2SideBytes, kG2MetaBase = kG2W4Base + 8192;
+constexpr int kG2W8Base = 2 * kG2TileBytes;
+constexpr int kG2WStride = 16384, kG2MetaStride = 512;
+constexpr size_t kG2LdsBytes = 160 * 1024;
 
 // MT = 32-row blocks per wave: 4 -> 4 waves (2 x 2, wave tile 128 x 64), 2 -> 8 waves
 // (4 x 2, wave tile 64 x 64, two waves per SIMD).
@@ -291,17 +301,18 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
     const u32x4_t* __restrict__ gs3,       // W4: [K/128][M] group-sum pieces; W8: unused
     int N, void* __restrict__ y, int out_f32) {
-  constexpr int kSteps = kW4 ? 9 : 8;       // MFMA k-steps per 128-k block
-  constexpr int kRawPerNt = kW4 ? 2 : 4;    // 128-bit weight loads per lane, 32 columns and k-block
+  constexpr int kSteps = kW4 ? 9 : 8;         // MFMA k-steps per 128-k block
+  constexpr int kWaves = 16 / MT;             // 4 or 8
+  constexpr int kWaveRows = 32 * MT;          // rows of the tile one wave computes
+  constexpr int kLoadRows = kG2BM / kWaves;   // rows of the tile one wave loads
+  constexpr int kBTiles = kW4 ? 8 : 16;       // 1 KiB private weight tiles per k-block and workgroup
+  constexpr int kWBase = kW4 ? kG2W4Base : kG2W8Base;
 
   extern __shared__ u32x4_t smem_raw[];
-  char* lds = reinterpret_cast<char*>(smem_raw);  // [2][64 KiB] tiles, then [2][4 KiB] side buffers
+  char* lds = reinterpret_cast<char*>(smem_raw);
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  constexpr int kWaves = 16 / MT;          // 4 or 8
-  constexpr int kWaveRows = 32 * MT;       // rows of the tile one wave computes
-  constexpr int kLoadRows = kG2BM / kWaves;  // rows of the tile one wave loads
   const int wm = wave >> 1, wn = wave & 1;
   const int col = lane & 31, kh = lane >> 5;
 
@@ -312,49 +323,45 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   const int G = K >> 7;
   const int ntiles16 = N / kTileN;
 
-  // ---- activations.  Wave w fills kLoadRows rows of the tile with wave-wide loads
-  // of 4 rows each; lane (row_in = l >> 4, slot = l & 15) of load q fetches chunk
-  // slot ^ ((4q + row_in) & 15) of its row, which depends on q only through q & 3.
+  // ---- global -> LDS, one k-block ahead, no registers in between.
+  // Activations: wave w fills kLoadRows rows with wave-wide loads of 4 rows each.  Chunk c
+  // of row r lives in slot (c & 8) | ((c & 7) ^ (r & 7)) of its row; lane (row_in, slot) of
+  // load q therefore fetches chunk (slot & 8) | ((slot & 7) ^ ((4q + row_in) & 7)), which
+  // depends on q only through q & 1.
   const int row_in = lane >> 4, slot = lane & 15;
-  uint32_t a_voff[4];
+  uint32_t a_voff[2];
 #pragma unroll
-  for (int v = 0; v < 4; ++v) a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)((slot ^ (4 * v + row_in)) * 16);
+  for (int v = 0; v < 2; ++v)
+    a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)(((slot & 8) | ((slot & 7) ^ ((4 * v + row_in) & 7))) * 16);
   const char* a_base = reinterpret_cast<const char*>(x) + (size_t)(m0 + kLoadRows * wave) * K * 2;
-  auto load_a = [&](int kb, int buf) {
+  const int nt16_0 = n0 / kTileN;
+  auto load_tiles = [&](int kb, int buf) {
     char* dst = lds + buf * kG2TileBytes + wave * (kLoadRows * 256);
     const char* src = a_base + (size_t)kb * 256;
 #pragma unroll
     for (int q = 0; q < kLoadRows / 4; ++q)
-      __builtin_amdgcn_global_load_lds((global_void_t*)(src + (size_t)q * 4 * K * 2 + a_voff[q & 3]),
+      __builtin_amdgcn_global_load_lds((global_void_t*)(src + (size_t)q * 4 * K * 2 + a_voff[q & 1]),
                                        (lds_void_t*)(dst + q * 1024), 16, 0, 0);
     if (kW4 && wave < 4)
       __builtin_amdgcn_global_load_lds((global_void_t*)(gs3 + (size_t)kb * M + m0 + 64 * wave + lane),
-                                       (lds_void_t*)(lds + 2 * kG2TileBytes + buf * kG2SideBytes + wave * 1024),
-                                       16, 0, 0);
-  };
-
-  // ---- weights: lane (col, kh) of a 32-column block reads, from the 16-row private
-  // tile that holds its column, the 16 bytes of tile lanes (kc = kh) and (kc = kh + 2):
-  // dword j of the first is k-step 2j, of the second k-step 2j + 1.
-  u32x4_t raw[2][kRawPerNt];
-  uint32_t mraw[2];
-  auto load_b = [&](int kb) {
+                                       (lds_void_t*)(lds + kG2SideBase + buf * kG2SideBytes + wave * 1024), 16, 0, 0);
+    // weights: a private tile is 1 KiB contiguous, one wave-wide load each
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int nt16 = min((n0 + wn * 64 + t * 32 + col) / kTileN, ntiles16 - 1);
-      const int nl = col & 15;
-      if (kW4) {
-        const u32x4_t* tile = wq + ((size_t)nt16 * G + kb) * 64;
-        raw[t][0] = tile[kh * 16 + nl];
-        raw[t][1] = tile[(kh + 2) * 16 + nl];
-        mraw[t] = meta[((size_t)nt16 * G + kb) * 16 + nl];
-      } else {
-        const u32x4_t* tile = wq + ((size_t)nt16 * (2 * G) + 2 * kb) * 64;
-        raw[t][0] = tile[kh * 16 + nl];
-        raw[t][1] = tile[(kh + 2) * 16 + nl];
-        raw[t][2] = tile[64 + kh * 16 + nl];
-        raw[t][3] = tile[64 + (kh + 2) * 16 + nl];
-      }
+    for (int u = 0; u < kBTiles / kWaves; ++u) {
+      const int T = wave * (kBTiles / kWaves) + u;
+      const u32x4_t* tile;
+      if (kW4)
+        tile = wq + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 64;
+      else
+        tile = wq + ((size_t)min(nt16_0 + (T >> 1), ntiles16 - 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
+      __builtin_amdgcn_global_load_lds((global_void_t*)(tile + lane),
+                                       (lds_void_t*)(lds + kWBase + buf * kG2WStride + T * 1024), 16, 0, 0);
+    }
+    if (kW4 && wave < 2) {  // meta words of 4 tiles per load
+      const int T = wave * 4 + (lane >> 4);
+      __builtin_amdgcn_global_load_lds(
+          (global_void_t*)(meta + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 16 + (lane & 15)),
+          (lds_void_t*)(lds + kG2MetaBase + buf * kG2MetaStride + wave * 256), 4, 0, 0);
     }
   };
 
@@ -366,17 +373,21 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
 
-  // ---- A fragment addresses: row r = kWaveRows wm + 32 i + col, chunk 2s + kh sits in slot
-  // (2s + kh) ^ (r & 15) = ((s ^ (col >> 1 & 7)) << 1) | (kh ^ (col & 1)).  The two tile
-  // buffers are 64 KiB apart, so one XOR flips all of them.
-  uint32_t a_off[8];
+  // ---- LDS read offsets.  A fragment of k-step s, row r = kWaveRows wm + 32 i + col: chunk
+  // 2s + kh sits at byte (s >> 2) * 128 + (((s & 3) ^ (col >> 1 & 3)) << 5) + ((kh ^ (col & 1)) << 4).
+  uint32_t a_off[4];
 #pragma unroll
-  for (int s = 0; s < 8; ++s)
-    a_off[s] = (uint32_t)((wm * kWaveRows + col) * 256 + (((s ^ ((col >> 1) & 7)) << 5) | ((kh ^ (col & 1)) << 4)));
-  uint32_t g_off = (uint32_t)(2 * kG2TileBytes + (wm * kWaveRows + col) * 16);
+  for (int v = 0; v < 4; ++v)
+    a_off[v] = (uint32_t)((wm * kWaveRows + col) * 256 + (((v ^ ((col >> 1) & 3)) << 5) | ((kh ^ (col & 1)) << 4)));
+  uint32_t g_off = (uint32_t)(kG2SideBase + (wm * kWaveRows + col) * 16);
+  // weights: lane (col, kh) of 32-column block t reads, from the 16-row private tile that
+  // holds its column, the 16 bytes of tile lanes (kc = kh) and (kc = kh + 2): dword j of the
+  // first is k-step 2j, of the second k-step 2j + 1.
+  const int c16 = wn * 4 + (col >> 4), nl = col & 15;
+  uint32_t b_off = (uint32_t)(kWBase + (kW4 ? c16 : 2 * c16) * 1024 + (kh * 16 + nl) * 16);
+  uint32_t m_off = (uint32_t)(kG2MetaBase + (c16 * 16 + nl) * 4);
 
-  load_a(0, 0);
-  load_b(0);
+  load_tiles(0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
@@ -385,74 +396,99 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   asm volatile("" : "+v"(magic));
 
   for (int kb = 0; kb < G; ++kb) {
-    const bool has_next = kb + 1 < G;
-    if (has_next) load_a(kb + 1, (kb + 1) & 1);
+    if (kb + 1 < G) load_tiles(kb + 1, (kb + 1) & 1);
 
-    // ---- unpack this block's weights into B fragments
-    u32x4_t bf[2][kSteps];
-    float sc[2];
+    // ---- this block's packed weights, LDS -> registers
+    u32x4_t raw[2][kW4 ? 2 : 4];
+    uint32_t mraw[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
+      const int tb = t * (kW4 ? 2048 : 4096);
+      raw[t][0] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb);
+      raw[t][1] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 512);
       if (kW4) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          bf[t][2 * j] = w4_unpack(raw[t][0][j], mask, magic);
-          bf[t][2 * j + 1] = w4_unpack(raw[t][1][j], mask, magic);
-        }
-        // ninth step: -(128 + z) against the three pieces of the group sum (lanes kh = 0 only)
-        const uint32_t z = (mraw[t] >> 19) & 0xFu;  // fp16(128 + z): z sits in mantissa bits 3..6
-        const uint32_t nz = kh == 0 ? (0xC300u | z) : 0u;
-        bf[t][8] = u32x4_t{nz | (nz << 16), nz, 0u, 0u};
-        sc[t] = f16_bits_to_f32(mraw[t] & 0xFFFFu);
+        mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
       } else {
-        // W8 tile tau (64 k), load h (kc = kh + 2h): dwords (2j, 2j+1) are k-step 4 tau + 2j + h
-#pragma unroll
-        for (int tau = 0; tau < 2; ++tau)
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const u32x2_t lo = w8_to_bf16(raw[t][2 * tau + h][2 * j]);
-              const u32x2_t hi = w8_to_bf16(raw[t][2 * tau + h][2 * j + 1]);
-              bf[t][4 * tau + 2 * j + h] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
-            }
+        raw[t][2] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 1024);
+        raw[t][3] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 1536);
       }
     }
-    if (has_next) load_b(kb + 1);
 
+    // ---- B fragments.  They are unpacked one k-step ahead of their first use, inside the
+    // wave's first 32-row block, so the unpacking (VALU) runs under the MFMAs.
+    u32x4_t bf[2][kSteps];
+    float sc[2];
+    auto unpack_step = [&](int s) {
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      if (kW4) {
-        f32x16_t part[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) part[t][r] = 0.f;
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-          const uint32_t off = (s < 8 ? a_off[s < 8 ? s : 0] + i * 32 * 256 : g_off + i * 32 * 16);
-          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(lds + off);
-#pragma unroll
-          for (int t = 0; t < 2; ++t) part[t] = mfma32(a, bf[t][s], part[t]);
-        }
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[i][t][r] += sc[t] * part[t][r];
-      } else {
-#pragma unroll
-        for (int s = 0; s < kSteps; ++s) {
-          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(lds + a_off[s] + i * 32 * 256);
-#pragma unroll
-          for (int t = 0; t < 2; ++t) acc[i][t] = mfma32(a, bf[t][s], acc[i][t]);
+      for (int t = 0; t < 2; ++t) {
+        if (kW4) {
+          if (s < 8) {
+            bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], mask, magic);
+          } else {
+            // ninth step: -(128 + z) against the three pieces of the group sum (lanes kh = 0 only)
+            const uint32_t z = (mraw[t] >> 19) & 0xFu;  // fp16(128 + z): z sits in mantissa bits 3..6
+            const uint32_t nz = kh == 0 ? (0xC300u | z) : 0u;
+            bf[t][8] = u32x4_t{nz | (nz << 16), nz, 0u, 0u};
+            sc[t] = f16_bits_to_f32(mraw[t] & 0xFFFFu);
+          }
+        } else {
+          // W8 tile tau (64 k), piece h (kc = kh + 2h): dwords (2j, 2j+1) are k-step 4 tau + 2j + h
+          const int tau = s >> 2, j = (s >> 1) & 1, h = s & 1;
+          const u32x2_t lo = w8_to_bf16(raw[t][2 * tau + h][2 * j]);
+          const u32x2_t hi = w8_to_bf16(raw[t][2 * tau + h][2 * j + 1]);
+          bf[t][s] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
         }
       }
-    }
-    // flip to the other tile / side buffer
+    };
+
+    // ---- MFMA loop, software-pipelined by hand: the A fragment of position p + kAhead is
+    // requested before the two MFMAs of position p are issued (position = 32-row block x
+    // k-step), and the order of LDS reads and MFMAs is pinned; VALU work may move freely.
+    constexpr int kPos = MT * kSteps;
+    constexpr int kAhead = 4;
+    auto a_addr = [&](int p) -> const u32x4_t* {
+      const int i = p / kSteps, s = p % kSteps;
+      const uint32_t off = s < 8 ? a_off[s & 3] + (s >> 2) * 128 + i * 32 * 256 : g_off + i * 32 * 16;
+      return reinterpret_cast<const u32x4_t*>(lds + off);
+    };
+    u32x4_t afr[kAhead + 1];
 #pragma unroll
-    for (int s = 0; s < 8; ++s) a_off[s] ^= (uint32_t)kG2TileBytes;
+    for (int p = 0; p < kAhead; ++p) afr[p] = *a_addr(p);
+    unpack_step(0);
+    f32x16_t part[2];
+#pragma unroll
+    for (int p = 0; p < kPos; ++p) {
+      const int i = p / kSteps, s = p % kSteps;
+      if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = *a_addr(p + kAhead);
+      if (i == 0 && s + 1 < kSteps) unpack_step(s + 1);
+      if (kW4) {
+        if (s == 0) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part[t][r] = 0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) part[t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], part[t]);
+        if (s == kSteps - 1) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][t][r] += sc[t] * part[t][r];
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) acc[i][t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], acc[i][t]);
+      }
+      __builtin_amdgcn_sched_barrier(0x2 | 0x4);  // VALU and SALU may cross
+    }
+    // flip every read offset to the other buffer
+#pragma unroll
+    for (int v = 0; v < 4; ++v) a_off[v] ^= (uint32_t)kG2TileBytes;
     g_off ^= (uint32_t)kG2SideBytes;
-    // the next tile must have landed and every wave must be done with this one
+    b_off ^= (uint32_t)kG2WStride;
+    m_off ^= (uint32_t)kG2MetaStride;
+    // the next block's tiles must have landed and every wave must be done with this one
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
