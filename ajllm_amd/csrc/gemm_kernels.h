@@ -233,8 +233,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void dequant_gemm_kerne
 //  * Weights: every wave loads the private tiles of its own 64 columns straight
 //    into registers and unpacks them once per k-block into B fragments that hold
 //    exact small integers (128+q, or q for int8).
-//  * A wave walks its four 32-row blocks in turn: A fragments are read from LDS
-//    just in time and each feeds the two 32-column blocks of the wave.
+//  * A wave walks its 32-row blocks in turn: A fragments are requested from LDS
+//    four MFMA pairs ahead and each feeds the two 32-column blocks of the wave; the
+//    loads of the next k-block are issued one at a time between the MFMAs.  The
+//    loop body is one basic block (no branch between MFMAs).
 //  * The last row tile is shifted up to end at row M (M >= 256), so no row is
 //    clamped or masked; rows it shares with its neighbour are computed twice
 //    with identical results.
@@ -325,30 +327,30 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
 
   // ---- global -> LDS, one k-block ahead, no registers in between.
   // Activations: wave w fills kLoadRows rows with wave-wide loads of 4 rows each.  Chunk c
-  // of row r lives in slot (c & 8) | ((c & 7) ^ (r & 7)) of its row; lane (row_in, slot) of
-  // load q therefore fetches chunk (slot & 8) | ((slot & 7) ^ ((4q + row_in) & 7)), which
-  // depends on q only through q & 1.
+  // of row r lives in slot c ^ (r & 15) of its row (the LDS serves 16 lanes of a 128-bit
+  // read per clock from 64 banks: 16 consecutive rows must fall in 16 different slots);
+  // lane (row_in, slot) of load q therefore fetches chunk slot ^ ((4q + row_in) & 15),
+  // which depends on q only through q & 3.
   const int row_in = lane >> 4, slot = lane & 15;
-  uint32_t a_voff[2];
+  uint32_t a_voff[4];
 #pragma unroll
-  for (int v = 0; v < 2; ++v)
-    a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)(((slot & 8) | ((slot & 7) ^ ((4 * v + row_in) & 7))) * 16);
+  for (int v = 0; v < 4; ++v)
+    a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)((slot ^ (4 * v + row_in)) * 16);
   const char* a_base = reinterpret_cast<const char*>(x) + (size_t)(m0 + kLoadRows * wave) * K * 2;
   const int nt16_0 = n0 / kTileN;
-  auto load_tiles = [&](int kb, int buf) {
-    char* dst = lds + buf * kG2TileBytes + wave * (kLoadRows * 256);
-    const char* src = a_base + (size_t)kb * 256;
-#pragma unroll
-    for (int q = 0; q < kLoadRows / 4; ++q)
-      __builtin_amdgcn_global_load_lds((global_void_t*)(src + (size_t)q * 4 * K * 2 + a_voff[q & 1]),
-                                       (lds_void_t*)(dst + q * 1024), 16, 0, 0);
-    if (kW4 && wave < 4)
-      __builtin_amdgcn_global_load_lds((global_void_t*)(gs3 + (size_t)kb * M + m0 + 64 * wave + lane),
-                                       (lds_void_t*)(lds + kG2SideBase + buf * kG2SideBytes + wave * 1024), 16, 0, 0);
-    // weights: a private tile is 1 KiB contiguous, one wave-wide load each
-#pragma unroll
-    for (int u = 0; u < kBTiles / kWaves; ++u) {
-      const int T = wave * (kBTiles / kWaves) + u;
+  // The loads of one k-block are numbered 0 .. kLoads - 1 so that the main loop can issue
+  // them one at a time between its MFMAs.
+  constexpr int kALoads = kLoadRows / 4;
+  constexpr int kBLoads = kBTiles / kWaves;
+  constexpr int kLoads = kALoads + kBLoads + (kW4 ? 2 : 0);
+  auto issue_load = [&](int j, int kb, int buf) {
+    if (j < kALoads) {
+      const char* src = a_base + (size_t)kb * 256 + (size_t)j * 4 * K * 2 + a_voff[j & 3];
+      char* dst = lds + buf * kG2TileBytes + wave * (kLoadRows * 256) + j * 1024;
+      __builtin_amdgcn_global_load_lds((global_void_t*)src, (lds_void_t*)dst, 16, 0, 0);
+    } else if (j < kALoads + kBLoads) {
+      // weights: a private tile is 1 KiB contiguous, one wave-wide load each
+      const int T = wave * kBLoads + (j - kALoads);
       const u32x4_t* tile;
       if (kW4)
         tile = wq + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 64;
@@ -356,12 +358,19 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
         tile = wq + ((size_t)min(nt16_0 + (T >> 1), ntiles16 - 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
       __builtin_amdgcn_global_load_lds((global_void_t*)(tile + lane),
                                        (lds_void_t*)(lds + kWBase + buf * kG2WStride + T * 1024), 16, 0, 0);
-    }
-    if (kW4 && wave < 2) {  // meta words of 4 tiles per load
-      const int T = wave * 4 + (lane >> 4);
+    } else if (j == kALoads + kBLoads) {
+      // group-sum pieces of 64 rows; with eight waves the upper four repeat the lower four
+      // (same bytes to the same place) rather than branch
+      const int e = wave & 3;
+      __builtin_amdgcn_global_load_lds((global_void_t*)(gs3 + (size_t)kb * M + m0 + 64 * e + lane),
+                                       (lds_void_t*)(lds + kG2SideBase + buf * kG2SideBytes + e * 1024), 16, 0, 0);
+    } else {
+      // meta words, 4 tiles per load; odd and even waves take one half each
+      const int e = wave & 1;
+      const int T = e * 4 + (lane >> 4);
       __builtin_amdgcn_global_load_lds(
           (global_void_t*)(meta + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 16 + (lane & 15)),
-          (lds_void_t*)(lds + kG2MetaBase + buf * kG2MetaStride + wave * 256), 4, 0, 0);
+          (lds_void_t*)(lds + kG2MetaBase + buf * kG2MetaStride + e * 256), 4, 0, 0);
     }
   };
 
@@ -374,11 +383,11 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
 
   // ---- LDS read offsets.  A fragment of k-step s, row r = kWaveRows wm + 32 i + col: chunk
-  // 2s + kh sits at byte (s >> 2) * 128 + (((s & 3) ^ (col >> 1 & 3)) << 5) + ((kh ^ (col & 1)) << 4).
-  uint32_t a_off[4];
+  // 2s + kh sits in slot (2s + kh) ^ (col & 15) = ((s ^ (col >> 1 & 7)) << 1) | (kh ^ (col & 1)).
+  uint32_t a_off[8];
 #pragma unroll
-  for (int v = 0; v < 4; ++v)
-    a_off[v] = (uint32_t)((wm * kWaveRows + col) * 256 + (((v ^ ((col >> 1) & 3)) << 5) | ((kh ^ (col & 1)) << 4)));
+  for (int v = 0; v < 8; ++v)
+    a_off[v] = (uint32_t)((wm * kWaveRows + col) * 256 + (((v ^ ((col >> 1) & 7)) << 5) | ((kh ^ (col & 1)) << 4)));
   uint32_t g_off = (uint32_t)(kG2SideBase + (wm * kWaveRows + col) * 16);
   // weights: lane (col, kh) of 32-column block t reads, from the 16-row private tile that
   // holds its column, the 16 bytes of tile lanes (kc = kh) and (kc = kh + 2): dword j of the
@@ -387,7 +396,8 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   uint32_t b_off = (uint32_t)(kWBase + (kW4 ? c16 : 2 * c16) * 1024 + (kh * 16 + nl) * 16);
   uint32_t m_off = (uint32_t)(kG2MetaBase + (c16 * 16 + nl) * 4);
 
-  load_tiles(0, 0);
+#pragma unroll
+  for (int j = 0; j < kLoads; ++j) issue_load(j, 0, 0);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
@@ -396,22 +406,27 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   asm volatile("" : "+v"(magic));
 
   for (int kb = 0; kb < G; ++kb) {
-    if (kb + 1 < G) load_tiles(kb + 1, (kb + 1) & 1);
+    // Loads are issued unconditionally (the last block is simply fetched again): a branch
+    // between the MFMAs would cut the loop body into separately scheduled pieces.
+    const int kb_next = min(kb + 1, G - 1);
 
-    // ---- this block's packed weights, LDS -> registers
+    // ---- this block's packed weights, LDS -> registers (W8: the second 64-k tile is
+    // fetched a few steps later, shortly before it is unpacked)
     u32x4_t raw[2][kW4 ? 2 : 4];
     uint32_t mraw[2];
+    auto read_raw = [&](int first, int count) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      const int tb = t * (kW4 ? 2048 : 4096);
-      raw[t][0] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb);
-      raw[t][1] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 512);
-      if (kW4) {
-        mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
-      } else {
-        raw[t][2] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 1024);
-        raw[t][3] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + 1536);
+      for (int t = 0; t < 2; ++t) {
+        const int tb = t * (kW4 ? 2048 : 4096);
+#pragma unroll
+        for (int q = first; q < first + count; ++q)
+          raw[t][q] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + q * 512);
       }
+    };
+    read_raw(0, 2);
+    if (kW4) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
     }
 
     // ---- B fragments.  They are unpacked one k-step ahead of their first use, inside the
@@ -433,6 +448,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
           }
         } else {
           // W8 tile tau (64 k), piece h (kc = kh + 2h): dwords (2j, 2j+1) are k-step 4 tau + 2j + h
+          if (s == 2 && t == 0) read_raw(2, 2);
           const int tau = s >> 2, j = (s >> 1) & 1, h = s & 1;
           const u32x2_t lo = w8_to_bf16(raw[t][2 * tau + h][2 * j]);
           const u32x2_t hi = w8_to_bf16(raw[t][2 * tau + h][2 * j + 1]);
@@ -448,7 +464,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     constexpr int kAhead = 4;
     auto a_addr = [&](int p) -> const u32x4_t* {
       const int i = p / kSteps, s = p % kSteps;
-      const uint32_t off = s < 8 ? a_off[s & 3] + (s >> 2) * 128 + i * 32 * 256 : g_off + i * 32 * 16;
+      const uint32_t off = s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16;
       return reinterpret_cast<const u32x4_t*>(lds + off);
     };
     u32x4_t afr[kAhead + 1];
@@ -461,6 +477,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
       const int i = p / kSteps, s = p % kSteps;
       if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = *a_addr(p + kAhead);
       if (i == 0 && s + 1 < kSteps) unpack_step(s + 1);
+      if (p < kLoads) issue_load(p, kb_next, (kb + 1) & 1);  // one load per position
       if (kW4) {
         if (s == 0) {
 #pragma unroll
@@ -484,7 +501,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     }
     // flip every read offset to the other buffer
 #pragma unroll
-    for (int v = 0; v < 4; ++v) a_off[v] ^= (uint32_t)kG2TileBytes;
+    for (int v = 0; v < 8; ++v) a_off[v] ^= (uint32_t)kG2TileBytes;
     g_off ^= (uint32_t)kG2SideBytes;
     b_off ^= (uint32_t)kG2WStride;
     m_off ^= (uint32_t)kG2MetaStride;
