@@ -1,0 +1,99 @@
+"""End-to-end greedy decoding of the 12-layer benchmark model with every linear quantized.
+
+The model is the reference architecture (src/ajllm/modeling/transformer.py:13-126) at the size the
+benchmark names: 12 layers, d_model 2048, 16 heads (head_dim 128), SwiGLU d_ff 5632, vocab 32000,
+RMSNorm, RoPE, untied lm_head, reference init under a fixed seed; all linears W4A16 group-128.
+Prompts are seeded random token ids ``[B, 512]``; 256 tokens are decoded greedily with a KV cache.
+Only the linears run in this library's kernels; norms, RoPE and attention are eager PyTorch, so the
+tokens/s reported here is bounded by launch overhead, not by the quantized linears (the share of
+the step spent in them is reported beside it).
+"""
+
+from __future__ import annotations
+
+import time
+
+import torch
+
+from . import modeling
+from .quant import QuantLinear, quantize_model_
+
+CONFIG = dict(vocab_size=32000, context_length=1024, d_model=2048, num_layers=12, num_heads=16, d_ff=5632)
+PROMPT_LEN = 512
+NEW_TOKENS = 256
+
+
+def build_quantized_model(device, scheme: str = "w4a16_g128", seed: int = 1234, config: dict | None = None):
+    torch.manual_seed(seed)
+    with torch.device(device):
+        model = modeling.TransformerLM(**(config or CONFIG)).eval()
+    quantize_model_(model, scheme)
+    torch.cuda.empty_cache()
+    return model
+
+
+def _linear_seconds_per_step(model, batch: int, device) -> float:
+    """Time of the quantized linears of one decode step on their own: every QuantLinear once, with
+    ``[batch, in_features]`` inputs, replayed from a HIP graph."""
+    layers = [m for m in model.modules() if isinstance(m, QuantLinear)]
+    inputs = [torch.randn((batch, m.in_features), device=device).to(torch.bfloat16) for m in layers]
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream), torch.no_grad():
+        for m, x in zip(layers, inputs):
+            m(x)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for m, x in zip(layers, inputs):
+                m(x)
+        graph.replay()
+        stream.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(20):
+            graph.replay()
+        stop.record(stream)
+        stop.synchronize()
+    return start.elapsed_time(stop) / 1e3 / 20
+
+
+@torch.no_grad()
+def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") -> list[dict]:
+    model = build_quantized_model(device, scheme)
+    packed = sum(m.wq.numel() * 4 + m.meta.numel() * m.meta.element_size()
+                 for m in model.modules() if isinstance(m, QuantLinear))
+    results = []
+    for batch in batches:
+        g = torch.Generator().manual_seed(100 + batch)
+        prompt = torch.randint(0, CONFIG["vocab_size"], (batch, PROMPT_LEN), generator=g).to(device)
+        modeling.greedy_decode(model, prompt[:, :32], 4)  # warm-up: library load, allocator
+        torch.cuda.synchronize()
+        cache = model.new_cache(batch, PROMPT_LEN + NEW_TOKENS)
+        t0 = time.perf_counter()
+        logits = model(prompt, cache, last_token_only=True)[:, -1, :]
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        tokens = [torch.argmax(logits, dim=-1, keepdim=True)]
+        t0 = time.perf_counter()
+        for _ in range(NEW_TOKENS - 1):
+            logits = model(tokens[-1], cache, last_token_only=True)[:, -1, :]
+            tokens.append(torch.argmax(logits, dim=-1, keepdim=True))
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t0
+        t_linear = _linear_seconds_per_step(model, batch, device)
+        step = t_decode / (NEW_TOKENS - 1)
+        r = {
+            "scheme": scheme, "batch": batch, "prompt": PROMPT_LEN, "new_tokens": NEW_TOKENS,
+            "prefill_s": t_prefill, "prefill_tok/s": batch * PROMPT_LEN / t_prefill,
+            "decode_s": t_decode, "decode_tok/s": batch * (NEW_TOKENS - 1) / t_decode,
+            "ms_per_step": step * 1e3,
+            "quant_linear_ms_per_step": t_linear * 1e3,
+            "quant_linear_share_of_step": t_linear / step,
+            "quant_linear_GB/s": packed / t_linear / 1e9,
+            "packed_weight_bytes": packed,
+            "loop": "eager PyTorch around the HIP linears (no graph capture of the decode step)",
+        }
+        log("decode", r)
+        results.append(r)
+        del cache
+    return results
