@@ -30,7 +30,7 @@ import torch
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor peak
-GEMV_W4_4096_M1_HBM_BYTES = 9.49e6  # measured: 4423 KiB x 2.093 fetched + 8 KiB x 1.047 written per launch
+GEMV_W4_4096_M1_HBM_BYTES = 9.03e6  # measured: 4407.6 KiB x 1.9993 fetched + 8 KiB x 1.0 written per launch
 
 
 def log(*args) -> None:
