@@ -275,7 +275,8 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   if (M >= kGemm256MinM) {
     if ((long long)M * K * 2 >= (1LL << 32))
       return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
-    hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
+    const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
+    hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
                        K, reinterpret_cast<u32x4_t*>(workspace));
     if (int s = launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_dtype == AJQ_OUT_F32,
                                      (hipStream_t)stream))

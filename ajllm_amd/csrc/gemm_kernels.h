@@ -244,30 +244,41 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void dequant_gemm_kerne
 
 // gs3[g][m] = 16 bytes: bf16 pieces h, m, l with h + m + l == the sum of the 128
 // activations of group g in row m to fp32 precision, then five zeros.
+// A 16-lane team sums four consecutive groups of one row (four 128-bit loads in
+// flight per lane); K / 128 must be a multiple of 4 or the tail teams clamp.
 __global__ __launch_bounds__(256) void group_sum3_kernel(const uint16_t* __restrict__ x, int M, int K,
                                                          u32x4_t* __restrict__ gs3) {
   const int G = K >> 7;
+  const int G4 = (G + 3) >> 2;
   const long long team = (long long)blockIdx.x * 16 + (threadIdx.x >> 4);
-  if (team >= (long long)M * G) return;
+  if (team >= (long long)M * G4) return;
   const int sub = threadIdx.x & 15;
-  const int m = (int)(team / G), g = (int)(team % G);
-  const u32x4_t v = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g * kGroup + sub * 8);
-  float s = 0.f;
+  const int m = (int)(team / G4), g0 = (int)(team % G4) * 4;
+  u32x4_t v[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    s += __uint_as_float(v[i] << 16);
-    s += __uint_as_float(v[i] & 0xFFFF0000u);
+  for (int u = 0; u < 4; ++u) {
+    const int g = min(g0 + u, G - 1);
+    v[u] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g * kGroup + sub * 8);
   }
 #pragma unroll
-  for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
-  if (sub == 0) {
-    // truncation keeps every remainder exactly representable
-    const uint32_t hb = __float_as_uint(s) & 0xFFFF0000u;
-    const float r1 = s - __uint_as_float(hb);
-    const uint32_t mb = __float_as_uint(r1) & 0xFFFF0000u;
-    const float r2 = r1 - __uint_as_float(mb);
-    const uint32_t lb = (uint32_t)f32_to_bf16_rne(r2);
-    gs3[(size_t)g * M + m] = u32x4_t{(hb >> 16) | mb, lb, 0u, 0u};
+  for (int u = 0; u < 4; ++u) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      s += __uint_as_float(v[u][i] << 16);
+      s += __uint_as_float(v[u][i] & 0xFFFF0000u);
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    if (sub == u && g0 + u < G) {
+      // truncation keeps every remainder exactly representable
+      const uint32_t hb = __float_as_uint(s) & 0xFFFF0000u;
+      const float r1 = s - __uint_as_float(hb);
+      const uint32_t mb = __float_as_uint(r1) & 0xFFFF0000u;
+      const float r2 = r1 - __uint_as_float(mb);
+      const uint32_t lb = (uint32_t)f32_to_bf16_rne(r2);
+      gs3[(size_t)(g0 + u) * M + m] = u32x4_t{(hb >> 16) | mb, lb, 0u, 0u};
+    }
   }
 }
 

@@ -150,7 +150,13 @@ class RotaryPositionalEmbedding(nn.Module):
 
 
 class KVCache:
-    """Per-layer key/value store for incremental decoding: ``[layers][B, kv_heads, max_len, head_dim]``."""
+    """Per-layer key/value store for incremental decoding: ``[layers][B, kv_heads, max_len, head_dim]``.
+
+    Two modes.  Dynamic (default): ``length`` is a Python int, a call appends ``seq`` positions and
+    attends over the first ``length + seq``.  Static (``static = True``, one token per call): the
+    write position is the device tensor ``position``, the new key/value row is scattered there and
+    attention runs over all ``max_len`` rows under a mask, so every shape is fixed and the step can
+    be recorded into a HIP graph; the caller advances ``position``."""
 
     def __init__(self, num_layers: int, batch: int, kv_heads: int, max_len: int, head_dim: int,
                  device, dtype) -> None:
@@ -158,6 +164,9 @@ class KVCache:
         self.values = [torch.zeros_like(k) for k in self.keys]
         self.length = 0
         self.max_len = max_len
+        self.static = False
+        self.position = torch.zeros(1, dtype=torch.long, device=device)
+        self.slots = torch.arange(max_len, device=device)
 
 
 class MultiHeadSelfAttention(nn.Module):
@@ -193,6 +202,20 @@ class MultiHeadSelfAttention(nn.Module):
         if self.rope is not None:
             q = self.rope(q, positions[:, None, :].expand(batch, self.num_heads, seq))
             k = self.rope(k, positions[:, None, :].expand(batch, self.num_kv_heads, seq))
+        if cache is not None and cache.static:
+            # fixed-shape step: scatter the new row at the device-side position, attend over the
+            # whole cache with the rows beyond that position masked out
+            cache.keys[layer_index].index_copy_(2, cache.position, k)
+            cache.values[layer_index].index_copy_(2, cache.position, v)
+            k, v = cache.keys[layer_index], cache.values[layer_index]
+            if self.num_kv_heads != self.num_heads:
+                rep = self.num_heads // self.num_kv_heads
+                k = k.repeat_interleave(rep, dim=1)
+                v = v.repeat_interleave(rep, dim=1)
+            mask = (cache.slots <= cache.position).view(1, cache.max_len)
+            attended = scaled_dot_product_attention(q, k, v, mask)
+            joined = attended.transpose(1, 2).contiguous().view(batch, seq, self.d_model)
+            return self.output_proj(joined)
         start = 0
         if cache is not None:
             start = cache.length
@@ -273,6 +296,19 @@ class TransformerLM(nn.Module):
     def forward(self, token_ids: torch.Tensor, cache: KVCache | None = None,
                 last_token_only: bool = False) -> torch.Tensor:
         batch, seq = token_ids.shape
+        if cache is not None and cache.static:
+            if seq != 1:
+                raise ValueError("a static KV cache takes one token per call")
+            positions = cache.position.view(1, 1).expand(batch, 1)
+            hidden = self.token_embeddings(token_ids)
+            if self.position_embeddings is not None:
+                hidden = hidden + self.position_embeddings(positions)
+            for index, layer in enumerate(self.layers):
+                hidden = layer(hidden, positions, cache, index)
+            hidden = self.final_norm(hidden)
+            if self.tie_embeddings:
+                return hidden @ self.token_embeddings.weight.transpose(0, 1)
+            return self.lm_head(hidden)
         start = cache.length if cache is not None else 0
         if start + seq > self.context_length:
             raise ValueError(f"Input length {start + seq} exceeds context length {self.context_length}")

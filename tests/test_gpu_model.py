@@ -7,7 +7,7 @@ import copy
 import pytest
 import torch
 
-from ajllm_amd import QuantLinear, modeling, quantize_model_
+from ajllm_amd import QuantLinear, decoding, modeling, quantize_model_
 from oracle import qspec
 from tests.helpers import MAX_ABS_TOL, REL_FRO_TOL, compare_greedy, errors, make_activations, make_weight
 
@@ -111,3 +111,32 @@ def test_greedy_tokens_match_the_oracle_model(cuda, scheme, batch):
     disagree = (pred_got != pred_ref)
     assert (margins[disagree] < noise).all(), margins[disagree]
     assert int(disagree.sum()) <= max(1, disagree.numel() // 10)
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_graph_replayed_decoding_matches_eager_decoding(cuda, batch):
+    """The decode step recorded into a HIP graph and replayed per token (with the program's own
+    eager work in between: prefill, clones, a second generate call) yields the tokens of the eager
+    loop; compared step by step, a difference is accepted only below the eager run's own margin noise."""
+    torch.manual_seed(3)
+    model = modeling.TransformerLM(vocab_size=512, context_length=96, d_model=256, num_layers=3, num_heads=2,
+                                   d_ff=640).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w4a16_g128")
+    prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(8)).to(cuda)
+    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True)
+    dec = decoding.GraphDecoder(fast, batch, 60)
+    dec.prefill(prompt)
+    first = dec.generate(10)          # eager step + capture + replays
+    torch.cuda.synchronize()
+    _ = fast(prompt)                  # unrelated eager work between replays
+    got = dec.generate(40)            # replays only
+    assert torch.equal(got[:, :10], first)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 20, noise=1e-3)
+    assert not report["unexplained"], report
+    # a second prompt through the same decoder (same graph, new state)
+    prompt2 = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(9)).to(cuda)
+    eager2, margins2 = modeling.greedy_decode(fast, prompt2, 12, return_margins=True)
+    dec.prefill(prompt2)
+    got2 = dec.generate(12)
+    report2 = compare_greedy(torch.cat((prompt2, got2), 1).cpu(), eager2.cpu(), margins2.cpu(), 20, noise=1e-3)
+    assert not report2["unexplained"], report2

@@ -140,3 +140,24 @@ def test_build_model_reads_reference_style_config():
     model = M.build_model(cfg, vocab_size=50)
     assert model.d_ff == 128  # ceil(8*48/3 = 128) to a multiple of 64
     assert M.build_model({**cfg, "feed_forward": {"type": "silu"}}, 50).d_ff == 192
+
+
+def test_static_cache_steps_equal_dynamic_decoding():
+    """One-token steps against a static KV cache (fixed shapes, device-side position) choose the
+    same tokens as the dynamic cache."""
+    torch.manual_seed(11)
+    model = _model(num_layers=2)
+    prompt = torch.randint(0, model.vocab_size, (2, 6))
+    want = M.greedy_decode(model, prompt, 7)
+    cache = model.new_cache(2, 13)
+    logits = model(prompt, cache, last_token_only=True)[:, -1]
+    cache.static = True
+    cache.position.fill_(6)
+    tokens = [logits.argmax(-1, keepdim=True)]
+    for _ in range(6):
+        logits = model(tokens[-1], cache)[:, -1]
+        cache.position.add_(1)
+        tokens.append(logits.argmax(-1, keepdim=True))
+    assert torch.equal(torch.cat([prompt] + tokens, dim=1), want)
+    with pytest.raises(ValueError):
+        model(prompt, cache)  # a static cache takes one token per call
