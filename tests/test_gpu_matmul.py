@@ -96,6 +96,18 @@ def test_gemv_ragged_m_and_small_shapes(cuda, scheme, m):
     _check(scheme, "gemv", m, 2048, 5632, seed=14, cuda=cuda)
 
 
+@pytest.mark.parametrize("m", [5, 8, 11, 16])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemv_wide_matrix_with_ragged_last_workgroup(cuda, scheme, m):
+    """N / 16 = 517 row tiles at K = 4096: several row tiles per workgroup, the last workgroup short."""
+    _check(scheme, "gemv", m, 16 * 517, 4096, seed=15, cuda=cuda)
+    w_hat, wq, meta = _quantized(scheme, 16 * 517, 4096, 15, cuda)
+    x = make_activations(m, 4096, 6).to(cuda)
+    first = _run(scheme, x, wq, meta, torch.float32, "gemv")
+    for _ in range(5):
+        assert torch.equal(_run(scheme, x, wq, meta, torch.float32, "gemv"), first)
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemv_is_deterministic(cuda, scheme):
     w_hat, wq, meta = _quantized(scheme, 4096, 4096, 11 if scheme == "w4" else 12, cuda)
