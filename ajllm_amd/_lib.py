@@ -8,7 +8,7 @@ CPU or PyTorch fallback behind any of these calls.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
 from pathlib import Path
 
 LIBRARY_PATH = Path(__file__).resolve().parent / "libajq.so"
@@ -39,6 +39,19 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "ajq_w8a16_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ajq_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p]),
+    "ajq_rope_cache": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+         c_void_p],
+    ),
+    "ajq_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "ajq_attn_decode": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t,
+         c_void_p],
+    ),
+    "ajq_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
 }
 
 _lib: ctypes.CDLL | None = None

@@ -7,6 +7,7 @@
 #include "quantize_kernels.h"
 #include "gemv_kernels.h"
 #include "gemm_kernels.h"
+#include "decode_kernels.h"
 
 using namespace ajq;
 
@@ -252,9 +253,20 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
     if (M <= 8) return launch_gemv_mt<8, 4, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, T, stream);
     return launch_gemv_mt<8, 4, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, T, stream);
   }
+  if (K == 8 * 2 * kGroup) {  // K = 2048: one batch of two groups per wave, straight-line kernel
+    if (M <= 1) return launch_gemv_cfg<8, 2, 1, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 2) return launch_gemv_cfg<8, 2, 2, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 4) return launch_gemv_cfg<8, 2, 4, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 8) return launch_gemv_cfg<8, 2, 8, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    return launch_gemv_cfg<8, 2, 16, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  }
   if (M <= 1) return launch_gemv_rows<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 2) return launch_gemv_rows<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 4) return launch_gemv_rows<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (K == 8 * 4 * kGroup) {  // one batch of four groups per wave covers K: straight-line kernel
+    if (M <= 8) return launch_gemv_cfg<8, 4, 8, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    return launch_gemv_cfg<8, 4, 16, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  }
   if (M <= 8) return launch_gemv_rows<8, 2, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   return launch_gemv_rows<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
@@ -342,6 +354,77 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                                              out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
   if (s) return s;
   return check_launch("ajq_w8a16_gemm");
+}
+
+}  // extern "C"
+
+// --------------------------------------------------- decode-step operators -----
+namespace {
+int attn_splits(int B, int H) {
+  int s = 256 / (B * H);
+  return s < 1 ? 1 : (s > 16 ? 16 : s);
+}
+}  // namespace
+
+extern "C" {
+
+int ajq_add_rmsnorm(float* hidden, const float* delta, const float* gain, float eps, uint16_t* out, int B, int D,
+                    void* stream) {
+  if (!hidden || !gain || !out) return fail(AJQ_ERR_NULL, "ajq_add_rmsnorm: null pointer argument");
+  if (B < 1 || D < 4 || D % 4 != 0)
+    return fail(AJQ_ERR_SHAPE, "ajq_add_rmsnorm: need B >= 1 and D a positive multiple of 4 (got %d, %d)", B, D);
+  if (!aligned16(hidden) || !aligned16(gain) || (delta && !aligned16(delta)) || (reinterpret_cast<uintptr_t>(out) & 7u))
+    return fail(AJQ_ERR_ALIGN, "ajq_add_rmsnorm: hidden, delta, gain must be 16-byte and out 8-byte aligned");
+  hipLaunchKernelGGL(add_rmsnorm_kernel, dim3(B), dim3(256), 0, (hipStream_t)stream, hidden, delta, gain, eps, out, D);
+  return check_launch("ajq_add_rmsnorm");
+}
+
+int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, float* q_out,
+                   float* kcache, float* vcache, int B, int H, int Hkv, int head_dim, int max_len, void* stream) {
+  if (!qkv || !cosine || !sine || !pos || !q_out || !kcache || !vcache)
+    return fail(AJQ_ERR_NULL, "ajq_rope_cache: null pointer argument");
+  if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || head_dim < 2 || head_dim % 2 != 0 || max_len < 1)
+    return fail(AJQ_ERR_SHAPE, "ajq_rope_cache: unsupported shape (B=%d H=%d Hkv=%d head_dim=%d max_len=%d)", B, H, Hkv,
+                head_dim, max_len);
+  const long long pairs = (long long)B * (H + 2 * Hkv) * (head_dim / 2);
+  hipLaunchKernelGGL(rope_cache_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream, qkv,
+                     cosine, sine, reinterpret_cast<const long long*>(pos), q_out, kcache, vcache, B, H, Hkv, head_dim,
+                     max_len);
+  return check_launch("ajq_rope_cache");
+}
+
+size_t ajq_attn_decode_workspace_bytes(int B, int H) {
+  if (B < 1 || H < 1) return 0;
+  return (size_t)B * H * attn_splits(B, H) * 130 * sizeof(float);
+}
+
+int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos, int B, int H, int Hkv,
+                    int head_dim, int max_len, uint16_t* out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!q || !kcache || !vcache || !pos || !out) return fail(AJQ_ERR_NULL, "ajq_attn_decode: null pointer argument");
+  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (only 128 is built)", head_dim);
+  if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
+    return fail(AJQ_ERR_SHAPE, "ajq_attn_decode: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
+  const int S = attn_splits(B, H);
+  if (S > 1 && (!workspace || workspace_bytes < ajq_attn_decode_workspace_bytes(B, H)))
+    return fail(AJQ_ERR_WORKSPACE, "ajq_attn_decode: workspace of %zu bytes needed, %zu given",
+                ajq_attn_decode_workspace_bytes(B, H), workspace_bytes);
+  const float scale = 1.0f / sqrtf((float)head_dim);
+  hipLaunchKernelGGL(attn_decode_kernel, dim3(B * H, S), dim3(256), 0, (hipStream_t)stream, q, kcache, vcache,
+                     reinterpret_cast<const long long*>(pos), H, Hkv, max_len, scale,
+                     reinterpret_cast<float*>(workspace), out);
+  if (S > 1)
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, (hipStream_t)stream,
+                       reinterpret_cast<const float*>(workspace), S, out);
+  return check_launch("ajq_attn_decode");
+}
+
+int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream) {
+  if (!ab || !out) return fail(AJQ_ERR_NULL, "ajq_swiglu: null pointer argument");
+  if (B < 1 || F < 2 || F % 2 != 0) return fail(AJQ_ERR_SHAPE, "ajq_swiglu: need B >= 1 and even F (got %d, %d)", B, F);
+  const long long pairs = (long long)B * (F / 2);
+  hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream, ab, out, B,
+                     F);
+  return check_launch("ajq_swiglu");
 }
 
 }  // extern "C"

@@ -1,0 +1,189 @@
+// The small operators of one decode step between the quantized linears: residual add +
+// RMSNorm, rotary embedding + KV-cache write, single-query attention over the cache, and
+// the SwiGLU gate.  All arithmetic is fp32 (the residual stream and the KV cache are fp32);
+// outputs that feed a quantized linear are written as bf16, which is what the linear's
+// own input cast would produce.  The write position of the step is read from device
+// memory, so a recorded HIP graph can be replayed for every token.
+#pragma once
+#include "ajq_common.h"
+
+namespace ajq {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  return v;
+}
+
+// hidden[b, :] += delta[b, :] (when delta != nullptr; written back), then
+// out[b, :] = bf16( (hidden / sqrt(mean(hidden^2) + eps)) * gain ).
+// One 256-thread workgroup per row; D % 4 == 0.
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
+                                                          const float* __restrict__ gain, float eps,
+                                                          uint16_t* __restrict__ out, int D) {
+  const int b = blockIdx.x;
+  float4* h4 = reinterpret_cast<float4*>(hidden + (size_t)b * D);
+  const float4* d4 = delta ? reinterpret_cast<const float4*>(delta + (size_t)b * D) : nullptr;
+  const float4* g4 = reinterpret_cast<const float4*>(gain);
+  const int n4 = D >> 2;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n4; i += 256) {
+    float4 v = h4[i];
+    if (d4) {
+      const float4 d = d4[i];
+      v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+      h4[i] = v;
+    }
+    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  }
+  ss = wave_sum(ss);
+  __shared__ float part[4];
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  ss = (part[0] + part[1]) + (part[2] + part[3]);
+  const float rms = sqrtf(ss / (float)D + eps);
+  uint2* o2 = reinterpret_cast<uint2*>(out + (size_t)b * D);
+  for (int i = threadIdx.x; i < n4; i += 256) {
+    const float4 v = h4[i];  // own writes above: same thread, same addresses
+    const float4 g = g4[i];
+    const uint32_t lo = f32_to_bf16_rne((v.x / rms) * g.x) | ((uint32_t)f32_to_bf16_rne((v.y / rms) * g.y) << 16);
+    const uint32_t hi = f32_to_bf16_rne((v.z / rms) * g.z) | ((uint32_t)f32_to_bf16_rne((v.w / rms) * g.w) << 16);
+    o2[i] = uint2{lo, hi};
+  }
+}
+
+// qkv [B, (H + 2 Hkv) * hd] fp32 (q heads, then k heads, then v heads) -> rotated q
+// [B, H, hd]; rotated k and plain v are written into the caches [B, Hkv, max_len, hd] at
+// row *pos.  Interleaved pairs: (x[2i], x[2i+1]) -> (e c - o s, e s + o c) with the tables'
+// row *pos.  One thread per pair.
+__global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict__ qkv, const float* __restrict__ cosine,
+                                                         const float* __restrict__ sine, const long long* __restrict__ pos,
+                                                         float* __restrict__ q_out, float* __restrict__ kcache,
+                                                         float* __restrict__ vcache, int B, int H, int Hkv, int hd,
+                                                         int max_len) {
+  const int half = hd >> 1;
+  const int heads = H + 2 * Hkv;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)B * heads * half) return;
+  const int i = (int)(idx % half);
+  const int head = (int)((idx / half) % heads);
+  const int b = (int)(idx / ((long long)half * heads));
+  const long long p = *pos;
+  const float2 v = *reinterpret_cast<const float2*>(qkv + ((size_t)b * heads + head) * hd + 2 * i);
+  if (head >= H + Hkv) {  // value head: stored as it is
+    const int hv = head - H - Hkv;
+    *reinterpret_cast<float2*>(vcache + (((size_t)b * Hkv + hv) * max_len + p) * hd + 2 * i) = v;
+    return;
+  }
+  const float c = cosine[p * half + i], s = sine[p * half + i];
+  const float2 r = float2{v.x * c - v.y * s, v.x * s + v.y * c};
+  if (head < H)
+    *reinterpret_cast<float2*>(q_out + ((size_t)b * H + head) * hd + 2 * i) = r;
+  else
+    *reinterpret_cast<float2*>(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i) = r;
+}
+
+// Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * H, S): a
+// workgroup of 4 waves takes chunk s of the rows; a wave walks its share of the chunk one
+// row at a time (a lane holds 2 of the 128 dimensions: one row is one coalesced 512-byte
+// read), keeping a running maximum, denominator and weighted value sum.  The 4 waves are
+// merged through LDS.  With S == 1 the result is normalised and written as bf16
+// [B, H * 128]; otherwise (max, denominator, 128 sums) go to `partial` for the merge kernel.
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ kcache,
+                                                          const float* __restrict__ vcache,
+                                                          const long long* __restrict__ pos, int H, int Hkv, int max_len,
+                                                          float scale, float* __restrict__ partial,
+                                                          uint16_t* __restrict__ out) {
+  constexpr int hd = 128;
+  const int bh = blockIdx.x, S = gridDim.y, s = blockIdx.y;
+  const int b = bh / H, h = bh % H;
+  const int hk = h / (H / Hkv);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rows = (int)(*pos) + 1;
+  const int per = (rows + S - 1) / S;
+  const int t_begin = s * per, t_end = min(rows, t_begin + per);
+  const float2 qv = *reinterpret_cast<const float2*>(q + (size_t)bh * hd + 2 * lane);
+  const float* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * hd + 2 * lane;
+  const float* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * hd + 2 * lane;
+  float m = -INFINITY, l = 0.f;
+  float2 acc = float2{0.f, 0.f};
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const float2 kv = *reinterpret_cast<const float2*>(kbase + (size_t)t * hd);
+    const float2 vv = *reinterpret_cast<const float2*>(vbase + (size_t)t * hd);
+    const float sc = wave_sum(qv.x * kv.x + qv.y * kv.y) * scale;
+    const float m_new = fmaxf(m, sc);
+    const float corr = expf(m - m_new), w = expf(sc - m_new);
+    l = l * corr + w;
+    acc.x = acc.x * corr + w * vv.x;
+    acc.y = acc.y * corr + w * vv.y;
+    m = m_new;
+  }
+  __shared__ float sm[4], sl[4];
+  __shared__ float2 sacc[4][64];
+  if (lane == 0) { sm[wave] = m; sl[wave] = l; }
+  sacc[wave][lane] = acc;
+  __syncthreads();
+  if (wave != 0) return;
+  float M4 = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+  float L = 0.f;
+  float2 A = float2{0.f, 0.f};
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float c = sm[w] == -INFINITY ? 0.f : expf(sm[w] - M4);
+    L += sl[w] * c;
+    A.x += sacc[w][lane].x * c;
+    A.y += sacc[w][lane].y * c;
+  }
+  if (S == 1) {
+    const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
+    reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
+  } else {
+    float* dst = partial + ((size_t)bh * S + s) * (hd + 2);
+    if (lane == 0) { dst[0] = M4; dst[1] = L; }
+    *reinterpret_cast<float2*>(dst + 2 + 2 * lane) = A;
+  }
+}
+
+// merge of the S partial results of attn_decode_kernel: one wave per (b, h)
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, int S,
+                                                        uint16_t* __restrict__ out) {
+  constexpr int hd = 128;
+  const int bh = blockIdx.x, lane = threadIdx.x;
+  const float* src = partial + (size_t)bh * S * (hd + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < S; ++s) M = fmaxf(M, src[s * (hd + 2)]);
+  float L = 0.f;
+  float2 A = float2{0.f, 0.f};
+  for (int s = 0; s < S; ++s) {
+    const float ms = src[s * (hd + 2)];
+    const float c = ms == -INFINITY ? 0.f : expf(ms - M);
+    L += src[s * (hd + 2) + 1] * c;
+    const float2 a = *reinterpret_cast<const float2*>(src + s * (hd + 2) + 2 + 2 * lane);
+    A.x += a.x * c;
+    A.y += a.y * c;
+  }
+  const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
+  reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
+}
+
+// ab [B, 2F] fp32 (gate projection, then up projection) -> out[b, f] = bf16( silu(a) * u ),
+// silu(a) = a * sigmoid(a).  F % 2 == 0; one thread per pair.
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ ab, uint16_t* __restrict__ out, int B,
+                                                     int F) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int half = F >> 1;
+  if (idx >= (long long)B * half) return;
+  const int b = (int)(idx / half), i = (int)(idx % half);
+  const float2 a = *reinterpret_cast<const float2*>(ab + (size_t)b * 2 * F + 2 * i);
+  const float2 u = *reinterpret_cast<const float2*>(ab + (size_t)b * 2 * F + F + 2 * i);
+  const float x0 = a.x * (1.0f / (1.0f + expf(-a.x))) * u.x;
+  const float x1 = a.y * (1.0f / (1.0f + expf(-a.y))) * u.y;
+  reinterpret_cast<uint32_t*>(out + (size_t)b * F)[i] = f32_to_bf16_rne(x0) | ((uint32_t)f32_to_bf16_rne(x1) << 16);
+}
+
+}  // namespace ajq

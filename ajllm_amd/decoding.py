@@ -12,7 +12,8 @@ from __future__ import annotations
 
 import torch
 
-from . import modeling
+from . import _lib, modeling
+from .quant import QuantLinear, w4a16_matmul, w8a16_matmul
 
 
 class GraphDecoder:
@@ -33,9 +34,13 @@ class GraphDecoder:
         self.graph: torch.cuda.CUDAGraph | None = None
         self.stream = torch.cuda.Stream(device=device)
 
+    def _logits(self) -> torch.Tensor:
+        """Logits ``[B, V]`` of the token in ``self.token`` at cache row ``cache.position``."""
+        return self.model(self.token, self.cache)[:, -1, :]
+
     @torch.no_grad()
     def _step(self) -> None:
-        logits = self.model(self.token, self.cache)[:, -1, :]
+        logits = self._logits()
         nxt = torch.argmax(logits, dim=-1, keepdim=True)
         self.out.index_copy_(1, self.step_index, nxt)
         self.token.copy_(nxt)
@@ -90,10 +95,121 @@ class GraphDecoder:
         return self.out[:, :new_tokens].clone()
 
 
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+class _FusedLinear:
+    """Several QuantLinears that share their input, as one matmul over their concatenated rows
+    (the private tiles are 16-row blocks, so concatenating along N is concatenating tensors)."""
+
+    def __init__(self, layers: list[QuantLinear]) -> None:
+        scheme = layers[0].scheme
+        if any(m.scheme != scheme or m.in_features != layers[0].in_features for m in layers):
+            raise ValueError("fused linears must share scheme and input width")
+        if any(m.out_features % 16 != 0 for m in layers[:-1]):
+            raise ValueError("only the last of several fused linears may have a ragged row count")
+        self.scheme = scheme
+        self.out_features = sum(m.out_features for m in layers)
+        self.wq = torch.cat([m.wq for m in layers], dim=0).contiguous()
+        self.meta = torch.cat([m.meta for m in layers], dim=0).contiguous()
+
+    def __call__(self, x_bf16: torch.Tensor) -> torch.Tensor:
+        fn = w8a16_matmul if self.scheme == "w8a16" else w4a16_matmul
+        return fn(x_bf16, self.wq, self.meta, torch.float32, kernel="gemv")
+
+
+class FusedDecoder(GraphDecoder):
+    """GraphDecoder whose step runs on this library's kernels only: fused q|k|v and w1|w3
+    matmuls, residual add + RMSNorm, RoPE + cache write, single-query attention and the SwiGLU
+    gate (``ajq_add_rmsnorm`` / ``ajq_rope_cache`` / ``ajq_attn_decode`` / ``ajq_swiglu``), plus
+    the embedding lookup and the argmax from PyTorch.  About ten launches per layer.
+
+    Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
+    head_dim 128, an untied quantized ``lm_head``, every linear a QuantLinear, batch <= 16."""
+
+    def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int) -> None:
+        super().__init__(model, batch, max_len)
+        if batch > 16:
+            raise ValueError("FusedDecoder decodes at most 16 sequences at a time")
+        first = model.layers[0]
+        ok = (
+            model.position_encoding == "rope" and first.norm_placement == "pre"
+            and isinstance(first.norm1, modeling.RMSNorm) and isinstance(first.feed_forward, modeling.SwiGLU)
+            and isinstance(model.final_norm, modeling.RMSNorm) and isinstance(model.lm_head, QuantLinear)
+            and model.d_model // model.num_heads == 128
+            and all(isinstance(m, QuantLinear) for layer in model.layers
+                    for m in (layer.attention.q_proj, layer.attention.k_proj, layer.attention.v_proj,
+                              layer.attention.output_proj, layer.feed_forward.w1, layer.feed_forward.w2,
+                              layer.feed_forward.w3))
+        )
+        if not ok:
+            raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128 and "
+                             "quantized linears everywhere (untied lm_head included)")
+        dev, d = self.device, model.d_model
+        self.heads, self.kv_heads, self.head_dim = model.num_heads, model.num_kv_heads, 128
+        self.d_ff = first.feed_forward.w1.out_features
+        self.layers = []
+        for layer in model.layers:
+            att, ff = layer.attention, layer.feed_forward
+            self.layers.append({
+                "g1": layer.norm1.weight.detach().float().contiguous(), "eps1": layer.norm1.epsilon,
+                "g2": layer.norm2.weight.detach().float().contiguous(), "eps2": layer.norm2.epsilon,
+                "qkv": _FusedLinear([att.q_proj, att.k_proj, att.v_proj]),
+                "o": _FusedLinear([att.output_proj]),
+                "w13": _FusedLinear([ff.w1, ff.w3]),
+                "w2": _FusedLinear([ff.w2]),
+                "cos": att.rope.cosine.float().contiguous(), "sin": att.rope.sine.float().contiguous(),
+            })
+        self.final_gain = model.final_norm.weight.detach().float().contiguous()
+        self.final_eps = model.final_norm.epsilon
+        self.head = _FusedLinear([model.lm_head])
+        self.vocab = model.lm_head.out_features
+        self.embedding = model.token_embeddings.weight.detach()
+        self.hidden = torch.zeros((batch, d), dtype=torch.float32, device=dev)
+        self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
+        self.q_rot = torch.zeros((batch, self.heads, 128), dtype=torch.float32, device=dev)
+        self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
+        self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)
+        lib = _lib.load()
+        self.attn_ws_bytes = int(lib.ajq_attn_decode_workspace_bytes(batch, self.heads))
+        self.attn_ws = torch.zeros(max(self.attn_ws_bytes, 16), dtype=torch.uint8, device=dev)
+
+    def _logits(self) -> torch.Tensor:
+        lib, st = _lib.load(), _stream()
+        b, d = self.batch, self.model.d_model
+        pos = self.cache.position
+        torch.index_select(self.embedding, 0, self.token.view(-1), out=self.hidden)
+        delta = None
+        for index, w in enumerate(self.layers):
+            _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                           w["g1"].data_ptr(), w["eps1"], self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+            qkv = w["qkv"](self.normed)
+            _lib.check(lib.ajq_rope_cache(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
+                                          self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
+                                          self.cache.values[index].data_ptr(), b, self.heads, self.kv_heads, 128,
+                                          self.max_len, st), "rope_cache")
+            _lib.check(lib.ajq_attn_decode(self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
+                                           self.cache.values[index].data_ptr(), pos.data_ptr(), b, self.heads,
+                                           self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
+                                           self.attn_ws.data_ptr(), self.attn_ws_bytes, st), "attn_decode")
+            attn_out = w["o"](self.attended)
+            _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), attn_out.data_ptr(), w["g2"].data_ptr(), w["eps2"],
+                                           self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+            ab = w["w13"](self.normed)
+            _lib.check(lib.ajq_swiglu(ab.data_ptr(), self.gated.data_ptr(), b, self.d_ff, st), "swiglu")
+            delta = w["w2"](self.gated)
+        _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), delta.data_ptr(), self.final_gain.data_ptr(),
+                                       self.final_eps, self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+        return self.head(self.normed)[:, : self.vocab]
+
+
 @torch.no_grad()
-def greedy_decode_graph(model: modeling.TransformerLM, prompt: torch.Tensor, max_new_tokens: int) -> torch.Tensor:
+def greedy_decode_graph(model: modeling.TransformerLM, prompt: torch.Tensor, max_new_tokens: int,
+                        fused: bool = False) -> torch.Tensor:
     """``[B, T + new]`` like ``modeling.greedy_decode``, with the per-token step replayed from a graph."""
-    decoder = GraphDecoder(model, prompt.shape[0], prompt.shape[1] + max_new_tokens)
+    cls = FusedDecoder if fused else GraphDecoder
+    decoder = cls(model, prompt.shape[0], prompt.shape[1] + max_new_tokens)
     decoder.prefill(prompt)
     new = decoder.generate(max_new_tokens)
     return torch.cat((prompt.to(new.device), new), dim=1)

@@ -102,6 +102,37 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
+/* ---- the small operators of one decode step around the linears -------------------
+ * fp32 residual stream and KV cache; outputs that feed a linear are bf16.  `pos` is a
+ * DEVICE pointer to the step's cache row, so a recorded HIP graph replays per token. */
+
+/* hidden[B, D] += delta[B, D] (delta may be NULL), out = bf16(RMSNorm(hidden) * gain)
+ * (RMSNorm.forward, src/ajllm/modeling/layers.py:70-74, with the residual add of
+ * TransformerBlock.forward, src/ajllm/modeling/transformer.py:45-50, in front). */
+int ajq_add_rmsnorm(float* hidden, const float* delta, const float* gain, float eps, uint16_t* out,
+                    int B, int D, void* stream);
+
+/* qkv[B, (H + 2 Hkv) * head_dim] -> rotated q[B, H, head_dim]; rotated k and v go to row
+ * *pos of the caches [B, Hkv, max_len, head_dim].  Interleaved-pair rotation with the
+ * cosine / sine tables [positions, head_dim / 2] (RotaryPositionalEmbedding.forward,
+ * src/ajllm/modeling/attention.py:36-60).  The reference has no KV cache
+ * (src/ajllm/generation/generator.py:20-27 recomputes the sequence): the cache is this build's. */
+int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
+                   float* q_out, float* kcache, float* vcache, int B, int H, int Hkv, int head_dim,
+                   int max_len, void* stream);
+
+/* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
+ * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
+ * H / Hkv query heads share a cache head).  head_dim 128 only. */
+size_t ajq_attn_decode_workspace_bytes(int B, int H);
+int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos,
+                    int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* ab[B, 2F] = (w1 x | w3 x) -> out[B, F] = bf16(silu(w1 x) * w3 x)
+ * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */
+int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -140,3 +140,95 @@ def test_graph_replayed_decoding_matches_eager_decoding(cuda, batch):
     got2 = dec.generate(12)
     report2 = compare_greedy(torch.cat((prompt2, got2), 1).cpu(), eager2.cpu(), margins2.cpu(), 20, noise=1e-3)
     assert not report2["unexplained"], report2
+
+
+def test_decode_step_operators_match_their_pytorch_statement(cuda):
+    """ajq_add_rmsnorm / ajq_rope_cache / ajq_attn_decode / ajq_swiglu against the model code's own
+    PyTorch operators on the same fp32 inputs (outputs are bf16: compared after the same cast)."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(21)
+    for b in (1, 3, 8):
+        d, heads, kv_heads, hd, max_len, ff = 512, 4, 2, 128, 40, 384
+        # residual add + RMSNorm
+        hidden = torch.randn((b, d), generator=g).to(cuda)
+        delta = torch.randn((b, d), generator=g).to(cuda)
+        norm = modeling.RMSNorm(d).to(cuda)
+        norm.weight.data = torch.rand(d, generator=g).to(cuda) + 0.5
+        want = norm(hidden + delta).to(torch.bfloat16)
+        out = torch.empty((b, d), dtype=torch.bfloat16, device=cuda)
+        h2 = hidden.clone()
+        _lib.check(lib.ajq_add_rmsnorm(h2.data_ptr(), delta.data_ptr(), norm.weight.data_ptr(), norm.epsilon,
+                                       out.data_ptr(), b, d, st), "add_rmsnorm")
+        assert torch.equal(h2, hidden + delta)
+        assert errors(out, want.cpu())[1] <= 3e-3 and (out.float() - want.float()).abs().max() <= 2 ** -6
+        # RoPE + cache write, then attention over the cache
+        att = modeling.MultiHeadSelfAttention(d, heads, 64, "rope", 10000.0, num_kv_heads=kv_heads).to(cuda)
+        qkv = torch.randn((b, (heads + 2 * kv_heads) * hd), generator=g).to(cuda)
+        kc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda)
+        vc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda)
+        for p in (0, 5, 39):
+            pos = torch.tensor([p], device=cuda)
+            q_rot = torch.empty((b, heads, hd), device=cuda)
+            k2, v2 = kc.clone(), vc.clone()
+            _lib.check(lib.ajq_rope_cache(qkv.data_ptr(), att.rope.cosine.data_ptr(), att.rope.sine.data_ptr(),
+                                          pos.data_ptr(), q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), b, heads,
+                                          kv_heads, hd, max_len, st), "rope_cache")
+            q_in = qkv[:, : heads * hd].view(b, heads, 1, hd)
+            k_in = qkv[:, heads * hd: (heads + kv_heads) * hd].view(b, kv_heads, 1, hd)
+            v_in = qkv[:, (heads + kv_heads) * hd:].view(b, kv_heads, 1, hd)
+            pp = pos.view(1, 1, 1)
+            q_want = att.rope(q_in, pp.expand(b, heads, 1))
+            k_want = att.rope(k_in, pp.expand(b, kv_heads, 1))
+            assert torch.allclose(q_rot, q_want[:, :, 0], atol=1e-6, rtol=1e-6)
+            assert torch.allclose(k2[:, :, p], k_want[:, :, 0], atol=1e-6, rtol=1e-6) and torch.equal(v2[:, :, p], v_in[:, :, 0])
+            untouched = torch.ones(max_len, dtype=torch.bool); untouched[p] = False
+            assert torch.equal(k2[:, :, untouched], kc[:, :, untouched]) and torch.equal(v2[:, :, untouched], vc[:, :, untouched])
+            ws_bytes = lib.ajq_attn_decode_workspace_bytes(b, heads)
+            ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
+            got = torch.empty((b, heads * hd), dtype=torch.bfloat16, device=cuda)
+            _lib.check(lib.ajq_attn_decode(q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), pos.data_ptr(), b, heads,
+                                           kv_heads, hd, max_len, got.data_ptr(), ws.data_ptr(), ws_bytes, st), "attn")
+            rep = heads // kv_heads
+            keys = k2[:, :, : p + 1].repeat_interleave(rep, dim=1)
+            vals = v2[:, :, : p + 1].repeat_interleave(rep, dim=1)
+            want_att = modeling.scaled_dot_product_attention(q_rot.unsqueeze(2), keys, vals)[:, :, 0].reshape(b, heads * hd)
+            assert (got.float() - want_att).abs().max() <= 2e-2 and errors(got, want_att.cpu())[1] <= 3e-3
+        # SwiGLU gate
+        ab = torch.randn((b, 2 * ff), generator=g).to(cuda) * 3
+        want_g = (modeling.silu(ab[:, :ff]) * ab[:, ff:]).to(torch.bfloat16)
+        got_g = torch.empty((b, ff), dtype=torch.bfloat16, device=cuda)
+        _lib.check(lib.ajq_swiglu(ab.data_ptr(), got_g.data_ptr(), b, ff, st), "swiglu")
+        assert errors(got_g, want_g.cpu())[1] <= 3e-3
+
+
+@pytest.mark.parametrize("scheme,batch", [("w4a16_g128", 1), ("w4a16_g128", 5), ("w8a16", 2)])
+def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch):
+    """The all-kernel decode step (FusedDecoder) against the eager model loop, replayed from a
+    graph; differences only below the eager run's own logit-margin noise."""
+    torch.manual_seed(4)
+    model = modeling.TransformerLM(vocab_size=512, context_length=96, d_model=256, num_layers=3, num_heads=2,
+                                   d_ff=640).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(10)).to(cuda)
+    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True)
+    dec = decoding.FusedDecoder(fast, batch, 60)
+    dec.prefill(prompt)
+    first = dec.generate(10)
+    torch.cuda.synchronize()
+    _ = fast(prompt)  # unrelated eager work between replays
+    got = dec.generate(40)
+    assert torch.equal(got[:, :10], first)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 20, noise=2e-3)
+    print(scheme, batch, report)
+    assert not report["unexplained"], report
+    # logits of one fused step against the eager model on the same context
+    dec.prefill(prompt)
+    with torch.no_grad():
+        logits_fused = dec._logits()
+        cache = fast.new_cache(batch, 60)
+        fast(prompt, cache)
+        logits_eager = fast(dec.token, cache)[:, -1, :]
+    max_abs, rel = errors(logits_fused, logits_eager.cpu())
+    assert rel <= 1e-3, (max_abs, rel)
