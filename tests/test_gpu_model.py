@@ -232,3 +232,25 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch):
         logits_eager = fast(dec.token, cache)[:, -1, :]
     max_abs, rel = errors(logits_fused, logits_eager.cpu())
     assert rel <= 1e-3, (max_abs, rel)
+
+
+def test_fused_decoder_tokens_match_the_oracle_model(cuda):
+    """The all-kernel, graph-replayed decode against the CPU oracle model (the restated Transformer
+    with the oracle's QuantLinearRef in every linear slot), batch 4, head_dim 128, GQA off: the
+    end-to-end statement of "identical greedy tokens", up to the oracle's own margin noise."""
+    torch.manual_seed(6)
+    model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=512, num_layers=4, num_heads=4,
+                                   d_ff=1408).eval()
+    ref = _oracle_model(model, "w4a16_g128")
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w4a16_g128")
+    prompt = torch.randint(0, 2048, (4, 64), generator=torch.Generator().manual_seed(12))
+    ref_tokens, margins = modeling.greedy_decode(ref, prompt, 48, return_margins=True)
+    dec = decoding.FusedDecoder(fast, 4, 112)
+    dec.prefill(prompt.to(cuda))
+    got = torch.cat((prompt, dec.generate(48).cpu()), dim=1)
+    with torch.no_grad():
+        noise = 3 * errors(fast(ref_tokens.to(cuda)), ref(ref_tokens))[0]
+    report = compare_greedy(got, ref_tokens, margins, 64, noise=noise)
+    print("fused vs oracle", noise, report)
+    assert not report["unexplained"], report
+    assert report["identical_rows"] + len(report["attributable"]) == 4
