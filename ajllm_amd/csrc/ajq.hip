@@ -97,7 +97,7 @@ constexpr int kGemm256MinM = 256;
 #define AJQ_G2_MT_W4 2
 #endif
 #ifndef AJQ_G2_MT_W8
-#define AJQ_G2_MT_W8 2
+#define AJQ_G2_MT_W8 4
 #endif
 
 }  // namespace

@@ -472,7 +472,10 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     // requested before the two MFMAs of position p are issued (position = 32-row block x
     // k-step), and the order of LDS reads and MFMAs is pinned; VALU work may move freely.
     constexpr int kPos = MT * kSteps;
-    constexpr int kAhead = 4;
+#ifndef AJQ_AHEAD
+#define AJQ_AHEAD 4
+#endif
+    constexpr int kAhead = AJQ_AHEAD;
     auto a_addr = [&](int p) -> const u32x4_t* {
       const int i = p / kSteps, s = p % kSteps;
       const uint32_t off = s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16;
