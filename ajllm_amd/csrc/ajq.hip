@@ -260,6 +260,12 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
     if (M <= 8) return launch_gemv_cfg<8, 2, 8, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
     return launch_gemv_cfg<8, 2, 16, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   }
+  if (K == 11 * 4 * kGroup && M <= 8) {  // K = 5632 (44 groups): eleven waves of four groups, straight-line kernel
+    if (M <= 1) return launch_gemv_cfg<11, 4, 1, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 2) return launch_gemv_cfg<11, 4, 2, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 4) return launch_gemv_cfg<11, 4, 4, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    return launch_gemv_cfg<11, 4, 8, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  }
   if (M <= 1) return launch_gemv_rows<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 2) return launch_gemv_rows<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 4) return launch_gemv_rows<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
