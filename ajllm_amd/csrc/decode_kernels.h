@@ -89,11 +89,13 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
 }
 
 // Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * H, S): a
-// workgroup of 4 waves takes chunk s of the rows; a wave walks its share of the chunk one
-// row at a time (a lane holds 2 of the 128 dimensions: one row is one coalesced 512-byte
-// read), keeping a running maximum, denominator and weighted value sum.  The 4 waves are
-// merged through LDS.  With S == 1 the result is normalised and written as bf16
-// [B, H * 128]; otherwise (max, denominator, 128 sums) go to `partial` for the merge kernel.
+// workgroup of 4 waves takes chunk s of the rows.  Sixteen lanes share one cache row (a
+// lane holds 8 of the 128 dimensions: two 128-bit loads per row and operand), so a wave
+// works on four rows at a time and a workgroup on sixteen, two rounds in flight; every
+// 16-lane team keeps a running maximum, denominator and weighted value sum of its rows.
+// The teams are merged through LDS.  With S == 1 the result is normalised and written as
+// bf16 [B, H * 128]; otherwise (max, denominator, 128 sums) go to `partial` for the merge
+// kernel.
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ kcache,
                                                           const float* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
@@ -103,48 +105,76 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   const int bh = blockIdx.x, S = gridDim.y, s = blockIdx.y;
   const int b = bh / H, h = bh % H;
   const int hk = h / (H / Hkv);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // 16 teams of 16 lanes
   const int rows = (int)(*pos) + 1;
   const int per = (rows + S - 1) / S;
   const int t_begin = s * per, t_end = min(rows, t_begin + per);
-  const float2 qv = *reinterpret_cast<const float2*>(q + (size_t)bh * hd + 2 * lane);
-  const float* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * hd + 2 * lane;
-  const float* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * hd + 2 * lane;
+  const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * hd + 8 * c);
+  const float4 qa = q4[0], qb = q4[1];
+  const float* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * hd + 8 * c;
+  const float* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * hd + 8 * c;
   float m = -INFINITY, l = 0.f;
-  float2 acc = float2{0.f, 0.f};
-  for (int t = t_begin + wave; t < t_end; t += 4) {
-    const float2 kv = *reinterpret_cast<const float2*>(kbase + (size_t)t * hd);
-    const float2 vv = *reinterpret_cast<const float2*>(vbase + (size_t)t * hd);
-    const float sc = wave_sum(qv.x * kv.x + qv.y * kv.y) * scale;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  auto team_dot = [&](const float4& ka, const float4& kb) {
+    float d = qa.x * ka.x + qa.y * ka.y + qa.z * ka.z + qa.w * ka.w + qb.x * kb.x + qb.y * kb.y + qb.z * kb.z + qb.w * kb.w;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) d += __shfl_xor(d, off);
+    return d * scale;
+  };
+  auto update = [&](float sc, const float4& va, const float4& vb) {
     const float m_new = fmaxf(m, sc);
     const float corr = expf(m - m_new), w = expf(sc - m_new);
     l = l * corr + w;
-    acc.x = acc.x * corr + w * vv.x;
-    acc.y = acc.y * corr + w * vv.y;
+    acc[0] = acc[0] * corr + w * va.x; acc[1] = acc[1] * corr + w * va.y;
+    acc[2] = acc[2] * corr + w * va.z; acc[3] = acc[3] * corr + w * va.w;
+    acc[4] = acc[4] * corr + w * vb.x; acc[5] = acc[5] * corr + w * vb.y;
+    acc[6] = acc[6] * corr + w * vb.z; acc[7] = acc[7] * corr + w * vb.w;
     m = m_new;
+  };
+  int t = t_begin + team;
+  for (; t + 16 < t_end; t += 32) {  // two rows per team in flight
+    const float4* k0 = reinterpret_cast<const float4*>(kbase + (size_t)t * hd);
+    const float4* k1 = reinterpret_cast<const float4*>(kbase + (size_t)(t + 16) * hd);
+    const float4* v0 = reinterpret_cast<const float4*>(vbase + (size_t)t * hd);
+    const float4* v1 = reinterpret_cast<const float4*>(vbase + (size_t)(t + 16) * hd);
+    const float4 k0a = k0[0], k0b = k0[1], k1a = k1[0], k1b = k1[1];
+    const float4 v0a = v0[0], v0b = v0[1], v1a = v1[0], v1b = v1[1];
+    const float s0 = team_dot(k0a, k0b), s1 = team_dot(k1a, k1b);
+    update(s0, v0a, v0b);
+    update(s1, v1a, v1b);
   }
-  __shared__ float sm[4], sl[4];
-  __shared__ float2 sacc[4][64];
-  if (lane == 0) { sm[wave] = m; sl[wave] = l; }
-  sacc[wave][lane] = acc;
+  for (; t < t_end; t += 16) {
+    const float4* k0 = reinterpret_cast<const float4*>(kbase + (size_t)t * hd);
+    const float4* v0 = reinterpret_cast<const float4*>(vbase + (size_t)t * hd);
+    const float4 k0a = k0[0], k0b = k0[1], v0a = v0[0], v0b = v0[1];
+    update(team_dot(k0a, k0b), v0a, v0b);
+  }
+  __shared__ float sm[16], sl[16];
+  __shared__ float sacc[16][hd];
+  if (c == 0) { sm[team] = m; sl[team] = l; }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sacc[team][8 * c + i] = acc[i];
   __syncthreads();
-  if (wave != 0) return;
-  float M4 = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x;  // two dimensions per lane from here on
+  float M16 = sm[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) M16 = fmaxf(M16, sm[w]);
   float L = 0.f;
   float2 A = float2{0.f, 0.f};
 #pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    const float c = sm[w] == -INFINITY ? 0.f : expf(sm[w] - M4);
-    L += sl[w] * c;
-    A.x += sacc[w][lane].x * c;
-    A.y += sacc[w][lane].y * c;
+  for (int w = 0; w < 16; ++w) {
+    const float cw = sm[w] == -INFINITY ? 0.f : expf(sm[w] - M16);
+    L += sl[w] * cw;
+    A.x += sacc[w][2 * lane] * cw;
+    A.y += sacc[w][2 * lane + 1] * cw;
   }
   if (S == 1) {
     const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
     reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
   } else {
     float* dst = partial + ((size_t)bh * S + s) * (hd + 2);
-    if (lane == 0) { dst[0] = M4; dst[1] = L; }
+    if (lane == 0) { dst[0] = M16; dst[1] = L; }
     *reinterpret_cast<float2*>(dst + 2 + 2 * lane) = A;
   }
 }
