@@ -135,6 +135,7 @@ class RotaryPositionalEmbedding(nn.Module):
         super().__init__()
         if head_dimension % 2 != 0:
             raise ValueError("RoPE requires an even attention head dimension")
+        self.theta = theta
         positions = torch.arange(max_sequence_length).unsqueeze(1)
         freqs = theta ** (-torch.arange(0, head_dimension, 2).float() / head_dimension)
         angles = positions * freqs

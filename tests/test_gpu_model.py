@@ -254,3 +254,34 @@ def test_fused_decoder_tokens_match_the_oracle_model(cuda):
     print("fused vs oracle", noise, report)
     assert not report["unexplained"], report
     assert report["identical_rows"] + len(report["attributable"]) == 4
+
+
+def test_quantized_checkpoint_round_trip(cuda, tmp_path):
+    """save_quantized -> load_quantized gives a model with the same canonical tensors and the same
+    logits; a dense reference-style checkpoint converts to the same file contents; a flipped byte is
+    caught by the manifest's digest."""
+    from ajllm_amd import checkpoint
+    torch.manual_seed(7)
+    cfg = dict(vocab_size=512, context_length=64, d_model=256, num_layers=2, num_heads=2, d_ff=640)
+    dense = modeling.TransformerLM(**cfg).eval()
+    torch.save({"model_state_dict": dense.state_dict(), "optimizer_state_dict": {}, "step": 5, "metadata": {}},
+               tmp_path / "dense.pt")
+    fast = quantize_model_(copy.deepcopy(dense).to(cuda), "w4a16_g128")
+    path = checkpoint.save_quantized(tmp_path / "q.safetensors", fast, "w4a16_g128",
+                                     config=checkpoint.model_config(fast), metadata={"note": "test"})
+    loaded, manifest = checkpoint.load_quantized(path, cuda)
+    assert manifest["scheme"] == "w4a16_g128" and manifest["group_size"] == 128 and manifest["metadata"]["note"] == "test"
+    a, b = fast.state_dict(), loaded.state_dict()
+    assert set(a) == set(b) and all(torch.equal(a[k], b[k]) for k in a)
+    tokens = torch.randint(0, 512, (2, 9), device=cuda)
+    assert torch.equal(fast(tokens), loaded(tokens))
+    converted = checkpoint.convert_dense_checkpoint(tmp_path / "dense.pt", tmp_path / "c.safetensors", cfg,
+                                                    "w4a16_g128", cuda)
+    t1, m1 = checkpoint.read_quantized(path)
+    t2, m2 = checkpoint.read_quantized(converted)
+    assert m1["sha256"] == m2["sha256"] and m2["metadata"]["step"] == 5
+    raw = bytearray(path.read_bytes())
+    raw[-10] ^= 0xFF
+    (tmp_path / "bad.safetensors").write_bytes(bytes(raw))
+    with pytest.raises(ValueError):
+        checkpoint.read_quantized(tmp_path / "bad.safetensors")

@@ -161,3 +161,18 @@ def test_static_cache_steps_equal_dynamic_decoding():
     assert torch.equal(torch.cat([prompt] + tokens, dim=1), want)
     with pytest.raises(ValueError):
         model(prompt, cache)  # a static cache takes one token per call
+
+
+def test_quantized_checkpoint_manifest_and_foreign_files(tmp_path):
+    """The checkpoint reader refuses files that are not its own format (no GPU needed)."""
+    from safetensors.torch import save_file
+
+    from ajllm_amd import checkpoint
+    save_file({"x": torch.zeros(2)}, str(tmp_path / "foreign.safetensors"))
+    with pytest.raises(ValueError):
+        checkpoint.read_quantized(tmp_path / "foreign.safetensors")
+    model = _model()
+    cfg = checkpoint.model_config(model)
+    assert M.TransformerLM(**cfg).state_dict().keys() == model.state_dict().keys()
+    with pytest.raises(ValueError):
+        checkpoint.save_quantized(tmp_path / "dense.safetensors", model, "w4a16_g128")  # nothing quantized
