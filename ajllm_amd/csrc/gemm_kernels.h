@@ -290,6 +290,28 @@ __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void global_void_t;
 
+// One wave-wide global -> LDS load of 16 bytes per lane: lane l reads base + voff(l) and
+// the 1 KiB lands at LDS byte address lds_addr + 16 l.  The address is given as a scalar
+// base plus a 32-bit per-lane offset so that no 64-bit vector arithmetic is spent on it
+// (the builtin form makes the compiler keep and increment 64-bit VGPR pointers).  The
+// loads are not known to the compiler's wait-count bookkeeping: callers wait for them
+// with an explicit s_waitcnt vmcnt before a barrier.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as clobbered on purpose
+__device__ __forceinline__ void dma16(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(const void* base, uint32_t voff, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 constexpr int kG2BM = 256, kG2BN = 128;
 constexpr int kG2TileBytes = kG2BM * 256;  // 64 KiB: one k-block of activations
 // LDS map (bytes).  Buffers of a pair differ in one address bit, so one XOR flips a
@@ -354,11 +376,15 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   constexpr int kALoads = kLoadRows / 4;
   constexpr int kBLoads = kBTiles / kWaves;
   constexpr int kLoads = kALoads + kBLoads + (kW4 ? 2 : 0);
+  const uint32_t lane16 = (uint32_t)lane * 16u;
+  // meta words of tile (wave & 1) * 4 + (lane >> 4) of the workgroup's eight, word (lane & 15);
+  // tiles past the matrix repeat the last one (their columns are never stored)
+  const uint32_t meta_voff =
+      (uint32_t)((min(nt16_0 + (wave & 1) * 4 + (lane >> 4), ntiles16 - 1) * G * 16 + (lane & 15)) * 4);
   auto issue_load = [&](int j, int kb, int buf) {
     if (j < kALoads) {
-      const char* src = a_base + (size_t)kb * 256 + (size_t)j * 4 * K * 2 + a_voff[j & 3];
-      char* dst = lds + buf * kG2TileBytes + wave * (kLoadRows * 256) + j * 1024;
-      __builtin_amdgcn_global_load_lds((global_void_t*)src, (lds_void_t*)dst, 16, 0, 0);
+      const char* src = a_base + (size_t)kb * 256 + (size_t)j * 4 * K * 2;
+      dma16(src, a_voff[j & 3], (uint32_t)(buf * kG2TileBytes + wave * (kLoadRows * 256) + j * 1024));
     } else if (j < kALoads + kBLoads) {
       // weights: a private tile is 1 KiB contiguous, one wave-wide load each
       const int T = wave * kBLoads + (j - kALoads);
@@ -367,21 +393,16 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
         tile = wq + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 64;
       else
         tile = wq + ((size_t)min(nt16_0 + (T >> 1), ntiles16 - 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
-      __builtin_amdgcn_global_load_lds((global_void_t*)(tile + lane),
-                                       (lds_void_t*)(lds + kWBase + buf * kG2WStride + T * 1024), 16, 0, 0);
+      dma16(tile, lane16, (uint32_t)(kWBase + buf * kG2WStride + T * 1024));
     } else if (j == kALoads + kBLoads) {
       // group-sum pieces of 64 rows; with eight waves the upper four repeat the lower four
       // (same bytes to the same place) rather than branch
       const int e = wave & 3;
-      __builtin_amdgcn_global_load_lds((global_void_t*)(gs3 + (size_t)kb * M + m0 + 64 * e + lane),
-                                       (lds_void_t*)(lds + kG2SideBase + buf * kG2SideBytes + e * 1024), 16, 0, 0);
+      dma16(gs3 + (size_t)kb * M + m0 + 64 * e, lane16, (uint32_t)(kG2SideBase + buf * kG2SideBytes + e * 1024));
     } else {
       // meta words, 4 tiles per load; odd and even waves take one half each
       const int e = wave & 1;
-      const int T = e * 4 + (lane >> 4);
-      __builtin_amdgcn_global_load_lds(
-          (global_void_t*)(meta + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 16 + (lane & 15)),
-          (lds_void_t*)(lds + kG2MetaBase + buf * kG2MetaStride + e * 256), 4, 0, 0);
+      dma4(meta + (size_t)kb * 16, meta_voff, (uint32_t)(kG2MetaBase + buf * kG2MetaStride + e * 256));
     }
   };
 
