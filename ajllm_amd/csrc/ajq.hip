@@ -7,6 +7,7 @@
 #include "quantize_kernels.h"
 #include "gemv_kernels.h"
 #include "gemm_kernels.h"
+#include "skinny_kernels.h"
 #include "decode_kernels.h"
 
 using namespace ajq;
@@ -37,18 +38,32 @@ constexpr int kGemmMpadTo = 256;
 int round_up(int v, int to) { return (v + to - 1) / to * to; }
 
 // Kernels that stage more than 64 KiB in LDS must be opted in once per process
-// (and per device); the largest size granted so far is remembered per kernel.
+// (and per device); the largest size granted so far is remembered per kernel and device.
 template <typename Kernel>
 int allow_big_lds(Kernel kernel, size_t bytes) {
-  static thread_local size_t granted[16] = {0};
+  struct Grant {
+    const void* kernel;
+    size_t bytes[16];
+  };
+  static thread_local Grant grants[64] = {};
   if (bytes <= 64 * 1024) return AJQ_OK;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = 0;
-  if (bytes <= granted[dev]) return AJQ_OK;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  const void* key = reinterpret_cast<const void*>(kernel);
+  Grant* g = nullptr;
+  for (Grant& e : grants) {
+    if (e.kernel == key || e.kernel == nullptr) {
+      g = &e;
+      break;
+    }
+  }
+  if (g && g->kernel == key && bytes <= g->bytes[dev]) return AJQ_OK;
+  hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
   if (e != hipSuccess) return fail(AJQ_ERR_HIP, "hipFuncSetAttribute(%zu B LDS): %s", bytes, hipGetErrorString(e));
-  granted[dev] = bytes;
+  if (g) {  // a full table only costs the repeated call
+    g->kernel = key;
+    g->bytes[dev] = bytes;
+  }
   return AJQ_OK;
 }
 
@@ -277,6 +292,29 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
   return launch_gemv_rows<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
+template <int TPW, int MROWS, bool kW4>
+int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                      const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  constexpr int kWaves = 8;
+  constexpr size_t lds = skinny_lds_bytes(kWaves, TPW, MROWS);
+  static_assert(lds <= 160 * 1024, "skinny configuration exceeds the 160 KiB LDS of a CU");
+  auto kernel = dequant_skinny_kernel<kWaves, TPW, MROWS, kW4>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN, (M + MROWS - 1) / MROWS), dim3(kWaves * 64), lds, stream,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32, scales8);
+  return AJQ_OK;
+}
+
+// 17 <= M < 256: row blocks of 32 (two k groups per batch), 48 or 64 rows (one group per batch:
+// the eight private activation slices have to fit the LDS)
+template <bool kW4>
+int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                  const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  if (M <= 32) return launch_skinny_cfg<2, 32, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (M <= 48) return launch_skinny_cfg<1, 48, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_skinny_cfg<1, 64, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+}
+
 }  // namespace
 
 extern "C" {
@@ -325,6 +363,13 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
       return s;
     return check_launch("ajq_w4a16_gemm");
   }
+#ifndef AJQ_OLD_MID
+  if (M > kMaxGemvM) {
+    if (int s = launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
+      return s;
+    return check_launch("ajq_w4a16_gemm");
+  }
+#endif
   const int Mpad = round_up(M, kGemmMpadTo);
   float* gsum = reinterpret_cast<float*>(workspace);
   hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
@@ -351,6 +396,13 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
       return s;
     return check_launch("ajq_w8a16_gemm");
   }
+#ifndef AJQ_OLD_MID
+  if (M > kMaxGemvM) {
+    if (int s = launch_skinny<false>(x, M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
+      return s;
+    return check_launch("ajq_w8a16_gemm");
+  }
+#endif
   int s;
   if (M <= 64)
     s = launch_gemm<64, 64, 32, 32, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,
@@ -366,9 +418,21 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 
 // --------------------------------------------------- decode-step operators -----
 namespace {
-int attn_splits(int B, int H) {
-  int s = 256 / (B * H);
-  return s < 1 ? 1 : (s > 16 ? 16 : s);
+#ifndef AJQ_ATTN_WGS
+#define AJQ_ATTN_WGS 256
+#endif
+constexpr int kAttnMaxSplits = 16;
+// row chunks per cache head: enough workgroups to cover the CUs
+int attn_splits(int B, int Hkv) {
+  int s = AJQ_ATTN_WGS / (B * Hkv);
+  return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
+}
+
+template <int R>
+void launch_attn(const float* q, const float* kcache, const float* vcache, const long long* pos, int B, int H, int Hkv,
+                 int max_len, float scale, int S, float* partial, uint16_t* out, hipStream_t stream) {
+  hipLaunchKernelGGL(attn_decode_kernel<R>, dim3(B * Hkv, S), dim3(256), 0, stream, q, kcache, vcache, pos, H, Hkv,
+                     max_len, scale, partial, out);
 }
 }  // namespace
 
@@ -401,7 +465,8 @@ int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, con
 
 size_t ajq_attn_decode_workspace_bytes(int B, int H) {
   if (B < 1 || H < 1) return 0;
-  return (size_t)B * H * attn_splits(B, H) * 130 * sizeof(float);
+  // sized for the largest split count: the number of cache heads is not known here
+  return (size_t)B * H * kAttnMaxSplits * 130 * sizeof(float);
 }
 
 int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos, int B, int H, int Hkv,
@@ -410,14 +475,17 @@ int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, co
   if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (only 128 is built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_attn_decode: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
-  const int S = attn_splits(B, H);
+  const int R = H / Hkv;
+  if (R != 1 && R != 2 && R != 4)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: %d query heads per cache head (1, 2 and 4 are built)", R);
+  const int S = attn_splits(B, Hkv);
   if (S > 1 && (!workspace || workspace_bytes < ajq_attn_decode_workspace_bytes(B, H)))
     return fail(AJQ_ERR_WORKSPACE, "ajq_attn_decode: workspace of %zu bytes needed, %zu given",
                 ajq_attn_decode_workspace_bytes(B, H), workspace_bytes);
   const float scale = 1.0f / sqrtf((float)head_dim);
-  hipLaunchKernelGGL(attn_decode_kernel, dim3(B * H, S), dim3(256), 0, (hipStream_t)stream, q, kcache, vcache,
-                     reinterpret_cast<const long long*>(pos), H, Hkv, max_len, scale,
-                     reinterpret_cast<float*>(workspace), out);
+  auto launch = R == 1 ? launch_attn<1> : R == 2 ? launch_attn<2> : launch_attn<4>;
+  launch(q, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len, scale, S,
+         reinterpret_cast<float*>(workspace), out, (hipStream_t)stream);
   if (S > 1)
     hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, (hipStream_t)stream,
                        reinterpret_cast<const float*>(workspace), S, out);

@@ -88,48 +88,64 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
     *reinterpret_cast<float2*>(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i) = r;
 }
 
-// Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * H, S): a
-// workgroup of 4 waves takes chunk s of the rows.  Sixteen lanes share one cache row (a
-// lane holds 8 of the 128 dimensions: two 128-bit loads per row and operand), so a wave
-// works on four rows at a time and a workgroup on sixteen, two rounds in flight; every
-// 16-lane team keeps a running maximum, denominator and weighted value sum of its rows.
-// The teams are merged through LDS.  With S == 1 the result is normalised and written as
-// bf16 [B, H * 128]; otherwise (max, denominator, 128 sums) go to `partial` for the merge
-// kernel.
+// Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * Hkv, S): a
+// workgroup of 4 waves takes chunk s of the rows of one cache head and serves the R = H / Hkv
+// query heads that share it, so a cache row is read once whatever R is.  Sixteen lanes share
+// one cache row (a lane holds 8 of the 128 dimensions: two 128-bit loads per row and
+// operand), so a wave works on four rows at a time and a workgroup on sixteen, two rounds in
+// flight; every 16-lane team keeps a running maximum, denominator and weighted value sum of
+// its rows per query head.  The teams are merged through LDS.  With S == 1 the result is
+// normalised and written as bf16 [B, H * 128]; otherwise (max, denominator, 128 sums) go to
+// `partial` for the merge kernel.
+template <int R>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ kcache,
                                                           const float* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
                                                           float scale, float* __restrict__ partial,
                                                           uint16_t* __restrict__ out) {
   constexpr int hd = 128;
-  const int bh = blockIdx.x, S = gridDim.y, s = blockIdx.y;
-  const int b = bh / H, h = bh % H;
-  const int hk = h / (H / Hkv);
+  const int bk = blockIdx.x, S = gridDim.y, s = blockIdx.y;
+  const int b = bk / Hkv, hk = bk % Hkv;
+  const int bh0 = b * H + hk * R;  // first of the R query heads
   const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // 16 teams of 16 lanes
   const int rows = (int)(*pos) + 1;
   const int per = (rows + S - 1) / S;
   const int t_begin = s * per, t_end = min(rows, t_begin + per);
-  const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)bh * hd + 8 * c);
-  const float4 qa = q4[0], qb = q4[1];
-  const float* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * hd + 8 * c;
-  const float* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * hd + 8 * c;
-  float m = -INFINITY, l = 0.f;
-  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  auto team_dot = [&](const float4& ka, const float4& kb) {
-    float d = qa.x * ka.x + qa.y * ka.y + qa.z * ka.z + qa.w * ka.w + qb.x * kb.x + qb.y * kb.y + qb.z * kb.z + qb.w * kb.w;
+  float4 qa[R], qb[R];
 #pragma unroll
-    for (int off = 8; off > 0; off >>= 1) d += __shfl_xor(d, off);
-    return d * scale;
-  };
-  auto update = [&](float sc, const float4& va, const float4& vb) {
-    const float m_new = fmaxf(m, sc);
-    const float corr = expf(m - m_new), w = expf(sc - m_new);
-    l = l * corr + w;
-    acc[0] = acc[0] * corr + w * va.x; acc[1] = acc[1] * corr + w * va.y;
-    acc[2] = acc[2] * corr + w * va.z; acc[3] = acc[3] * corr + w * va.w;
-    acc[4] = acc[4] * corr + w * vb.x; acc[5] = acc[5] * corr + w * vb.y;
-    acc[6] = acc[6] * corr + w * vb.z; acc[7] = acc[7] * corr + w * vb.w;
-    m = m_new;
+  for (int r = 0; r < R; ++r) {
+    const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)(bh0 + r) * hd + 8 * c);
+    qa[r] = q4[0];
+    qb[r] = q4[1];
+  }
+  const float* kbase = kcache + (size_t)bk * max_len * hd + 8 * c;
+  const float* vbase = vcache + (size_t)bk * max_len * hd + 8 * c;
+  float m[R], l[R], acc[R][8];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+  }
+  // one cache row against the R queries
+  auto row = [&](const float4& ka, const float4& kb, const float4& va, const float4& vb) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float d = qa[r].x * ka.x + qa[r].y * ka.y + qa[r].z * ka.z + qa[r].w * ka.w + qb[r].x * kb.x + qb[r].y * kb.y +
+                qb[r].z * kb.z + qb[r].w * kb.w;
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) d += __shfl_xor(d, off);
+      const float sc = d * scale;
+      const float m_new = fmaxf(m[r], sc);
+      const float corr = expf(m[r] - m_new), w = expf(sc - m_new);
+      l[r] = l[r] * corr + w;
+      acc[r][0] = acc[r][0] * corr + w * va.x; acc[r][1] = acc[r][1] * corr + w * va.y;
+      acc[r][2] = acc[r][2] * corr + w * va.z; acc[r][3] = acc[r][3] * corr + w * va.w;
+      acc[r][4] = acc[r][4] * corr + w * vb.x; acc[r][5] = acc[r][5] * corr + w * vb.y;
+      acc[r][6] = acc[r][6] * corr + w * vb.z; acc[r][7] = acc[r][7] * corr + w * vb.w;
+      m[r] = m_new;
+    }
   };
   int t = t_begin + team;
   for (; t + 16 < t_end; t += 32) {  // two rows per team in flight
@@ -139,43 +155,47 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     const float4* v1 = reinterpret_cast<const float4*>(vbase + (size_t)(t + 16) * hd);
     const float4 k0a = k0[0], k0b = k0[1], k1a = k1[0], k1b = k1[1];
     const float4 v0a = v0[0], v0b = v0[1], v1a = v1[0], v1b = v1[1];
-    const float s0 = team_dot(k0a, k0b), s1 = team_dot(k1a, k1b);
-    update(s0, v0a, v0b);
-    update(s1, v1a, v1b);
+    row(k0a, k0b, v0a, v0b);
+    row(k1a, k1b, v1a, v1b);
   }
   for (; t < t_end; t += 16) {
     const float4* k0 = reinterpret_cast<const float4*>(kbase + (size_t)t * hd);
     const float4* v0 = reinterpret_cast<const float4*>(vbase + (size_t)t * hd);
     const float4 k0a = k0[0], k0b = k0[1], v0a = v0[0], v0b = v0[1];
-    update(team_dot(k0a, k0b), v0a, v0b);
+    row(k0a, k0b, v0a, v0b);
   }
-  __shared__ float sm[16], sl[16];
-  __shared__ float sacc[16][hd];
-  if (c == 0) { sm[team] = m; sl[team] = l; }
+  __shared__ float sm[R][16], sl[R][16];
+  __shared__ float sacc[R][16][hd];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) sacc[team][8 * c + i] = acc[i];
+  for (int r = 0; r < R; ++r) {
+    if (c == 0) { sm[r][team] = m[r]; sl[r][team] = l[r]; }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sacc[r][team][8 * c + i] = acc[r][i];
+  }
   __syncthreads();
-  if (threadIdx.x >= 64) return;
-  const int lane = threadIdx.x;  // two dimensions per lane from here on
-  float M16 = sm[0];
+  // wave w merges query heads w, w + 4, ...; two dimensions per lane from here on
+  const int lane = threadIdx.x & 63;
+  for (int r = threadIdx.x >> 6; r < R; r += 4) {
+    float M16 = sm[r][0];
 #pragma unroll
-  for (int w = 1; w < 16; ++w) M16 = fmaxf(M16, sm[w]);
-  float L = 0.f;
-  float2 A = float2{0.f, 0.f};
+    for (int w = 1; w < 16; ++w) M16 = fmaxf(M16, sm[r][w]);
+    float L = 0.f;
+    float2 A = float2{0.f, 0.f};
 #pragma unroll
-  for (int w = 0; w < 16; ++w) {
-    const float cw = sm[w] == -INFINITY ? 0.f : expf(sm[w] - M16);
-    L += sl[w] * cw;
-    A.x += sacc[w][2 * lane] * cw;
-    A.y += sacc[w][2 * lane + 1] * cw;
-  }
-  if (S == 1) {
-    const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
-    reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
-  } else {
-    float* dst = partial + ((size_t)bh * S + s) * (hd + 2);
-    if (lane == 0) { dst[0] = M16; dst[1] = L; }
-    *reinterpret_cast<float2*>(dst + 2 + 2 * lane) = A;
+    for (int w = 0; w < 16; ++w) {
+      const float cw = sm[r][w] == -INFINITY ? 0.f : expf(sm[r][w] - M16);
+      L += sl[r][w] * cw;
+      A.x += sacc[r][w][2 * lane] * cw;
+      A.y += sacc[r][w][2 * lane + 1] * cw;
+    }
+    if (S == 1) {
+      const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
+      reinterpret_cast<uint32_t*>(out + (size_t)(bh0 + r) * hd)[lane] = o;
+    } else {
+      float* dst = partial + ((size_t)(bh0 + r) * S + s) * (hd + 2);
+      if (lane == 0) { dst[0] = M16; dst[1] = L; }
+      *reinterpret_cast<float2*>(dst + 2 + 2 * lane) = A;
+    }
   }
 }
 

@@ -1,0 +1,195 @@
+// Batched-decode dequant matmul, 17 <= M < 256:  y[M, N] = x[M, K] @ W_hat[N, K]^T.
+//
+// Still bound by the weight stream (a 4096 x 4096 int8 matrix is 16 MB, 32 rows of
+// activations are 256 KB), so this is the decode GEMV's layout with more rows:
+//  * one workgroup owns one 16-row tile of N, one block of MROWS rows of M and all
+//    of K; wave w owns a contiguous run of 128-wide k groups (a contiguous run of
+//    the private 1 KiB weight tiles) and works through it TPW groups at a time, the
+//    next batch in flight while one is computed;
+//  * a wave stages ITS k-slice of the activation block in a wave-private LDS region
+//    (rows padded by 16 B, no workgroup barrier) and reads it back as MFMA A
+//    fragments, one per 16 rows; a weight fragment is unpacked once and meets
+//    MROWS / 16 of them;
+//  * W4 zero points: the group sums of the activations come from MFMAs against an
+//    all-ones operand, in the accumulator's layout, as in the GEMV;
+//  * the waves' partial sums meet once in LDS (each wave's own region, which it no
+//    longer needs) and are added in wave order: no atomics, run-to-run identical.
+// Every workgroup reads its whole activation block from L2 (MROWS * K * 2 bytes
+// against 16 * K weight bytes or half that), which is what bounds the kernel for
+// M above about 32: a CU's vector memory path moves 64 bytes per clock.
+#pragma once
+#include "gemv_kernels.h"
+
+namespace ajq {
+
+template <int kWaves, int TPW, int MROWS, bool kW4>
+__global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
+    const u32x4_t* __restrict__ wq,
+    const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
+    const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
+    const uint16_t* __restrict__ scales8) {  // W8: fp16 [N]; W4: unused
+  static_assert(MROWS % 16 == 0, "row block is a whole number of MFMA tiles");
+  constexpr int MB = MROWS / 16;
+  constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
+  constexpr int kStride = kSlice + 8;      // padded LDS row, bf16 elements
+  constexpr int kVecPerRow = kSlice / 8;   // 16-byte vectors per slice row
+  constexpr int kXLoads = MROWS * kVecPerRow / 64;
+  constexpr int kLoadsPerGroup = kW4 ? 1 : 2;
+  using Batch = GemvBatch<TPW, kXLoads, kLoadsPerGroup>;
+
+  extern __shared__ u32x4_t smem_raw[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nl = lane & 15, kc = lane >> 4;
+  const int nt = blockIdx.x;
+  const int m0 = blockIdx.y * MROWS;
+  const int G = K >> 7;
+  constexpr int kRegion = MROWS * kStride;  // bf16 elements of one wave's region
+  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * kRegion;
+
+  const int per_wave = (G + kWaves - 1) / kWaves;
+  const int g_begin = wave * per_wave;
+  const int g_end = min(G, g_begin + per_wave);
+
+  const u32x4_t* wtile = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
+  const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
+
+  // unconditional loads with clamped addresses: the number in flight is static
+  auto load = [&](Batch& b, int g0) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      const int g = min(g0 + p, g_end - 1);
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
+    }
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = lane + 64 * i;
+      const int m = min(m0 + v / kVecPerRow, M - 1), c = v % kVecPerRow;
+      const int k = min(g0 * kGroup + 8 * c, K - 8);
+      b.x[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + k);
+    }
+    if (kW4) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) b.m[p] = mtile[(size_t)min(g0 + p, g_end - 1) * 16];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const uint32_t mask = 0x000F000Fu;
+  uint32_t magic = 0x43004300u;
+  asm volatile("" : "+v"(magic));  // keep it in a VGPR for v_and_or_b32
+  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  const uint16_t* xrow = xs + nl * kStride + 8 * kc;  // A fragment of row block 0; block b is 16 rows further
+  f32x4_t acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  auto compute = [&](Batch& b, int g0) {
+    float sc[TPW], zc[TPW];
+    if (kW4) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) {
+        sc[p] = f16_bits_to_f32(b.m[p] & 0xFFFFu);
+        zc[p] = f16_bits_to_f32(b.m[p] >> 16);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // LDS operations of one wave execute in order: the previous batch's reads are done
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = lane + 64 * i;
+      *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = b.x[i];
+    }
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      if (g0 + p < g_end) {
+        if (kW4) {
+          f32x4_t part[MB], asum[MB];
+#pragma unroll
+          for (int r = 0; r < MB; ++r) part[r] = asum[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x4_t w = w4_unpack(b.w[p][0][j], mask, magic);
+#pragma unroll
+            for (int r = 0; r < MB; ++r) {
+              const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + r * 16 * kStride + p * kGroup + 32 * j);
+              part[r] = mfma16(a, w, part[r]);
+              asum[r] = mfma16(a, ones, asum[r]);
+            }
+          }
+          // (128+q) and (128+z) cancel in fp32 before the scale is applied
+#pragma unroll
+          for (int r = 0; r < MB; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[r][i] += sc[p] * (part[r][i] - zc[p] * asum[r][i]);
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u32x2_t lo = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1)]);
+            const u32x2_t hi = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1) + 1]);
+            const u32x4_t w = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+            for (int r = 0; r < MB; ++r) {
+              const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + r * 16 * kStride + p * kGroup + 32 * j);
+              acc[r] = mfma16(a, w, acc[r]);
+            }
+          }
+        }
+      }
+    }
+  };
+
+  if (g_begin < g_end) {
+    Batch b0, b1;
+    load(b0, g_begin);
+    for (int g0 = g_begin; g0 < g_end; g0 += 2 * TPW) {
+      const bool has1 = g0 + TPW < g_end;
+      if (has1) load(b1, g0 + TPW);
+      compute(b0, g0);
+      if (g0 + 2 * TPW < g_end) load(b0, g0 + 2 * TPW);
+      if (has1) compute(b1, g0 + TPW);
+    }
+  }
+
+  // ---- partial sums: every wave parks its MB accumulators at the start of its own region
+  // (its LDS reads are done: same wave, in order); wave r adds row block r in wave order
+#pragma unroll
+  for (int r = 0; r < MB; ++r) asm volatile("" : "+v"(acc[r]));
+  f32x4_t* mine = reinterpret_cast<f32x4_t*>(xs);
+#pragma unroll
+  for (int r = 0; r < MB; ++r) mine[r * 64 + lane] = acc[r];
+  __syncthreads();
+  const int n = nt * kTileN + nl;
+  float cs = 1.0f;
+  if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
+  for (int r = wave; r < MB; r += kWaves) {
+    f32x4_t part[kWaves];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+      part[w] = reinterpret_cast<const f32x4_t*>(reinterpret_cast<uint16_t*>(smem_raw) + w * kRegion)[r * 64 + lane];
+    f32x4_t sum = part[0];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) sum += part[w];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * r + 4 * kc + i;
+      if (m < M) {
+        const float v = sum[i] * cs;
+        if (out_f32)
+          reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
+        else
+          reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+      }
+    }
+  }
+}
+
+// LDS bytes of one workgroup of dequant_skinny_kernel<kWaves, TPW, MROWS, *>
+constexpr size_t skinny_lds_bytes(int waves, int tpw, int mrows) {
+  return (size_t)waves * mrows * (tpw * kGroup + 8) * 2;
+}
+
+}  // namespace ajq

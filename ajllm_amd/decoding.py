@@ -48,13 +48,20 @@ class GraphDecoder:
         self.step_index.add_(1)
 
     @torch.no_grad()
-    def prefill(self, prompt: torch.Tensor) -> None:
-        """Run the prompt ``[B, T]`` through the model (eagerly) and choose the first new token."""
+    def prefill(self, prompt: torch.Tensor, rows_per_pass: int | None = None) -> None:
+        """Run the prompt ``[B, T]`` through the model (eagerly) and choose the first new token.
+        ``rows_per_pass`` sequences go through the model at a time (default: all of them)."""
         if prompt.shape[0] != self.batch or prompt.shape[1] >= self.max_len:
             raise ValueError("prompt must be [batch, T] with T < max_len")
         self.cache.static = False
-        self.cache.length = 0
-        logits = self.model(prompt.to(self.device), self.cache, last_token_only=True)[:, -1, :]
+        prompt = prompt.to(self.device)
+        step = rows_per_pass or self.batch
+        parts = []
+        for start in range(0, self.batch, step):
+            rows = self.cache.rows(start, min(start + step, self.batch))
+            parts.append(self.model(prompt[start:start + step], rows, last_token_only=True)[:, -1, :])
+        logits = torch.cat(parts, dim=0)
+        self.cache.length = prompt.shape[1]
         self.cache.static = True
         self.cache.position.fill_(prompt.shape[1])
         self.step_index.zero_()
@@ -116,7 +123,7 @@ class _FusedLinear:
 
     def __call__(self, x_bf16: torch.Tensor) -> torch.Tensor:
         fn = w8a16_matmul if self.scheme == "w8a16" else w4a16_matmul
-        return fn(x_bf16, self.wq, self.meta, torch.float32, kernel="gemv")
+        return fn(x_bf16, self.wq, self.meta, torch.float32)
 
 
 class FusedDecoder(GraphDecoder):
@@ -126,18 +133,17 @@ class FusedDecoder(GraphDecoder):
     the embedding lookup and the argmax from PyTorch.  About ten launches per layer.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
-    head_dim 128, an untied quantized ``lm_head``, every linear a QuantLinear, batch <= 16."""
+    head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
+    linear a QuantLinear."""
 
     def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int) -> None:
         super().__init__(model, batch, max_len)
-        if batch > 16:
-            raise ValueError("FusedDecoder decodes at most 16 sequences at a time")
         first = model.layers[0]
         ok = (
             model.position_encoding == "rope" and first.norm_placement == "pre"
             and isinstance(first.norm1, modeling.RMSNorm) and isinstance(first.feed_forward, modeling.SwiGLU)
             and isinstance(model.final_norm, modeling.RMSNorm) and isinstance(model.lm_head, QuantLinear)
-            and model.d_model // model.num_heads == 128
+            and model.d_model // model.num_heads == 128 and model.num_heads // model.num_kv_heads in (1, 2, 4)
             and all(isinstance(m, QuantLinear) for layer in model.layers
                     for m in (layer.attention.q_proj, layer.attention.k_proj, layer.attention.v_proj,
                               layer.attention.output_proj, layer.feed_forward.w1, layer.feed_forward.w2,

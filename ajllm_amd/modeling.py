@@ -136,11 +136,14 @@ class RotaryPositionalEmbedding(nn.Module):
         if head_dimension % 2 != 0:
             raise ValueError("RoPE requires an even attention head dimension")
         self.theta = theta
-        positions = torch.arange(max_sequence_length).unsqueeze(1)
-        freqs = theta ** (-torch.arange(0, head_dimension, 2).float() / head_dimension)
+        # the tables are not stored in checkpoints: always form them on the host, so that a model
+        # built directly on a GPU gets the same values as one built on the host and moved there
+        target = torch.empty(0).device
+        positions = torch.arange(max_sequence_length, device="cpu").unsqueeze(1)
+        freqs = theta ** (-torch.arange(0, head_dimension, 2, device="cpu").float() / head_dimension)
         angles = positions * freqs
-        self.register_buffer("cosine", torch.cos(angles), persistent=False)
-        self.register_buffer("sine", torch.sin(angles), persistent=False)
+        self.register_buffer("cosine", torch.cos(angles).to(target), persistent=False)
+        self.register_buffer("sine", torch.sin(angles).to(target), persistent=False)
 
     def forward(self, inputs: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         cos, sin = self.cosine[positions], self.sine[positions]
@@ -168,6 +171,19 @@ class KVCache:
         self.static = False
         self.position = torch.zeros(1, dtype=torch.long, device=device)
         self.slots = torch.arange(max_len, device=device)
+
+    def rows(self, start: int, stop: int) -> "KVCache":
+        """A cache over sequences ``start .. stop - 1`` of this one, sharing its storage (dynamic
+        mode, empty): what a prompt that is processed a few sequences at a time writes into."""
+        view = object.__new__(KVCache)
+        view.keys = [k[start:stop] for k in self.keys]
+        view.values = [v[start:stop] for v in self.values]
+        view.length = 0
+        view.max_len = self.max_len
+        view.static = False
+        view.position = self.position
+        view.slots = self.slots
+        return view
 
 
 class MultiHeadSelfAttention(nn.Module):

@@ -152,6 +152,23 @@ def test_gemm_ragged_m(cuda, scheme, m):
     _check(scheme, "gemm", m, 272, 640, seed=33, cuda=cuda, outliers=True)
 
 
+@pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [32, 40, 64, 128, 255])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_batched_decode_matmul(cuda, scheme, m, n, k):
+    """17 <= M < 256 (several sequences decoded together): the weight-streaming kernel with
+    32-, 48- and 64-row activation blocks, at the sweep's matrix sizes."""
+    _check(scheme, "gemm", m, n, k, seed=31, cuda=cuda, outliers=True, max_rows=64)
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_batched_decode_matmul_is_deterministic(cuda, scheme):
+    w_hat, wq, meta = _quantized(scheme, 4096, 4096, 31, cuda)
+    x = make_activations(32, 4096, 9).to(cuda)
+    runs = [_run(scheme, x, wq, meta, torch.float32, "gemm") for _ in range(3)]
+    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemv_and_gemm_agree(cuda, scheme):
     w_hat, wq, meta = _quantized(scheme, 2048, 2048, 41, cuda)
