@@ -107,7 +107,10 @@ int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   return AJQ_OK;
 }
 
-constexpr int kGemm256MinM = 256;
+#ifndef AJQ_GEMM256_MIN_M
+#define AJQ_GEMM256_MIN_M 256
+#endif
+constexpr int kGemm256MinM = AJQ_GEMM256_MIN_M;
 #ifndef AJQ_G2_MT_W4
 #define AJQ_G2_MT_W4 2
 #endif
@@ -292,27 +295,39 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
   return launch_gemv_rows<8, 2, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
-template <int TPW, int MROWS, bool kW4>
+template <int TPW, int MROWS, int NT, bool kW4>
 int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                       const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   constexpr int kWaves = 8;
   constexpr size_t lds = skinny_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "skinny configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_skinny_kernel<kWaves, TPW, MROWS, kW4>;
+  auto kernel = dequant_skinny_kernel<kWaves, TPW, MROWS, NT, kW4>;
   if (int s = allow_big_lds(kernel, lds)) return s;
-  hipLaunchKernelGGL(kernel, dim3(N / kTileN, (M + MROWS - 1) / MROWS), dim3(kWaves * 64), lds, stream,
+  const int ntiles = N / kTileN;
+  hipLaunchKernelGGL(kernel, dim3((ntiles + NT - 1) / NT, (M + MROWS - 1) / MROWS), dim3(kWaves * 64), lds, stream,
                      reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32, scales8);
   return AJQ_OK;
 }
 
-// 17 <= M < 256: row blocks of 32 (two k groups per batch), 48 or 64 rows (one group per batch:
-// the eight private activation slices have to fit the LDS)
+#ifndef AJQ_SKINNY_FORCE_NT
+#define AJQ_SKINNY_FORCE_NT 0
+#endif
+
+// 17 <= M < 256.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup: as
+// many as still leave a workgroup for every CU.  (Wider row blocks lose to more row tiles: a
+// workgroup's traffic is K * (2 * rows + bytes per weight * 16 * tiles) for rows * 16 * tiles
+// outputs.)
 template <bool kW4>
 int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
-  if (M <= 32) return launch_skinny_cfg<2, 32, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  if (M <= 48) return launch_skinny_cfg<1, 48, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
-  return launch_skinny_cfg<1, 64, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  const int ntiles = N / kTileN;
+  const int mblocks = (M + 31) / 32;
+  int nt = 1;
+  while (nt < 4 && (ntiles / (2 * nt)) * mblocks >= 256) nt *= 2;
+  if (AJQ_SKINNY_FORCE_NT) nt = AJQ_SKINNY_FORCE_NT;
+  if (nt == 1) return launch_skinny_cfg<2, 32, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  if (nt == 2) return launch_skinny_cfg<1, 32, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  return launch_skinny_cfg<1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
 }  // namespace

@@ -2,14 +2,15 @@
 //
 // Still bound by the weight stream (a 4096 x 4096 int8 matrix is 16 MB, 32 rows of
 // activations are 256 KB), so this is the decode GEMV's layout with more rows:
-//  * one workgroup owns one 16-row tile of N, one block of MROWS rows of M and all
-//    of K; wave w owns a contiguous run of 128-wide k groups (a contiguous run of
-//    the private 1 KiB weight tiles) and works through it TPW groups at a time, the
-//    next batch in flight while one is computed;
+//  * one workgroup owns NT consecutive 16-row tiles of N, one block of MROWS rows of
+//    M and all of K; wave w owns a contiguous run of 128-wide k groups (a contiguous
+//    run of the private 1 KiB weight tiles of each row tile) and works through it
+//    TPW groups at a time, the next batch in flight while one is computed;
 //  * a wave stages ITS k-slice of the activation block in a wave-private LDS region
 //    (rows padded by 16 B, no workgroup barrier) and reads it back as MFMA A
 //    fragments, one per 16 rows; a weight fragment is unpacked once and meets
-//    MROWS / 16 of them;
+//    MROWS / 16 of them, an activation fragment is read once and meets NT weight
+//    fragments (NT > 1 is for shapes with more row tiles than the chip has CUs);
 //  * W4 zero points: the group sums of the activations come from MFMAs against an
 //    all-ones operand, in the accumulator's layout, as in the GEMV;
 //  * the waves' partial sums meet once in LDS (each wave's own region, which it no
@@ -22,7 +23,14 @@
 
 namespace ajq {
 
-template <int kWaves, int TPW, int MROWS, bool kW4>
+template <int NT, int TPW, int kXLoads, int kLoadsPerGroup>
+struct SkinnyBatch {
+  u32x4_t w[NT][TPW][kLoadsPerGroup];
+  u32x4_t x[kXLoads];
+  uint32_t m[NT][TPW];
+};
+
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4>
 __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -35,13 +43,15 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
   constexpr int kVecPerRow = kSlice / 8;   // 16-byte vectors per slice row
   constexpr int kXLoads = MROWS * kVecPerRow / 64;
   constexpr int kLoadsPerGroup = kW4 ? 1 : 2;
-  using Batch = GemvBatch<TPW, kXLoads, kLoadsPerGroup>;
+  using Batch = SkinnyBatch<NT, TPW, kXLoads, kLoadsPerGroup>;
+  static_assert(NT * MB * 1024 <= MROWS * (kSlice + 8) * 2, "a wave's partial sums must fit its own LDS region");
 
   extern __shared__ u32x4_t smem_raw[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nl = lane & 15, kc = lane >> 4;
-  const int nt = blockIdx.x;
+  const int nt0 = blockIdx.x * NT;
+  const int ntiles = N / kTileN;
   const int m0 = blockIdx.y * MROWS;
   const int G = K >> 7;
   constexpr int kRegion = MROWS * kStride;  // bf16 elements of one wave's region
@@ -51,19 +61,28 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
   const int g_begin = wave * per_wave;
   const int g_end = min(G, g_begin + per_wave);
 
-  const u32x4_t* wtile = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
-  const uint32_t* mtile = meta + (size_t)nt * G * 16 + nl;
+  // row tiles past the matrix repeat the last one (their results are not stored)
+  const u32x4_t* wtile[NT];
+  const uint32_t* mtile[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int nt = min(nt0 + t, ntiles - 1);
+    wtile[t] = wq + (size_t)nt * G * kLoadsPerGroup * 64 + lane;
+    mtile[t] = meta + (size_t)nt * G * 16 + nl;
+  }
 
   // unconditional loads with clamped addresses: the number in flight is static
   auto load = [&](Batch& b, int g0) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      const int g = min(g0 + p, g_end - 1);
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h)
-        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
-    }
+      for (int p = 0; p < TPW; ++p) {
+        const int g = min(g0 + p, g_end - 1);
+#pragma unroll
+        for (int h = 0; h < kLoadsPerGroup; ++h)
+          b.w[t][p][h] = __builtin_nontemporal_load(wtile[t] + ((size_t)g * kLoadsPerGroup + h) * 64);
+      }
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = lane + 64 * i;
@@ -73,7 +92,9 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
     }
     if (kW4) {
 #pragma unroll
-      for (int p = 0; p < TPW; ++p) b.m[p] = mtile[(size_t)min(g0 + p, g_end - 1) * 16];
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int p = 0; p < TPW; ++p) b.m[t][p] = mtile[t][(size_t)min(g0 + p, g_end - 1) * 16];
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -83,18 +104,22 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
   asm volatile("" : "+v"(magic));  // keep it in a VGPR for v_and_or_b32
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + nl * kStride + 8 * kc;  // A fragment of row block 0; block b is 16 rows further
-  f32x4_t acc[MB];
+  f32x4_t acc[NT][MB];
 #pragma unroll
-  for (int b = 0; b < MB; ++b) acc[b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[t][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   auto compute = [&](Batch& b, int g0) {
-    float sc[TPW], zc[TPW];
+    float sc[NT][TPW], zc[NT][TPW];
     if (kW4) {
 #pragma unroll
-      for (int p = 0; p < TPW; ++p) {
-        sc[p] = f16_bits_to_f32(b.m[p] & 0xFFFFu);
-        zc[p] = f16_bits_to_f32(b.m[p] >> 16);
-      }
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int p = 0; p < TPW; ++p) {
+          sc[t][p] = f16_bits_to_f32(b.m[t][p] & 0xFFFFu);
+          zc[t][p] = f16_bits_to_f32(b.m[t][p] >> 16);
+        }
       __builtin_amdgcn_sched_barrier(0);
     }
     // LDS operations of one wave execute in order: the previous batch's reads are done
@@ -107,34 +132,48 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
     for (int p = 0; p < TPW; ++p) {
       if (g0 + p < g_end) {
         if (kW4) {
-          f32x4_t part[MB], asum[MB];
+          f32x4_t part[NT][MB], asum[MB];
 #pragma unroll
-          for (int r = 0; r < MB; ++r) part[r] = asum[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          for (int r = 0; r < MB; ++r) {
+            asum[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < NT; ++t) part[t][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+          }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const u32x4_t w = w4_unpack(b.w[p][0][j], mask, magic);
+            u32x4_t w[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) w[t] = w4_unpack(b.w[t][p][0][j], mask, magic);
 #pragma unroll
             for (int r = 0; r < MB; ++r) {
               const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + r * 16 * kStride + p * kGroup + 32 * j);
-              part[r] = mfma16(a, w, part[r]);
               asum[r] = mfma16(a, ones, asum[r]);
+#pragma unroll
+              for (int t = 0; t < NT; ++t) part[t][r] = mfma16(a, w[t], part[t][r]);
             }
           }
           // (128+q) and (128+z) cancel in fp32 before the scale is applied
 #pragma unroll
-          for (int r = 0; r < MB; ++r)
+          for (int t = 0; t < NT; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[r][i] += sc[p] * (part[r][i] - zc[p] * asum[r][i]);
+            for (int r = 0; r < MB; ++r)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) acc[t][r][i] += sc[t][p] * (part[t][r][i] - zc[t][p] * asum[r][i]);
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const u32x2_t lo = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1)]);
-            const u32x2_t hi = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1) + 1]);
-            const u32x4_t w = {lo.x, lo.y, hi.x, hi.y};
+            u32x4_t w[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+              const u32x2_t lo = w8_to_bf16(b.w[t][p][j >> 1][2 * (j & 1)]);
+              const u32x2_t hi = w8_to_bf16(b.w[t][p][j >> 1][2 * (j & 1) + 1]);
+              w[t] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+            }
 #pragma unroll
             for (int r = 0; r < MB; ++r) {
               const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + r * 16 * kStride + p * kGroup + 32 * j);
-              acc[r] = mfma16(a, w, acc[r]);
+#pragma unroll
+              for (int t = 0; t < NT; ++t) acc[t][r] = mfma16(a, w[t], acc[t][r]);
             }
           }
         }
@@ -154,25 +193,32 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
     }
   }
 
-  // ---- partial sums: every wave parks its MB accumulators at the start of its own region
-  // (its LDS reads are done: same wave, in order); wave r adds row block r in wave order
+  // ---- partial sums: every wave parks its NT * MB accumulators at the start of its own region
+  // (its LDS reads are done: same wave, in order); the (row tile, row block) units are dealt
+  // round-robin to the waves, which add them in wave order
 #pragma unroll
-  for (int r = 0; r < MB; ++r) asm volatile("" : "+v"(acc[r]));
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < MB; ++r) asm volatile("" : "+v"(acc[t][r]));
   f32x4_t* mine = reinterpret_cast<f32x4_t*>(xs);
 #pragma unroll
-  for (int r = 0; r < MB; ++r) mine[r * 64 + lane] = acc[r];
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < MB; ++r) mine[(t * MB + r) * 64 + lane] = acc[t][r];
   __syncthreads();
-  const int n = nt * kTileN + nl;
-  float cs = 1.0f;
-  if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
-  for (int r = wave; r < MB; r += kWaves) {
+  for (int u = wave; u < NT * MB; u += kWaves) {
+    const int t = u / MB, r = u % MB;
+    if (nt0 + t >= ntiles) break;
     f32x4_t part[kWaves];
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
-      part[w] = reinterpret_cast<const f32x4_t*>(reinterpret_cast<uint16_t*>(smem_raw) + w * kRegion)[r * 64 + lane];
+      part[w] = reinterpret_cast<const f32x4_t*>(reinterpret_cast<uint16_t*>(smem_raw) + w * kRegion)[u * 64 + lane];
     f32x4_t sum = part[0];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w) sum += part[w];
+    const int n = (nt0 + t) * kTileN + nl;
+    float cs = 1.0f;
+    if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = m0 + 16 * r + 4 * kc + i;

@@ -208,6 +208,8 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=64, help="distinct weight matrices per step")
     ap.add_argument("--sweep", action="store_true", help="also time the full decode and prefill sweeps")
     ap.add_argument("--decode", action="store_true", help="also time end-to-end greedy decode")
+    ap.add_argument("--stack", action="store_true",
+                    help="also time the Llama-3-8B-shaped W8A16 stack (4 x 2048 prefill, batch-32 decode at context 2048)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="timed region only")
     args = ap.parse_args()
@@ -256,6 +258,10 @@ def main() -> int:
         from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
 
         extras["decode"] = bench_decode(device, log)
+    if args.stack:
+        from ajllm_amd.stack_bench import bench_stack
+
+        extras["stack_8b_w8a16"] = bench_stack(device, log)
     # a plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     # counters of a profiling run are scaled by (64 MiB read + 64 MiB written per launch)
     calib_src = torch.empty(64 * 2**20, dtype=torch.uint8, device=device)
