@@ -33,9 +33,6 @@ int check_launch(const char* what) {
 }
 
 constexpr int kMaxGemvM = 16;
-constexpr int kGemmMpadTo = 256;
-
-int round_up(int v, int to) { return (v + to - 1) / to * to; }
 
 // Kernels that stage more than 64 KiB in LDS must be opted in once per process
 // (and per device); the largest size granted so far is remembered per kernel and device.
@@ -77,20 +74,6 @@ int check_matmul_args(const char* name, const void* x, int M, int K, const void*
     return fail(AJQ_ERR_UNSUPPORTED, "%s: out_dtype %d is neither AJQ_OUT_BF16 nor AJQ_OUT_F32", name, out_dtype);
   if (!aligned16(x) || !aligned16(wq) || !aligned16(y))
     return fail(AJQ_ERR_ALIGN, "%s: x, wq and y must be 16-byte aligned", name);
-  return AJQ_OK;
-}
-
-template <int BM, int BN, int WM, int WN, bool kW4>
-int launch_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
-                       const uint16_t* scales8, const float* gsum, int Mpad, int N, void* y, int out_f32,
-                       hipStream_t stream) {
-  constexpr int kThreads = (BM / WM) * (BN / WN) * 64;
-  const size_t lds = (size_t)2 * BM * (128 + 8) * 2;
-  auto kernel = dequant_gemm_kernel<BM, BN, WM, WN, kW4>;
-  if (int s = allow_big_lds(kernel, lds)) return s;
-  const int tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), lds, stream, x, M, K,
-                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8, gsum, Mpad, N, y, out_f32);
   return AJQ_OK;
 }
 
@@ -354,78 +337,48 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 
 // --------------------------------------------------------------- GEMM -----
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K) {
-  if (M < 1 || K < kGroup) return 0;
-  // covers both layouts: fp32 [G][Mpad] (small M) and 16-byte pieces [G][M] (M >= 256)
-  return (size_t)(K / kGroup) * round_up(M, kGemmMpadTo) * 16;
+  if (M < kGemm256MinM || K < kGroup) return 0;  // only the large-M kernel needs the group sums
+  return (size_t)(K / kGroup) * M * 16;
 }
 
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
                    int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   if (int s = check_matmul_args("ajq_w4a16_gemm", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  const bool out_f32 = out_dtype == AJQ_OUT_F32;
+  if (M < kGemm256MinM) {
+    const int s = M <= kMaxGemvM ? launch_gemv<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream)
+                                 : launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream);
+    return s ? s : check_launch("ajq_w4a16_gemm");
+  }
   const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
   if (!workspace || workspace_bytes < need)
     return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm: workspace must be 16-byte aligned");
-  const long long teams = (long long)M * (K / kGroup);
-  if (M >= kGemm256MinM) {
-    if ((long long)M * K * 2 >= (1LL << 32))
-      return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
-    const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
-    hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
-                       K, reinterpret_cast<u32x4_t*>(workspace));
-    if (int s = launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_dtype == AJQ_OUT_F32,
-                                     (hipStream_t)stream))
-      return s;
-    return check_launch("ajq_w4a16_gemm");
-  }
-#ifndef AJQ_OLD_MID
-  if (M > kMaxGemvM) {
-    if (int s = launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
-      return s;
-    return check_launch("ajq_w4a16_gemm");
-  }
-#endif
-  const int Mpad = round_up(M, kGemmMpadTo);
-  float* gsum = reinterpret_cast<float*>(workspace);
-  hipLaunchKernelGGL(group_sum_kernel, dim3((unsigned)((teams + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
-                     K, Mpad, gsum);
-  int s;
-  if (M <= 64)
-    s = launch_gemm<64, 64, 32, 32, true>(x, M, K, wq, meta, nullptr, gsum, Mpad, N, y, out_dtype == AJQ_OUT_F32,
-                                          (hipStream_t)stream);
-  else
-    s = launch_gemm<128, 128, 64, 64, true>(x, M, K, wq, meta, nullptr, gsum, Mpad, N, y,
-                                            out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
-  if (s) return s;
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
+  hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
+                     K, reinterpret_cast<u32x4_t*>(workspace));
+  if (int s = launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32,
+                                                 (hipStream_t)stream))
+    return s;
   return check_launch("ajq_w4a16_gemm");
 }
 
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
                    int out_dtype, void* stream) {
   if (int s = check_matmul_args("ajq_w8a16_gemm", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
-  if (M >= kGemm256MinM) {
-    if ((long long)M * K * 2 >= (1LL << 32))
-      return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
-    if (int s = launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_dtype == AJQ_OUT_F32,
-                                      (hipStream_t)stream))
-      return s;
-    return check_launch("ajq_w8a16_gemm");
+  const bool out_f32 = out_dtype == AJQ_OUT_F32;
+  if (M < kGemm256MinM) {
+    const int s = M <= kMaxGemvM ? launch_gemv<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream)
+                                 : launch_skinny<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream);
+    return s ? s : check_launch("ajq_w8a16_gemm");
   }
-#ifndef AJQ_OLD_MID
-  if (M > kMaxGemvM) {
-    if (int s = launch_skinny<false>(x, M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
-      return s;
-    return check_launch("ajq_w8a16_gemm");
-  }
-#endif
-  int s;
-  if (M <= 64)
-    s = launch_gemm<64, 64, 32, 32, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,
-                                           out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
-  else
-    s = launch_gemm<128, 128, 64, 64, false>(x, M, K, wq, nullptr, scales, nullptr, 0, N, y,
-                                             out_dtype == AJQ_OUT_F32, (hipStream_t)stream);
-  if (s) return s;
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  if (int s = launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32,
+                                                  (hipStream_t)stream))
+    return s;
   return check_launch("ajq_w8a16_gemm");
 }
 

@@ -93,9 +93,11 @@ int ajq_w4a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
-/* prefill shapes, any M >= 1 (tuned for M >= 256); bf16 MFMA.
- * The W4 GEMM needs a workspace of ajq_w4a16_gemm_workspace_bytes(M, K) bytes
- * (per-row, per-group activation sums). */
+/* any M >= 1; bf16 MFMA.  M >= 256 (prefill) runs the 256 x 128 tile kernel, 17 <= M < 256
+ * (several sequences decoded together) a weight-streaming kernel with 32-row activation
+ * blocks, M <= 16 the GEMV above.
+ * The W4 GEMM needs a workspace of ajq_w4a16_gemm_workspace_bytes(M, K) bytes (per-row,
+ * per-group activation sums; 0 bytes below M = 256, where workspace may be NULL). */
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K);
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                    void* y, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
@@ -123,7 +125,8 @@ int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, con
 
 /* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
  * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
- * H / Hkv query heads share a cache head).  head_dim 128 only. */
+ * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of
+ * them).  head_dim 128 only.  The workspace holds the partial results of up to 16 row chunks. */
 size_t ajq_attn_decode_workspace_bytes(int B, int H);
 int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos,
                     int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace,
