@@ -15,6 +15,8 @@ LIBRARY_PATH = Path(__file__).resolve().parent / "libajq.so"
 
 AJQ_OUT_BF16 = 0
 AJQ_OUT_F32 = 1
+AJQ_KV_F32 = 0
+AJQ_KV_BF16 = 1
 
 # status -> exception class; argument errors are ValueError (the reference CLI turns
 # ValueError into a clean exit, src/ajllm/cli.py:57-60), runtime errors RuntimeError.
@@ -43,13 +45,13 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_rope_cache": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-         c_void_p],
+         c_int, c_void_p],
     ),
     "ajq_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int]),
     "ajq_attn_decode": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t,
-         c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
+         c_size_t, c_void_p],
     ),
     "ajq_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
 }

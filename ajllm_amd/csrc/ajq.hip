@@ -396,10 +396,11 @@ int attn_splits(int B, int Hkv) {
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
 }
 
-template <int R>
-void launch_attn(const float* q, const float* kcache, const float* vcache, const long long* pos, int B, int H, int Hkv,
+template <int R, typename CacheT>
+void launch_attn(const float* q, const void* kcache, const void* vcache, const long long* pos, int B, int H, int Hkv,
                  int max_len, float scale, int S, float* partial, uint16_t* out, hipStream_t stream) {
-  hipLaunchKernelGGL(attn_decode_kernel<R>, dim3(B * Hkv, S), dim3(256), 0, stream, q, kcache, vcache, pos, H, Hkv,
+  hipLaunchKernelGGL((attn_decode_kernel<R, CacheT>), dim3(B * Hkv, S), dim3(256), 0, stream, q,
+                     reinterpret_cast<const CacheT*>(kcache), reinterpret_cast<const CacheT*>(vcache), pos, H, Hkv,
                      max_len, scale, partial, out);
 }
 }  // namespace
@@ -418,16 +419,25 @@ int ajq_add_rmsnorm(float* hidden, const float* delta, const float* gain, float 
 }
 
 int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, float* q_out,
-                   float* kcache, float* vcache, int B, int H, int Hkv, int head_dim, int max_len, void* stream) {
+                   void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len,
+                   void* stream) {
   if (!qkv || !cosine || !sine || !pos || !q_out || !kcache || !vcache)
     return fail(AJQ_ERR_NULL, "ajq_rope_cache: null pointer argument");
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || head_dim < 2 || head_dim % 2 != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_rope_cache: unsupported shape (B=%d H=%d Hkv=%d head_dim=%d max_len=%d)", B, H, Hkv,
                 head_dim, max_len);
+  if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_rope_cache: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
   const long long pairs = (long long)B * (H + 2 * Hkv) * (head_dim / 2);
-  hipLaunchKernelGGL(rope_cache_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, (hipStream_t)stream, qkv,
-                     cosine, sine, reinterpret_cast<const long long*>(pos), q_out, kcache, vcache, B, H, Hkv, head_dim,
-                     max_len);
+  const dim3 grid((unsigned)((pairs + 255) / 256));
+  const long long* p = reinterpret_cast<const long long*>(pos);
+  if (cache_dtype == AJQ_KV_F32)
+    hipLaunchKernelGGL(rope_cache_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, qkv, cosine, sine, p, q_out,
+                       reinterpret_cast<float*>(kcache), reinterpret_cast<float*>(vcache), B, H, Hkv, head_dim, max_len);
+  else
+    hipLaunchKernelGGL(rope_cache_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, qkv, cosine, sine, p, q_out,
+                       reinterpret_cast<uint16_t*>(kcache), reinterpret_cast<uint16_t*>(vcache), B, H, Hkv, head_dim,
+                       max_len);
   return check_launch("ajq_rope_cache");
 }
 
@@ -437,8 +447,9 @@ size_t ajq_attn_decode_workspace_bytes(int B, int H) {
   return (size_t)B * H * kAttnMaxSplits * 130 * sizeof(float);
 }
 
-int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos, int B, int H, int Hkv,
-                    int head_dim, int max_len, uint16_t* out, void* workspace, size_t workspace_bytes, void* stream) {
+int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, const int64_t* pos, int B,
+                    int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace, size_t workspace_bytes,
+                    void* stream) {
   if (!q || !kcache || !vcache || !pos || !out) return fail(AJQ_ERR_NULL, "ajq_attn_decode: null pointer argument");
   if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (only 128 is built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
@@ -451,7 +462,13 @@ int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, co
     return fail(AJQ_ERR_WORKSPACE, "ajq_attn_decode: workspace of %zu bytes needed, %zu given",
                 ajq_attn_decode_workspace_bytes(B, H), workspace_bytes);
   const float scale = 1.0f / sqrtf((float)head_dim);
-  auto launch = R == 1 ? launch_attn<1> : R == 2 ? launch_attn<2> : launch_attn<4>;
+  if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+  if (!aligned16(kcache) || !aligned16(vcache) || !aligned16(q))
+    return fail(AJQ_ERR_ALIGN, "ajq_attn_decode: q and the caches must be 16-byte aligned");
+  auto launch = cache_dtype == AJQ_KV_F32
+                    ? (R == 1 ? launch_attn<1, float> : R == 2 ? launch_attn<2, float> : launch_attn<4, float>)
+                    : (R == 1 ? launch_attn<1, uint16_t> : R == 2 ? launch_attn<2, uint16_t> : launch_attn<4, uint16_t>);
   launch(q, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len, scale, S,
          reinterpret_cast<float*>(workspace), out, (hipStream_t)stream);
   if (S > 1)

@@ -61,10 +61,17 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
 // [B, H, hd]; rotated k and plain v are written into the caches [B, Hkv, max_len, hd] at
 // row *pos.  Interleaved pairs: (x[2i], x[2i+1]) -> (e c - o s, e s + o c) with the tables'
 // row *pos.  One thread per pair.
+// The caches hold fp32 or (kBf16) bf16, rounded to nearest even.
+__device__ __forceinline__ void store_pair(float* p, float2 v) { *reinterpret_cast<float2*>(p) = v; }
+__device__ __forceinline__ void store_pair(uint16_t* p, float2 v) {
+  *reinterpret_cast<uint32_t*>(p) = f32_to_bf16_rne(v.x) | ((uint32_t)f32_to_bf16_rne(v.y) << 16);
+}
+
+template <typename CacheT>
 __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict__ qkv, const float* __restrict__ cosine,
                                                          const float* __restrict__ sine, const long long* __restrict__ pos,
-                                                         float* __restrict__ q_out, float* __restrict__ kcache,
-                                                         float* __restrict__ vcache, int B, int H, int Hkv, int hd,
+                                                         float* __restrict__ q_out, CacheT* __restrict__ kcache,
+                                                         CacheT* __restrict__ vcache, int B, int H, int Hkv, int hd,
                                                          int max_len) {
   const int half = hd >> 1;
   const int heads = H + 2 * Hkv;
@@ -77,7 +84,7 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
   const float2 v = *reinterpret_cast<const float2*>(qkv + ((size_t)b * heads + head) * hd + 2 * i);
   if (head >= H + Hkv) {  // value head: stored as it is
     const int hv = head - H - Hkv;
-    *reinterpret_cast<float2*>(vcache + (((size_t)b * Hkv + hv) * max_len + p) * hd + 2 * i) = v;
+    store_pair(vcache + (((size_t)b * Hkv + hv) * max_len + p) * hd + 2 * i, v);
     return;
   }
   const float c = cosine[p * half + i], s = sine[p * half + i];
@@ -85,7 +92,7 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
   if (head < H)
     *reinterpret_cast<float2*>(q_out + ((size_t)b * H + head) * hd + 2 * i) = r;
   else
-    *reinterpret_cast<float2*>(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i) = r;
+    store_pair(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i, r);
 }
 
 // Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * Hkv, S): a
@@ -96,10 +103,28 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
 // flight; every 16-lane team keeps a running maximum, denominator and weighted value sum of
 // its rows per query head.  The teams are merged through LDS.  With S == 1 the result is
 // normalised and written as bf16 [B, H * 128]; otherwise (max, denominator, 128 sums) go to
-// `partial` for the merge kernel.
-template <int R>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const float* __restrict__ kcache,
-                                                          const float* __restrict__ vcache,
+// `partial` for the merge kernel.  A bf16 cache row is 256 B: one 128-bit load per lane and
+// operand, widened to fp32 in registers; all arithmetic is fp32 either way.
+struct KvRow8 {
+  float4 a, b;
+};
+__device__ __forceinline__ KvRow8 load_row8(const float* p) {
+  const float4* p4 = reinterpret_cast<const float4*>(p);
+  return KvRow8{p4[0], p4[1]};
+}
+__device__ __forceinline__ KvRow8 load_row8(const uint16_t* p) {
+  const u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
+  KvRow8 r;
+  r.a = float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u), __uint_as_float(v.y << 16),
+               __uint_as_float(v.y & 0xFFFF0000u)};
+  r.b = float4{__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xFFFF0000u), __uint_as_float(v.w << 16),
+               __uint_as_float(v.w & 0xFFFF0000u)};
+  return r;
+}
+
+template <int R, typename CacheT>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
+                                                          const CacheT* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
                                                           float scale, float* __restrict__ partial,
                                                           uint16_t* __restrict__ out) {
@@ -118,8 +143,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     qa[r] = q4[0];
     qb[r] = q4[1];
   }
-  const float* kbase = kcache + (size_t)bk * max_len * hd + 8 * c;
-  const float* vbase = vcache + (size_t)bk * max_len * hd + 8 * c;
+  const CacheT* kbase = kcache + (size_t)bk * max_len * hd + 8 * c;
+  const CacheT* vbase = vcache + (size_t)bk * max_len * hd + 8 * c;
   float m[R], l[R], acc[R][8];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -149,20 +174,14 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   };
   int t = t_begin + team;
   for (; t + 16 < t_end; t += 32) {  // two rows per team in flight
-    const float4* k0 = reinterpret_cast<const float4*>(kbase + (size_t)t * hd);
-    const float4* k1 = reinterpret_cast<const float4*>(kbase + (size_t)(t + 16) * hd);
-    const float4* v0 = reinterpret_cast<const float4*>(vbase + (size_t)t * hd);
-    const float4* v1 = reinterpret_cast<const float4*>(vbase + (size_t)(t + 16) * hd);
-    const float4 k0a = k0[0], k0b = k0[1], k1a = k1[0], k1b = k1[1];
-    const float4 v0a = v0[0], v0b = v0[1], v1a = v1[0], v1b = v1[1];
-    row(k0a, k0b, v0a, v0b);
-    row(k1a, k1b, v1a, v1b);
+    const KvRow8 k0 = load_row8(kbase + (size_t)t * hd), k1 = load_row8(kbase + (size_t)(t + 16) * hd);
+    const KvRow8 v0 = load_row8(vbase + (size_t)t * hd), v1 = load_row8(vbase + (size_t)(t + 16) * hd);
+    row(k0.a, k0.b, v0.a, v0.b);
+    row(k1.a, k1.b, v1.a, v1.b);
   }
   for (; t < t_end; t += 16) {
-    const float4* k0 = reinterpret_cast<const float4*>(kbase + (size_t)t * hd);
-    const float4* v0 = reinterpret_cast<const float4*>(vbase + (size_t)t * hd);
-    const float4 k0a = k0[0], k0b = k0[1], v0a = v0[0], v0b = v0[1];
-    row(k0a, k0b, v0a, v0b);
+    const KvRow8 k0 = load_row8(kbase + (size_t)t * hd), v0 = load_row8(vbase + (size_t)t * hd);
+    row(k0.a, k0.b, v0.a, v0.b);
   }
   __shared__ float sm[R][16], sl[R][16];
   __shared__ float sacc[R][16][hd];

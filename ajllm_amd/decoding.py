@@ -17,7 +17,8 @@ from .quant import QuantLinear, w4a16_matmul, w8a16_matmul
 
 
 class GraphDecoder:
-    def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int) -> None:
+    def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int,
+                 kv_dtype: torch.dtype | None = None) -> None:
         if max_len > model.context_length:
             raise ValueError(f"max_len {max_len} exceeds the model's context length {model.context_length}")
         self.model = model.eval()
@@ -27,7 +28,7 @@ class GraphDecoder:
         if device.type != "cuda":
             raise ValueError("GraphDecoder needs the model on a ROCm device")
         self.device = device
-        self.cache = model.new_cache(batch, max_len)
+        self.cache = model.new_cache(batch, max_len, dtype=kv_dtype)
         self.token = torch.zeros((batch, 1), dtype=torch.long, device=device)
         self.out = torch.zeros((batch, max_len), dtype=torch.long, device=device)
         self.step_index = torch.zeros(1, dtype=torch.long, device=device)
@@ -134,10 +135,16 @@ class FusedDecoder(GraphDecoder):
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
-    linear a QuantLinear."""
+    linear a QuantLinear.  ``kv_dtype``: torch.float32 (default, the model's own dtype) or
+    torch.bfloat16 (keys and values rounded to nearest even on write, half the cache traffic)."""
 
-    def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int) -> None:
-        super().__init__(model, batch, max_len)
+    def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int,
+                 kv_dtype: torch.dtype | None = None) -> None:
+        super().__init__(model, batch, max_len, kv_dtype)
+        cache_dtype = self.cache.keys[0].dtype
+        if cache_dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("the KV cache must be float32 or bfloat16")
+        self.kv_flag = _lib.AJQ_KV_F32 if cache_dtype == torch.float32 else _lib.AJQ_KV_BF16
         first = model.layers[0]
         ok = (
             model.position_encoding == "rope" and first.norm_placement == "pre"
@@ -193,11 +200,11 @@ class FusedDecoder(GraphDecoder):
             qkv = w["qkv"](self.normed)
             _lib.check(lib.ajq_rope_cache(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
                                           self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
-                                          self.cache.values[index].data_ptr(), b, self.heads, self.kv_heads, 128,
-                                          self.max_len, st), "rope_cache")
+                                          self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
+                                          self.kv_heads, 128, self.max_len, st), "rope_cache")
             _lib.check(lib.ajq_attn_decode(self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
-                                           self.cache.values[index].data_ptr(), pos.data_ptr(), b, self.heads,
-                                           self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
+                                           self.cache.values[index].data_ptr(), self.kv_flag, pos.data_ptr(), b,
+                                           self.heads, self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
                                            self.attn_ws.data_ptr(), self.attn_ws_bytes, st), "attn_decode")
             attn_out = w["o"](self.attended)
             _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), attn_out.data_ptr(), w["g2"].data_ptr(), w["eps2"],
@@ -212,10 +219,10 @@ class FusedDecoder(GraphDecoder):
 
 @torch.no_grad()
 def greedy_decode_graph(model: modeling.TransformerLM, prompt: torch.Tensor, max_new_tokens: int,
-                        fused: bool = False) -> torch.Tensor:
+                        fused: bool = False, kv_dtype: torch.dtype | None = None) -> torch.Tensor:
     """``[B, T + new]`` like ``modeling.greedy_decode``, with the per-token step replayed from a graph."""
     cls = FusedDecoder if fused else GraphDecoder
-    decoder = cls(model, prompt.shape[0], prompt.shape[1] + max_new_tokens)
+    decoder = cls(model, prompt.shape[0], prompt.shape[1] + max_new_tokens, kv_dtype)
     decoder.prefill(prompt)
     new = decoder.generate(max_new_tokens)
     return torch.cat((prompt.to(new.device), new), dim=1)

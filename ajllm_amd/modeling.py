@@ -222,9 +222,11 @@ class MultiHeadSelfAttention(nn.Module):
         if cache is not None and cache.static:
             # fixed-shape step: scatter the new row at the device-side position, attend over the
             # whole cache with the rows beyond that position masked out
-            cache.keys[layer_index].index_copy_(2, cache.position, k)
-            cache.values[layer_index].index_copy_(2, cache.position, v)
+            cache.keys[layer_index].index_copy_(2, cache.position, k.to(cache.keys[layer_index].dtype))
+            cache.values[layer_index].index_copy_(2, cache.position, v.to(cache.values[layer_index].dtype))
             k, v = cache.keys[layer_index], cache.values[layer_index]
+            if k.dtype != q.dtype:  # a cache kept in a narrower type: attention itself stays in q's
+                k, v = k.to(q.dtype), v.to(q.dtype)
             if self.num_kv_heads != self.num_heads:
                 rep = self.num_heads // self.num_kv_heads
                 k = k.repeat_interleave(rep, dim=1)
@@ -240,6 +242,8 @@ class MultiHeadSelfAttention(nn.Module):
             cache.values[layer_index][:, :, start:start + seq] = v
             k = cache.keys[layer_index][:, :, :start + seq]
             v = cache.values[layer_index][:, :, :start + seq]
+            if k.dtype != q.dtype:
+                k, v = k.to(q.dtype), v.to(q.dtype)
         total = start + seq
         if self.num_kv_heads != self.num_heads:
             rep = self.num_heads // self.num_kv_heads
@@ -374,7 +378,8 @@ def build_model(config: dict[str, Any], vocab_size: int) -> TransformerLM:
 
 @torch.no_grad()
 def greedy_decode(model: TransformerLM, prompt_tokens: torch.Tensor, max_new_tokens: int,
-                  eos_token_id: int | None = None, return_margins: bool = False):
+                  eos_token_id: int | None = None, return_margins: bool = False,
+                  kv_dtype: torch.dtype | None = None):
     """Batched greedy decoding with a KV cache.
 
     Same token rule as the reference's ``generate`` at temperature <= 0
@@ -386,7 +391,7 @@ def greedy_decode(model: TransformerLM, prompt_tokens: torch.Tensor, max_new_tok
     model.eval()
     tokens = prompt_tokens if prompt_tokens.dim() == 2 else prompt_tokens.reshape(1, -1)
     batch, prompt_len = tokens.shape
-    cache = model.new_cache(batch, prompt_len + max_new_tokens)
+    cache = model.new_cache(batch, prompt_len + max_new_tokens, dtype=kv_dtype)
     out = [tokens]
     margins = []
     done = torch.zeros(batch, dtype=torch.bool, device=tokens.device)

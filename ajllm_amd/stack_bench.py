@@ -63,7 +63,7 @@ def _eager_linear_seconds(model, rows: int, device) -> float:
 
 @torch.no_grad()
 def bench_stack(device, log=print, config: dict | None = None, batch: int = BATCH, context: int = CONTEXT,
-                decode_steps: int = 32, scheme: str = "w8a16") -> dict:
+                decode_steps: int = 32, scheme: str = "w8a16", kv_dtype: torch.dtype | None = None) -> dict:
     config = dict(config or CONFIG)
     t0 = time.perf_counter()
     model = build_quantized_model(device, scheme, seed=4321, config=config)
@@ -75,7 +75,7 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     prompt = torch.randint(0, config["vocab_size"], (batch, context), generator=g).to(device)
 
     # ---- prefill, PREFILL_ROWS sequences (PREFILL_ROWS * context tokens) per pass, into the decoder's cache
-    dec = decoding.FusedDecoder(model, batch, context + decode_steps + 8)
+    dec = decoding.FusedDecoder(model, batch, context + decode_steps + 8, kv_dtype)
     dec.prefill(prompt[:, :64], rows_per_pass=PREFILL_ROWS)  # warm-up: library load, allocator
     torch.cuda.synchronize()
     pass_times = []
@@ -130,8 +130,9 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
         st = torch.cuda.current_stream().cuda_stream
         for index in range(len(dec.layers)):
             _lib.check(lib.ajq_attn_decode(dec.q_rot.data_ptr(), dec.cache.keys[index].data_ptr(),
-                                           dec.cache.values[index].data_ptr(), dec.cache.position.data_ptr(), batch,
-                                           dec.heads, dec.kv_heads, 128, dec.max_len, dec.attended.data_ptr(),
+                                           dec.cache.values[index].data_ptr(), dec.kv_flag,
+                                           dec.cache.position.data_ptr(), batch, dec.heads, dec.kv_heads, 128,
+                                           dec.max_len, dec.attended.data_ptr(),
                                            dec.attn_ws.data_ptr(), dec.attn_ws_bytes, st), "attn_decode")
 
     t_attention = _graph_seconds(attention, stream)

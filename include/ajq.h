@@ -57,6 +57,10 @@ typedef enum ajq_status {
 #define AJQ_OUT_BF16 0
 #define AJQ_OUT_F32 1 /* same accumulation, final cast skipped (parity checks) */
 
+/* element type of the key/value caches of the decode-step operators */
+#define AJQ_KV_F32 0
+#define AJQ_KV_BF16 1 /* rounded to nearest even on write; attention still computes in fp32 */
+
 int ajq_version(void);
 const char* ajq_last_error(void);
 const char* ajq_status_string(int status);
@@ -105,7 +109,7 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                    void* y, int out_dtype, void* stream);
 
 /* ---- the small operators of one decode step around the linears -------------------
- * fp32 residual stream and KV cache; outputs that feed a linear are bf16.  `pos` is a
+ * fp32 residual stream; fp32 or bf16 KV cache (cache_dtype); outputs that feed a linear are bf16.  `pos` is a
  * DEVICE pointer to the step's cache row, so a recorded HIP graph replays per token. */
 
 /* hidden[B, D] += delta[B, D] (delta may be NULL), out = bf16(RMSNorm(hidden) * gain)
@@ -120,17 +124,17 @@ int ajq_add_rmsnorm(float* hidden, const float* delta, const float* gain, float 
  * src/ajllm/modeling/attention.py:36-60).  The reference has no KV cache
  * (src/ajllm/generation/generator.py:20-27 recomputes the sequence): the cache is this build's. */
 int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
-                   float* q_out, float* kcache, float* vcache, int B, int H, int Hkv, int head_dim,
-                   int max_len, void* stream);
+                   float* q_out, void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv,
+                   int head_dim, int max_len, void* stream);
 
 /* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
  * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
  * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of
  * them).  head_dim 128 only.  The workspace holds the partial results of up to 16 row chunks. */
 size_t ajq_attn_decode_workspace_bytes(int B, int H);
-int ajq_attn_decode(const float* q, const float* kcache, const float* vcache, const int64_t* pos,
-                    int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace,
-                    size_t workspace_bytes, void* stream);
+int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype,
+                    const int64_t* pos, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
+                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* ab[B, 2F] = (w1 x | w3 x) -> out[B, F] = bf16(silu(w1 x) * w3 x)
  * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */

@@ -166,15 +166,17 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         # RoPE + cache write, then attention over the cache
         att = modeling.MultiHeadSelfAttention(d, heads, 64, "rope", 10000.0, num_kv_heads=kv_heads).to(cuda)
         qkv = torch.randn((b, (heads + 2 * kv_heads) * hd), generator=g).to(cuda)
-        kc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda)
-        vc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda)
+        cache_dtype = torch.bfloat16 if b in (3, 32) else torch.float32  # both cache element types
+        kv_flag = _lib.AJQ_KV_BF16 if cache_dtype == torch.bfloat16 else _lib.AJQ_KV_F32
+        kc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
+        vc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
         for p in (0, 5, 39):
             pos = torch.tensor([p], device=cuda)
             q_rot = torch.empty((b, heads, hd), device=cuda)
             k2, v2 = kc.clone(), vc.clone()
             _lib.check(lib.ajq_rope_cache(qkv.data_ptr(), att.rope.cosine.data_ptr(), att.rope.sine.data_ptr(),
-                                          pos.data_ptr(), q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), b, heads,
-                                          kv_heads, hd, max_len, st), "rope_cache")
+                                          pos.data_ptr(), q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), kv_flag, b,
+                                          heads, kv_heads, hd, max_len, st), "rope_cache")
             q_in = qkv[:, : heads * hd].view(b, heads, 1, hd)
             k_in = qkv[:, heads * hd: (heads + kv_heads) * hd].view(b, kv_heads, 1, hd)
             v_in = qkv[:, (heads + kv_heads) * hd:].view(b, kv_heads, 1, hd)
@@ -182,17 +184,22 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
             q_want = att.rope(q_in, pp.expand(b, heads, 1))
             k_want = att.rope(k_in, pp.expand(b, kv_heads, 1))
             assert torch.allclose(q_rot, q_want[:, :, 0], atol=1e-6, rtol=1e-6)
-            assert torch.allclose(k2[:, :, p], k_want[:, :, 0], atol=1e-6, rtol=1e-6) and torch.equal(v2[:, :, p], v_in[:, :, 0])
+            if cache_dtype == torch.float32:
+                assert torch.allclose(k2[:, :, p], k_want[:, :, 0], atol=1e-6, rtol=1e-6)
+            else:  # the bf16 row is the rounding of the fp32 rotation (1 ulp where that sits on a tie)
+                assert (k2[:, :, p].float() - k_want[:, :, 0]).abs().max() <= 2 ** -7 * k_want.abs().max()
+            assert torch.equal(v2[:, :, p], v_in[:, :, 0].to(cache_dtype))
             untouched = torch.ones(max_len, dtype=torch.bool); untouched[p] = False
             assert torch.equal(k2[:, :, untouched], kc[:, :, untouched]) and torch.equal(v2[:, :, untouched], vc[:, :, untouched])
             ws_bytes = lib.ajq_attn_decode_workspace_bytes(b, heads)
             ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
             got = torch.empty((b, heads * hd), dtype=torch.bfloat16, device=cuda)
-            _lib.check(lib.ajq_attn_decode(q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), pos.data_ptr(), b, heads,
-                                           kv_heads, hd, max_len, got.data_ptr(), ws.data_ptr(), ws_bytes, st), "attn")
+            _lib.check(lib.ajq_attn_decode(q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), kv_flag, pos.data_ptr(), b,
+                                           heads, kv_heads, hd, max_len, got.data_ptr(), ws.data_ptr(), ws_bytes, st),
+                       "attn")
             rep = heads // kv_heads
-            keys = k2[:, :, : p + 1].repeat_interleave(rep, dim=1)
-            vals = v2[:, :, : p + 1].repeat_interleave(rep, dim=1)
+            keys = k2[:, :, : p + 1].float().repeat_interleave(rep, dim=1)
+            vals = v2[:, :, : p + 1].float().repeat_interleave(rep, dim=1)
             want_att = modeling.scaled_dot_product_attention(q_rot.unsqueeze(2), keys, vals)[:, :, 0].reshape(b, heads * hd)
             assert (got.float() - want_att).abs().max() <= 2e-2 and errors(got, want_att.cpu())[1] <= 3e-3
         # SwiGLU gate
@@ -203,9 +210,10 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         assert errors(got_g, want_g.cpu())[1] <= 3e-3
 
 
-@pytest.mark.parametrize("scheme,batch,kv_heads", [("w4a16_g128", 1, 2), ("w4a16_g128", 5, 2), ("w8a16", 2, 2),
-                                                   ("w8a16", 32, 1), ("w4a16_g128", 20, 1)])
-def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads):
+@pytest.mark.parametrize("scheme,batch,kv_heads,kv_dtype", [
+    ("w4a16_g128", 1, 2, None), ("w4a16_g128", 5, 2, None), ("w8a16", 2, 2, None), ("w8a16", 32, 1, None),
+    ("w4a16_g128", 20, 1, None), ("w4a16_g128", 3, 2, torch.bfloat16), ("w8a16", 24, 1, torch.bfloat16)])
+def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_dtype):
     """The all-kernel decode step (FusedDecoder) against the eager model loop, replayed from a
     graph; differences only below the eager run's own logit-margin noise.  Batches above 16 take
     the batched-decode matmul; one key/value head under two query heads is grouped-query attention."""
@@ -214,8 +222,8 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads):
                                    d_ff=640, num_kv_heads=kv_heads).eval()
     fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
     prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(10)).to(cuda)
-    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True)
-    dec = decoding.FusedDecoder(fast, batch, 60)
+    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True, kv_dtype=kv_dtype)
+    dec = decoding.FusedDecoder(fast, batch, 60, kv_dtype)
     dec.prefill(prompt, rows_per_pass=8 if batch > 16 else None)
     first = dec.generate(10)
     torch.cuda.synchronize()
@@ -232,7 +240,7 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads):
         dec.generate(step)
         with torch.no_grad():
             fused_logits = dec._logits()[row].float()
-            eager_logits = fast(eager[row:row + 1, : 20 + step])[0, -1].float()
+            eager_logits = fast(eager[row:row + 1, : 20 + step], fast.new_cache(1, 60, dtype=kv_dtype))[0, -1].float()
         gap = float((fused_logits - eager_logits).abs().max())
         print("row", row, "step", step, "eager margin", margin, "logit difference", gap)
         assert gap <= 1e-2 and margin <= 2 * gap, (row, step, margin, gap)
@@ -240,7 +248,7 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads):
     dec.prefill(prompt)
     with torch.no_grad():
         logits_fused = dec._logits()
-        cache = fast.new_cache(batch, 60)
+        cache = fast.new_cache(batch, 60, dtype=kv_dtype)
         fast(prompt, cache)
         logits_eager = fast(dec.token, cache)[:, -1, :]
     max_abs, rel = errors(logits_fused, logits_eager.cpu())
