@@ -287,7 +287,8 @@ int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const
   auto kernel = dequant_skinny_kernel<kWaves, TPW, MROWS, NT, kW4>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   const int ntiles = N / kTileN;
-  hipLaunchKernelGGL(kernel, dim3((ntiles + NT - 1) / NT, (M + MROWS - 1) / MROWS), dim3(kWaves * 64), lds, stream,
+  const int ngroups = (ntiles + NT - 1) / NT, mblocks = (M + MROWS - 1) / MROWS;
+  hipLaunchKernelGGL(kernel, dim3(8 * ((ngroups + 7) / 8) * mblocks), dim3(kWaves * 64), lds, stream,
                      reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32, scales8);
   return AJQ_OK;
 }
@@ -296,7 +297,7 @@ int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
 
-// 17 <= M < 256.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup: as
+// M >= 17.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup: as
 // many as still leave a workgroup for every CU.  (Wider row blocks lose to more row tiles: a
 // workgroup's traffic is K * (2 * rows + bytes per weight * 16 * tiles) for rows * 16 * tiles
 // outputs.)
@@ -311,6 +312,19 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
   if (nt == 1) return launch_skinny_cfg<2, 32, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (nt == 2) return launch_skinny_cfg<1, 32, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   return launch_skinny_cfg<1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+}
+
+// M >= 256: the 256 x 128 tile kernel needs about a workgroup per CU to be worth its long K
+// loop; below that the weight-streaming kernel is faster.  Both times are modelled from
+// measurements: a k-block of the tile kernel takes about 1.8 us per round of 256 workgroups,
+// the streaming kernel sustains about 370 TFLOP/s for M >= 256.
+bool streaming_kernel_is_faster(int M, int N, int K) {
+  if (M < kGemm256MinM) return true;
+  const double tiles = (double)((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
+  const double rounds = (double)(long long)((tiles + 255) / 256);
+  const double us_tiles = rounds * (K / kGroup) * 1.8 + 3.0;
+  const double us_stream = 2.0 * M * N * (double)K / 370e6;
+  return us_stream < us_tiles;
 }
 
 }  // namespace
@@ -345,7 +359,7 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                    int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   if (int s = check_matmul_args("ajq_w4a16_gemm", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
   const bool out_f32 = out_dtype == AJQ_OUT_F32;
-  if (M < kGemm256MinM) {
+  if (streaming_kernel_is_faster(M, N, K)) {
     const int s = M <= kMaxGemvM ? launch_gemv<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream)
                                  : launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream);
     return s ? s : check_launch("ajq_w4a16_gemm");
@@ -369,7 +383,7 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                    int out_dtype, void* stream) {
   if (int s = check_matmul_args("ajq_w8a16_gemm", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
   const bool out_f32 = out_dtype == AJQ_OUT_F32;
-  if (M < kGemm256MinM) {
+  if (streaming_kernel_is_faster(M, N, K)) {
     const int s = M <= kMaxGemvM ? launch_gemv<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream)
                                  : launch_skinny<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream);
     return s ? s : check_launch("ajq_w8a16_gemm");

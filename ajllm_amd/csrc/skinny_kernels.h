@@ -50,9 +50,18 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int nl = lane & 15, kc = lane >> 4;
-  const int nt0 = blockIdx.x * NT;
+  // Workgroup -> (row-tile group, row block).  Workgroups are dealt to the 8 XCDs round-robin
+  // by index, and each XCD has its own L2: the row blocks of one row-tile group, which read
+  // the same weights, are given consecutive slots of ONE XCD, so the weights come out of HBM
+  // once and the other row blocks find them in that L2.
   const int ntiles = N / kTileN;
-  const int m0 = blockIdx.y * MROWS;
+  const int ngroups = (ntiles + NT - 1) / NT;
+  const int mblocks = (M + MROWS - 1) / MROWS;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int ng = xcd + 8 * (slot / mblocks);
+  if (ng >= ngroups) return;  // padding of the last round (whole workgroup: no barrier is left waiting)
+  const int nt0 = ng * NT;
+  const int m0 = (slot % mblocks) * MROWS;
   const int G = K >> 7;
   constexpr int kRegion = MROWS * kStride;  // bf16 elements of one wave's region
   uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * kRegion;
