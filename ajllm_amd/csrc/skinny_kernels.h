@@ -31,7 +31,7 @@ struct SkinnyBatch {
 };
 
 template <int kWaves, int TPW, int MROWS, int NT, bool kW4>
-__global__ __launch_bounds__(kWaves * 64) void dequant_skinny_kernel(
+__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_kernel(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
