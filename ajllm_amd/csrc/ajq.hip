@@ -413,12 +413,23 @@ int attn_splits(int B, int Hkv) {
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
 }
 
-template <int R, typename CacheT>
-void launch_attn(const float* q, const void* kcache, const void* vcache, const long long* pos, int B, int H, int Hkv,
-                 int max_len, float scale, int S, float* partial, uint16_t* out, hipStream_t stream) {
-  hipLaunchKernelGGL((attn_decode_kernel<R, CacheT>), dim3(B * Hkv, S), dim3(256), 0, stream, q,
-                     reinterpret_cast<const CacheT*>(kcache), reinterpret_cast<const CacheT*>(vcache), pos, H, Hkv,
-                     max_len, scale, partial, out);
+template <int R, typename CacheT, bool kStep>
+void launch_attn(const float* q, void* kcache, void* vcache, const long long* pos, int B, int H, int Hkv, int max_len,
+                 float scale, int S, float* partial, uint16_t* out, const float* cosine, const float* sine,
+                 hipStream_t stream) {
+  hipLaunchKernelGGL((attn_decode_kernel<R, CacheT, kStep>), dim3(B * Hkv, S), dim3(256), 0, stream, q,
+                     reinterpret_cast<CacheT*>(kcache), reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale,
+                     partial, out, cosine, sine);
+  if (S > 1)
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, stream, partial, S, out);
+}
+
+template <bool kStep>
+auto pick_attn(int R, int cache_dtype) {
+  if (cache_dtype == AJQ_KV_F32)
+    return R == 1 ? launch_attn<1, float, kStep> : R == 2 ? launch_attn<2, float, kStep> : launch_attn<4, float, kStep>;
+  return R == 1 ? launch_attn<1, uint16_t, kStep>
+                : R == 2 ? launch_attn<2, uint16_t, kStep> : launch_attn<4, uint16_t, kStep>;
 }
 }  // namespace
 
@@ -483,15 +494,41 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
   if (!aligned16(kcache) || !aligned16(vcache) || !aligned16(q))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_decode: q and the caches must be 16-byte aligned");
-  auto launch = cache_dtype == AJQ_KV_F32
-                    ? (R == 1 ? launch_attn<1, float> : R == 2 ? launch_attn<2, float> : launch_attn<4, float>)
-                    : (R == 1 ? launch_attn<1, uint16_t> : R == 2 ? launch_attn<2, uint16_t> : launch_attn<4, uint16_t>);
-  launch(q, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len, scale, S,
-         reinterpret_cast<float*>(workspace), out, (hipStream_t)stream);
-  if (S > 1)
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, (hipStream_t)stream,
-                       reinterpret_cast<const float*>(workspace), S, out);
+  pick_attn<false>(R, cache_dtype)(q, const_cast<void*>(kcache), const_cast<void*>(vcache),
+                                   reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len, scale, S,
+                                   reinterpret_cast<float*>(workspace), out, nullptr, nullptr, (hipStream_t)stream);
   return check_launch("ajq_attn_decode");
+}
+
+size_t ajq_attn_step_workspace_bytes(int B, int H) {
+  if (B < 1 || H < 1) return 0;
+  return ajq_attn_decode_workspace_bytes(B, H);
+}
+
+int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, void* kcache,
+                  void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+  if (!qkv || !cosine || !sine || !pos || !kcache || !vcache || !out)
+    return fail(AJQ_ERR_NULL, "ajq_attn_step: null pointer argument");
+  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: head_dim %d (only 128 is built)", head_dim);
+  if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
+    return fail(AJQ_ERR_SHAPE, "ajq_attn_step: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
+  const int R = H / Hkv;
+  if (R != 1 && R != 2 && R != 4)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: %d query heads per cache head (1, 2 and 4 are built)", R);
+  if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+  if (!aligned16(qkv) || !aligned16(cosine) || !aligned16(sine) || !aligned16(kcache) || !aligned16(vcache))
+    return fail(AJQ_ERR_ALIGN, "ajq_attn_step: qkv, the tables and the caches must be 16-byte aligned");
+  const int S = attn_splits(B, Hkv);
+  if (S > 1 && (!workspace || workspace_bytes < ajq_attn_step_workspace_bytes(B, H) || !aligned16(workspace)))
+    return fail(AJQ_ERR_WORKSPACE, "ajq_attn_step: 16-byte aligned workspace of %zu bytes needed, %zu given",
+                ajq_attn_step_workspace_bytes(B, H), workspace_bytes);
+  const float scale = 1.0f / sqrtf((float)head_dim);
+  pick_attn<true>(R, cache_dtype)(qkv, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len,
+                                  scale, S, reinterpret_cast<float*>(workspace), out, cosine, sine,
+                                  (hipStream_t)stream);
+  return check_launch("ajq_attn_step");
 }
 
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream) {

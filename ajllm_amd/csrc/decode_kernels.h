@@ -122,26 +122,71 @@ __device__ __forceinline__ KvRow8 load_row8(const uint16_t* p) {
   return r;
 }
 
-template <int R, typename CacheT>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
-                                                          const CacheT* __restrict__ vcache,
+// kStep: the whole attention part of a decode step in one launch.  `q` is then the fused
+// projection output qkv [B, (H + 2 Hkv) * 128] (query heads, key heads, value heads): the
+// workgroup rotates its R query heads itself (interleaved pairs, the tables' row *pos); the
+// workgroup whose chunk holds row *pos also rotates the new key, writes it and the new value
+// into the caches and attends to them from registers.  (Merging the S partial results in the
+// workgroup that finishes last was tried and lost: the device-scope fences it needs write back
+// and invalidate the XCD's L2, several microseconds per launch; the merge stays a launch.)
+__device__ __forceinline__ void rotate4(float4& v, const float4 c, const float4 s) {
+  // pairs (x, y) and (z, w) with the angles of c.x/s.x and c.y/s.y
+  v = float4{v.x * c.x - v.y * s.x, v.x * s.x + v.y * c.x, v.z * c.y - v.w * s.y, v.z * s.y + v.w * c.y};
+}
+__device__ __forceinline__ void store_row8(float* p, float4& a, float4& b) {
+  reinterpret_cast<float4*>(p)[0] = a;
+  reinterpret_cast<float4*>(p)[1] = b;
+}
+__device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
+  // rounds to bf16 and hands the rounded values back: what a later read of the cache would give
+  u32x4_t v;
+  v.x = f32_to_bf16_rne(a.x) | ((uint32_t)f32_to_bf16_rne(a.y) << 16);
+  v.y = f32_to_bf16_rne(a.z) | ((uint32_t)f32_to_bf16_rne(a.w) << 16);
+  v.z = f32_to_bf16_rne(b.x) | ((uint32_t)f32_to_bf16_rne(b.y) << 16);
+  v.w = f32_to_bf16_rne(b.z) | ((uint32_t)f32_to_bf16_rne(b.w) << 16);
+  *reinterpret_cast<u32x4_t*>(p) = v;
+  a = float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u), __uint_as_float(v.y << 16),
+             __uint_as_float(v.y & 0xFFFF0000u)};
+  b = float4{__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xFFFF0000u), __uint_as_float(v.w << 16),
+             __uint_as_float(v.w & 0xFFFF0000u)};
+}
+
+template <int R, typename CacheT, bool kStep>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, CacheT* __restrict__ kcache,
+                                                          CacheT* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
-                                                          float scale, float* __restrict__ partial,
-                                                          uint16_t* __restrict__ out) {
+                                                          float scale, float* __restrict__ partial, uint16_t* __restrict__ out,
+                                                          const float* __restrict__ cosine,
+                                                          const float* __restrict__ sine) {
   constexpr int hd = 128;
   const int bk = blockIdx.x, S = gridDim.y, s = blockIdx.y;
   const int b = bk / Hkv, hk = bk % Hkv;
   const int bh0 = b * H + hk * R;  // first of the R query heads
   const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // 16 teams of 16 lanes
-  const int rows = (int)(*pos) + 1;
+  const long long p = *pos;
+  const int rows = (int)p + 1;
   const int per = (rows + S - 1) / S;
-  const int t_begin = s * per, t_end = min(rows, t_begin + per);
+  const int t_begin = s * per;
+  int t_end = min(rows, t_begin + per);
   float4 qa[R], qb[R];
+  float4 ca, cb, sa, sb;  // kStep: cosines / sines of this lane's four pairs, two per float4 half
+  const float* qkv_row = q + (size_t)b * (H + 2 * Hkv) * hd + 8 * c;  // kStep only
+  if (kStep) {
+    const float4 c4 = *reinterpret_cast<const float4*>(cosine + p * (hd / 2) + 4 * c);
+    const float4 s4 = *reinterpret_cast<const float4*>(sine + p * (hd / 2) + 4 * c);
+    ca = float4{c4.x, c4.y, 0.f, 0.f}; cb = float4{c4.z, c4.w, 0.f, 0.f};
+    sa = float4{s4.x, s4.y, 0.f, 0.f}; sb = float4{s4.z, s4.w, 0.f, 0.f};
+  }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float4* q4 = reinterpret_cast<const float4*>(q + (size_t)(bh0 + r) * hd + 8 * c);
+    const float4* q4 = reinterpret_cast<const float4*>(kStep ? qkv_row + (size_t)(hk * R + r) * hd
+                                                             : q + (size_t)(bh0 + r) * hd + 8 * c);
     qa[r] = q4[0];
     qb[r] = q4[1];
+    if (kStep) {
+      rotate4(qa[r], ca, sa);
+      rotate4(qb[r], cb, sb);
+    }
   }
   const CacheT* kbase = kcache + (size_t)bk * max_len * hd + 8 * c;
   const CacheT* vbase = vcache + (size_t)bk * max_len * hd + 8 * c;
@@ -172,6 +217,20 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
       m[r] = m_new;
     }
   };
+  if (kStep && t_begin <= (int)p && (int)p < t_end) {
+    // the step's own row: rotate the key, store both, attend from registers (team 0)
+    t_end = (int)p;
+    if (team == 0) {
+      const float4* k4 = reinterpret_cast<const float4*>(qkv_row + (size_t)(H + hk) * hd);
+      const float4* v4 = reinterpret_cast<const float4*>(qkv_row + (size_t)(H + Hkv + hk) * hd);
+      float4 ka = k4[0], kb = k4[1], va = v4[0], vb = v4[1];
+      rotate4(ka, ca, sa);
+      rotate4(kb, cb, sb);
+      store_row8(kcache + ((size_t)bk * max_len + p) * hd + 8 * c, ka, kb);
+      store_row8(vcache + ((size_t)bk * max_len + p) * hd + 8 * c, va, vb);
+      row(ka, kb, va, vb);
+    }
+  }
   int t = t_begin + team;
   for (; t + 16 < t_end; t += 32) {  // two rows per team in flight
     const KvRow8 k0 = load_row8(kbase + (size_t)t * hd), k1 = load_row8(kbase + (size_t)(t + 16) * hd);

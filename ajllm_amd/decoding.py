@@ -129,9 +129,9 @@ class _FusedLinear:
 
 class FusedDecoder(GraphDecoder):
     """GraphDecoder whose step runs on this library's kernels only: fused q|k|v and w1|w3
-    matmuls, residual add + RMSNorm, RoPE + cache write, single-query attention and the SwiGLU
-    gate (``ajq_add_rmsnorm`` / ``ajq_rope_cache`` / ``ajq_attn_decode`` / ``ajq_swiglu``), plus
-    the embedding lookup and the argmax from PyTorch.  About ten launches per layer.
+    matmuls, residual add + RMSNorm, RoPE + cache write + single-query attention in one launch
+    and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), plus the
+    embedding lookup and the argmax from PyTorch.  Nine launches per layer (eight where the attention needs no merge).
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
@@ -181,11 +181,10 @@ class FusedDecoder(GraphDecoder):
         self.embedding = model.token_embeddings.weight.detach()
         self.hidden = torch.zeros((batch, d), dtype=torch.float32, device=dev)
         self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
-        self.q_rot = torch.zeros((batch, self.heads, 128), dtype=torch.float32, device=dev)
         self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)
         lib = _lib.load()
-        self.attn_ws_bytes = int(lib.ajq_attn_decode_workspace_bytes(batch, self.heads))
+        self.attn_ws_bytes = int(lib.ajq_attn_step_workspace_bytes(batch, self.heads))
         self.attn_ws = torch.zeros(max(self.attn_ws_bytes, 16), dtype=torch.uint8, device=dev)
 
     def _logits(self) -> torch.Tensor:
@@ -198,14 +197,11 @@ class FusedDecoder(GraphDecoder):
             _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), delta.data_ptr() if delta is not None else None,
                                            w["g1"].data_ptr(), w["eps1"], self.normed.data_ptr(), b, d, st), "add_rmsnorm")
             qkv = w["qkv"](self.normed)
-            _lib.check(lib.ajq_rope_cache(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
-                                          self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
-                                          self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
-                                          self.kv_heads, 128, self.max_len, st), "rope_cache")
-            _lib.check(lib.ajq_attn_decode(self.q_rot.data_ptr(), self.cache.keys[index].data_ptr(),
-                                           self.cache.values[index].data_ptr(), self.kv_flag, pos.data_ptr(), b,
-                                           self.heads, self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
-                                           self.attn_ws.data_ptr(), self.attn_ws_bytes, st), "attn_decode")
+            _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
+                                         self.cache.keys[index].data_ptr(), self.cache.values[index].data_ptr(),
+                                         self.kv_flag, b, self.heads, self.kv_heads, 128, self.max_len,
+                                         self.attended.data_ptr(), self.attn_ws.data_ptr(), self.attn_ws_bytes, st),
+                       "attn_step")
             attn_out = w["o"](self.attended)
             _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), attn_out.data_ptr(), w["g2"].data_ptr(), w["eps2"],
                                            self.normed.data_ptr(), b, d, st), "add_rmsnorm")

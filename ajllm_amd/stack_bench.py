@@ -126,14 +126,16 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     from . import _lib
     lib = _lib.load()
 
+    qkv = torch.randn((batch, (dec.heads + 2 * dec.kv_heads) * 128), device=device)
+
     def attention():
         st = torch.cuda.current_stream().cuda_stream
-        for index in range(len(dec.layers)):
-            _lib.check(lib.ajq_attn_decode(dec.q_rot.data_ptr(), dec.cache.keys[index].data_ptr(),
-                                           dec.cache.values[index].data_ptr(), dec.kv_flag,
-                                           dec.cache.position.data_ptr(), batch, dec.heads, dec.kv_heads, 128,
-                                           dec.max_len, dec.attended.data_ptr(),
-                                           dec.attn_ws.data_ptr(), dec.attn_ws_bytes, st), "attn_decode")
+        for index, w in enumerate(dec.layers):
+            _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
+                                         dec.cache.position.data_ptr(), dec.cache.keys[index].data_ptr(),
+                                         dec.cache.values[index].data_ptr(), dec.kv_flag, batch, dec.heads,
+                                         dec.kv_heads, 128, dec.max_len, dec.attended.data_ptr(),
+                                         dec.attn_ws.data_ptr(), dec.attn_ws_bytes, st), "attn_step")
 
     t_attention = _graph_seconds(attention, stream)
     kv_bytes = 2 * len(dec.layers) * batch * dec.kv_heads * (context + decode_steps // 2) * 128 * dec.cache.keys[0].element_size()

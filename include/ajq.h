@@ -136,6 +136,13 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
                     const int64_t* pos, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* The two operators above in one kernel: qkv as for ajq_rope_cache; the step's key and value
+ * rows are written to row *pos of the caches and attended to from registers. */
+size_t ajq_attn_step_workspace_bytes(int B, int H);
+int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
+                  void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
+                  int max_len, uint16_t* out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ab[B, 2F] = (w1 x | w3 x) -> out[B, F] = bf16(silu(w1 x) * w3 x)
  * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);

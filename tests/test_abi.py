@@ -70,8 +70,9 @@ def test_shape_alignment_and_option_errors():
     assert need == 4 * 300 * 16                                             # G=4 groups x 300 rows x 16 bytes
     assert lib.ajq_w4a16_gemm_workspace_bytes(255, 512) == 0                 # below 256 rows no workspace is used
     assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 2, 128, 8, p, p, 1 << 20, None) == -4  # 8 query heads per cache head
-    assert lib.ajq_w4a16_gemm(p, 300, 512, p, p, 16, p, 0, None, 0, None) == -6
-    assert lib.ajq_w4a16_gemm(p, 300, 512, p, p, 16, p, 0, p, need - 1, None) == -6
+    need = lib.ajq_w4a16_gemm_workspace_bytes(2048, 4096)                    # a shape the tile kernel takes
+    assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, None, 0, None) == -6
+    assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, p, need - 1, None) == -6
     with pytest.raises(ValueError):
         _lib.check(-6, "probe")
     with pytest.raises(RuntimeError):

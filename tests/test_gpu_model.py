@@ -202,6 +202,23 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
             vals = v2[:, :, : p + 1].float().repeat_interleave(rep, dim=1)
             want_att = modeling.scaled_dot_product_attention(q_rot.unsqueeze(2), keys, vals)[:, :, 0].reshape(b, heads * hd)
             assert (got.float() - want_att).abs().max() <= 2e-2 and errors(got, want_att.cpu())[1] <= 3e-3
+            # the same step as one launch: same cache rows, same attention output (the step's own
+            # row enters the running softmax first instead of last: rounding differs, nothing else)
+            k3, v3 = kc.clone(), vc.clone()
+            ws3_bytes = lib.ajq_attn_step_workspace_bytes(b, heads)
+            ws3 = torch.zeros(max(ws3_bytes, 16), dtype=torch.uint8, device=cuda)
+            for _ in range(2):
+                got3 = torch.zeros((b, heads * hd), dtype=torch.bfloat16, device=cuda)
+                _lib.check(lib.ajq_attn_step(qkv.data_ptr(), att.rope.cosine.data_ptr(), att.rope.sine.data_ptr(),
+                                             pos.data_ptr(), k3.data_ptr(), v3.data_ptr(), kv_flag, b, heads, kv_heads,
+                                             hd, max_len, got3.data_ptr(), ws3.data_ptr(), ws3_bytes, st), "attn_step")
+                assert torch.equal(v3, v2)
+                if cache_dtype == torch.float32:  # the two kernels may contract the rotation's FMAs differently
+                    assert torch.allclose(k3, k2, atol=1e-6, rtol=1e-6)
+                else:
+                    assert (k3.float() - k2.float()).abs().max() <= 2 ** -7 * k2.float().abs().max()
+                assert (got3.float() - want_att).abs().max() <= 2e-2 and errors(got3, want_att.cpu())[1] <= 3e-3
+                assert (got3.float() - got.float()).abs().max() <= 2 ** -6
         # SwiGLU gate
         ab = torch.randn((b, 2 * ff), generator=g).to(cuda) * 3
         want_g = (modeling.silu(ab[:, :ff]) * ab[:, ff:]).to(torch.bfloat16)
