@@ -48,6 +48,19 @@ SIGNATURES: dict[str, tuple] = {
          c_int, c_void_p],
     ),
     "ajq_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "ajq_gemv_fused_supported": (c_int, [c_int, c_int]),
+    "ajq_w4a16_gemv_norm": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
+         c_void_p],
+    ),
+    "ajq_w8a16_gemv_norm": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
+         c_void_p],
+    ),
+    "ajq_w4a16_gemv_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ajq_w8a16_gemv_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_attn_step_workspace_bytes": (c_size_t, [c_int, c_int]),
     "ajq_attn_step": (
         c_int,

@@ -6,6 +6,7 @@
 
 #include "quantize_kernels.h"
 #include "gemv_kernels.h"
+#include "gemv_fused_kernels.h"
 #include "gemm_kernels.h"
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
@@ -317,6 +318,67 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
   return launch_skinny_cfg<8, 1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
+// ---- GEMV with the activations produced on the way in (norm / gate prologue)
+template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
+int launch_gemv_pro_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
+                        int out_f32, const float* src0, const float* src1, const float* gain, float eps, float* h_out,
+                        hipStream_t stream) {
+  constexpr size_t lds = gemv_pro_lds_bytes(kWaves, TPW, MROWS);
+  static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
+  auto kernel = dequant_gemv_pro_kernel<kWaves, TPW, MROWS, kW4, kPro>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
+                     meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out);
+  return AJQ_OK;
+}
+
+// K = waves * TPW * 128 for (8, 1), (8, 2), (8, 4), (11, 4) waves x groups; the row bound times
+// TPW stays <= 32 (eight loads of fp32 sources per lane: more would not fit the registers).
+bool gemv_pro_supported(int M, int K) {
+  if (M < 1) return false;
+  if (K == 1024) return M <= 16;
+  if (K == 2048) return M <= 16;
+  if (K == 4096 || K == 5632) return M <= 8;
+  return false;
+}
+
+template <bool kW4, int kPro>
+int launch_gemv_pro(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
+                    int out_f32, const float* src0, const float* src1, const float* gain, float eps, float* h_out,
+                    hipStream_t stream) {
+#define AJQ_PRO(W, T, R) \
+  return launch_gemv_pro_cfg<W, T, R, kW4, kPro>(M, K, wq, meta, scales8, N, y, out_f32, src0, src1, gain, eps, h_out, stream)
+  if (K == 1024) {
+    if (M <= 1) AJQ_PRO(8, 1, 1);
+    if (M <= 4) AJQ_PRO(8, 1, 4);
+    if (M <= 8) AJQ_PRO(8, 1, 8);
+    AJQ_PRO(8, 1, 16);
+  }
+  if (K == 2048) {
+    if (M <= 1) AJQ_PRO(8, 2, 1);
+    if (M <= 4) AJQ_PRO(8, 2, 4);
+    if (M <= 8) AJQ_PRO(8, 2, 8);
+    AJQ_PRO(8, 2, 16);
+  }
+  if (K == 4096) {
+    if (M <= 1) AJQ_PRO(8, 4, 1);
+    if (M <= 4) AJQ_PRO(8, 4, 4);
+    AJQ_PRO(8, 4, 8);
+  }
+  if (M <= 1) AJQ_PRO(11, 4, 1);
+  if (M <= 4) AJQ_PRO(11, 4, 4);
+  AJQ_PRO(11, 4, 8);
+#undef AJQ_PRO
+}
+
+int check_pro(const char* name, int M, int K, const void* a, const void* b) {
+  if (!gemv_pro_supported(M, K))
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d is not built (ajq_gemv_fused_supported)", name, M, K);
+  if (!a || !aligned16(a) || (b && !aligned16(b)))
+    return fail(a ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: the fp32 sources must be non-null and 16-byte aligned", name);
+  return AJQ_OK;
+}
+
 // M >= 256: the 256 x 128 tile kernel needs about a workgroup per CU to be worth its long K
 // loop; below that the weight-streaming kernel is faster.  Both times are modelled from
 // measurements: a k-block of the tile kernel takes about 1.8 us per round of 256 workgroups,
@@ -350,6 +412,52 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   if (int s = launch_gemv<false>(x, M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemv");
+}
+
+int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1 : 0; }
+
+int ajq_w4a16_gemv_norm(const float* h_in, const float* delta, const float* gain, float eps, float* h_out, int M, int K,
+                        const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemv_norm", h_in, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  if (int s = check_pro("ajq_w4a16_gemv_norm", M, K, gain, delta)) return s;
+  if (!h_out || !aligned16(h_out) || h_out == h_in)
+    return fail(AJQ_ERR_NULL, "ajq_w4a16_gemv_norm: h_out must be a 16-byte aligned buffer other than h_in");
+  if (int s = launch_gemv_pro<true, kProNorm>(M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, h_in, delta, gain,
+                                              eps, h_out, (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w4a16_gemv_norm");
+}
+
+int ajq_w8a16_gemv_norm(const float* h_in, const float* delta, const float* gain, float eps, float* h_out, int M, int K,
+                        const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemv_norm", h_in, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
+  if (int s = check_pro("ajq_w8a16_gemv_norm", M, K, gain, delta)) return s;
+  if (!h_out || !aligned16(h_out) || h_out == h_in)
+    return fail(AJQ_ERR_NULL, "ajq_w8a16_gemv_norm: h_out must be a 16-byte aligned buffer other than h_in");
+  if (int s = launch_gemv_pro<false, kProNorm>(M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, h_in, delta,
+                                               gain, eps, h_out, (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w8a16_gemv_norm");
+}
+
+int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                        int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemv_gate", ab, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  if (int s = check_pro("ajq_w4a16_gemv_gate", M, K, ab, nullptr)) return s;
+  if (int s = launch_gemv_pro<true, kProGate>(M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, ab, nullptr,
+                                              nullptr, 0.f, nullptr, (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w4a16_gemv_gate");
+}
+
+int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                        int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemv_gate", ab, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
+  if (int s = check_pro("ajq_w8a16_gemv_gate", M, K, ab, nullptr)) return s;
+  if (int s = launch_gemv_pro<false, kProGate>(M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, ab, nullptr,
+                                               nullptr, 0.f, nullptr, (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w8a16_gemv_gate");
 }
 
 // --------------------------------------------------------------- GEMM -----

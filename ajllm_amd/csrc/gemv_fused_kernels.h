@@ -1,0 +1,243 @@
+// Decode GEMV whose activations are produced on the way in (1 <= M <= 16,
+// K == kWaves * TPW * 128):
+//   kPro == kProNorm:  x = bf16( RMSNorm(h + delta) * gain ),  h + delta also written out
+//                      (the residual update and the norm in front of q|k|v and w1|w3);
+//   kPro == kProGate:  x = bf16( silu(a) * u ) for ab = (a | u)  (the SwiGLU gate in front of w2).
+// The matmul is dequant_gemv_kernel's straight-line variant: one workgroup per 16-row tile of
+// N, wave w owns k groups [w * TPW, (w + 1) * TPW), weight loads first.  What changes is where
+// a wave's k-slice of the activations comes from: it loads the fp32 sources of its slice (every
+// workgroup repeats that work; the sources are a few KB and sit in L2), forms the bf16 values
+// in registers and stages them in its private LDS rows as before.  The norm needs the whole
+// row's sum of squares: every wave reduces its slice per row, the eight partial sums meet in
+// LDS behind one barrier (the weight loads are in flight meanwhile).  Workgroup 0 writes the
+// updated residual stream, to a buffer other than the one being read.
+#pragma once
+#include "gemv_kernels.h"
+
+namespace ajq {
+
+constexpr int kProNorm = 1, kProGate = 2;
+
+template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
+__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
+    const u32x4_t* __restrict__ wq,
+    const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
+    int K,
+    int m_flags,  // M | out_f32 << 8
+    int N, void* __restrict__ y,
+    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
+    const float* __restrict__ src0,        // norm: h_in [M, K];  gate: ab [M, 2K]
+    const float* __restrict__ src1,        // norm: delta [M, K] or nullptr
+    const float* __restrict__ gain,        // norm: [K]
+    float eps,                             // norm
+    float* __restrict__ h_out) {           // norm: h_in + delta [M, K]; must not alias h_in
+  const int M = m_flags & 0xFF;
+  const bool out_f32 = (m_flags >> 8) != 0;
+  constexpr int kSlice = TPW * kGroup;
+  constexpr int kStride = kSlice + 8;
+  constexpr int kVecPerRow = kSlice / 8;  // 16 (TPW 1), 32 or 64 lanes hold one row's slice
+  constexpr int kVecs = MROWS * kVecPerRow;
+  constexpr int kXLoads = (kVecs + 63) / 64;
+  constexpr int kLoadsPerGroup = kW4 ? 1 : 2;
+  constexpr int kRowQuads = (MROWS + 3) / 4;
+  static_assert(kVecPerRow <= 64, "a row's slice must fit one wave-wide load");
+
+  extern __shared__ u32x4_t smem_raw[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int nl = lane & 15, kc = lane >> 4;
+  const int nt = blockIdx.x;
+  const int G = K >> 7;
+  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * (MROWS * kStride);
+  float* red = reinterpret_cast<float*>(reinterpret_cast<uint16_t*>(smem_raw) + kWaves * (MROWS * kStride));
+  float* ssq = red + kWaves * 64 * 4;  // [MROWS][kWaves] partial sums of squares
+  const int g0 = wave * TPW;
+
+  // ---- loads: weights first, then the fp32 sources of this wave's activation slice, then meta
+  u32x4_t w[TPW][kLoadsPerGroup];
+  uint32_t mw[TPW];
+  float4 a0[kXLoads][2], a1[kXLoads][2], a2[kXLoads][2];
+  __builtin_amdgcn_sched_barrier(0);
+  {
+    const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
+#pragma unroll
+    for (int p = 0; p < TPW; ++p)
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        w[p][h] = __builtin_nontemporal_load(wtile + (p * kLoadsPerGroup + h) * 64);
+  }
+#pragma unroll
+  for (int i = 0; i < kXLoads; ++i) {
+    const int v = min(lane + 64 * i, kVecs - 1);
+    const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
+    const int k = g0 * kGroup + 8 * c;
+    if (kPro == kProNorm) {
+      const float4* ph = reinterpret_cast<const float4*>(src0 + (size_t)m * K + k);
+      a0[i][0] = ph[0];
+      a0[i][1] = ph[1];
+      if (src1) {
+        const float4* pd = reinterpret_cast<const float4*>(src1 + (size_t)m * K + k);
+        a1[i][0] = pd[0];
+        a1[i][1] = pd[1];
+      } else {
+        a1[i][0] = a1[i][1] = float4{0.f, 0.f, 0.f, 0.f};
+      }
+      const float4* pg = reinterpret_cast<const float4*>(gain + k);
+      a2[i][0] = pg[0];
+      a2[i][1] = pg[1];
+    } else {
+      const float4* pa = reinterpret_cast<const float4*>(src0 + (size_t)m * 2 * K + k);
+      const float4* pu = reinterpret_cast<const float4*>(src0 + (size_t)m * 2 * K + K + k);
+      a0[i][0] = pa[0];
+      a0[i][1] = pa[1];
+      a1[i][0] = pu[0];
+      a1[i][1] = pu[1];
+    }
+  }
+  if (kW4) {
+    const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  float sc[TPW], zc[TPW];
+  if (kW4) {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      sc[p] = f16_bits_to_f32(mw[p] & 0xFFFFu);
+      zc[p] = f16_bits_to_f32(mw[p] >> 16);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // ---- the activations of this slice, 8 per lane and load
+  float xv[kXLoads][8];
+  if (kPro == kProNorm) {
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const float4 h0 = a0[i][0], h1 = a0[i][1], d0 = a1[i][0], d1 = a1[i][1];
+      xv[i][0] = h0.x + d0.x; xv[i][1] = h0.y + d0.y; xv[i][2] = h0.z + d0.z; xv[i][3] = h0.w + d0.w;
+      xv[i][4] = h1.x + d1.x; xv[i][5] = h1.y + d1.y; xv[i][6] = h1.z + d1.z; xv[i][7] = h1.w + d1.w;
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += xv[i][e] * xv[i][e];
+      // the kVecPerRow consecutive lanes of a row
+#pragma unroll
+      for (int off = kVecPerRow / 2; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+      const int v = lane + 64 * i;
+      if (v < kVecs && (v % kVecPerRow) == 0) ssq[(v / kVecPerRow) * kWaves + wave] = ss;
+      if (nt == 0 && v < kVecs && v / kVecPerRow < M) {  // the updated residual stream, once
+        float4* po = reinterpret_cast<float4*>(h_out + (size_t)(v / kVecPerRow) * K + g0 * kGroup + 8 * (v % kVecPerRow));
+        po[0] = float4{xv[i][0], xv[i][1], xv[i][2], xv[i][3]};
+        po[1] = float4{xv[i][4], xv[i][5], xv[i][6], xv[i][7]};
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = min(lane + 64 * i, kVecs - 1);
+      const float* part = ssq + (v / kVecPerRow) * kWaves;
+      float total = 0.f;
+#pragma unroll
+      for (int u = 0; u < kWaves; ++u) total += part[u];
+      const float rms = sqrtf(total / (float)K + eps);
+      const float4 g0v = a2[i][0], g1v = a2[i][1];
+      xv[i][0] = (xv[i][0] / rms) * g0v.x; xv[i][1] = (xv[i][1] / rms) * g0v.y;
+      xv[i][2] = (xv[i][2] / rms) * g0v.z; xv[i][3] = (xv[i][3] / rms) * g0v.w;
+      xv[i][4] = (xv[i][4] / rms) * g1v.x; xv[i][5] = (xv[i][5] / rms) * g1v.y;
+      xv[i][6] = (xv[i][6] / rms) * g1v.z; xv[i][7] = (xv[i][7] / rms) * g1v.w;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const float av[8] = {a0[i][0].x, a0[i][0].y, a0[i][0].z, a0[i][0].w, a0[i][1].x, a0[i][1].y, a0[i][1].z, a0[i][1].w};
+      const float uv[8] = {a1[i][0].x, a1[i][0].y, a1[i][0].z, a1[i][0].w, a1[i][1].x, a1[i][1].y, a1[i][1].z, a1[i][1].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xv[i][e] = av[e] * (1.0f / (1.0f + expf(-av[e]))) * uv[e];
+    }
+  }
+  // bf16, into the wave's own LDS rows
+#pragma unroll
+  for (int i = 0; i < kXLoads; ++i) {
+    const int v = lane + 64 * i;
+    u32x4_t pk;
+    pk.x = f32_to_bf16_rne(xv[i][0]) | ((uint32_t)f32_to_bf16_rne(xv[i][1]) << 16);
+    pk.y = f32_to_bf16_rne(xv[i][2]) | ((uint32_t)f32_to_bf16_rne(xv[i][3]) << 16);
+    pk.z = f32_to_bf16_rne(xv[i][4]) | ((uint32_t)f32_to_bf16_rne(xv[i][5]) << 16);
+    pk.w = f32_to_bf16_rne(xv[i][6]) | ((uint32_t)f32_to_bf16_rne(xv[i][7]) << 16);
+    if ((i + 1) * 64 <= kVecs || v < kVecs)
+      *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = pk;
+  }
+
+  // ---- the matmul, as in dequant_gemv_kernel
+  const uint32_t mask = 0x000F000Fu;
+  uint32_t magic = 0x43004300u;
+  asm volatile("" : "+v"(magic));
+  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  if (kW4) {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+        part = mfma16(a, w4_unpack(w[p][0][j], mask, magic), part);
+        asum = mfma16(a, ones, asum);
+      }
+#pragma unroll
+      for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
+    }
+  } else {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+        const u32x2_t lo = w8_to_bf16(w[p][j >> 1][2 * (j & 1)]);
+        const u32x2_t hi = w8_to_bf16(w[p][j >> 1][2 * (j & 1) + 1]);
+        acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);
+      }
+  }
+
+  // ---- the waves' partial sums meet in LDS; wave 0 adds them in wave order
+  asm volatile("" : "+v"(acc));
+  constexpr int kLive = MROWS < 4 ? MROWS : 4;
+  typedef float live_t __attribute__((ext_vector_type(kLive == 3 ? 4 : kLive)));
+  live_t* redv = reinterpret_cast<live_t*>(red);
+  live_t mine;
+#pragma unroll
+  for (int i = 0; i < kLive; ++i) mine[i] = acc[i];
+  if (kc < kRowQuads) redv[wave * (16 * kRowQuads) + lane] = mine;
+  __syncthreads();
+  if (wave != 0 || kc >= kRowQuads) return;
+  live_t part[kWaves];
+#pragma unroll
+  for (int u = 0; u < kWaves; ++u) part[u] = redv[u * (16 * kRowQuads) + lane];
+  live_t sum = part[0];
+#pragma unroll
+  for (int u = 1; u < kWaves; ++u) sum += part[u];
+  const int n = nt * kTileN + nl;
+  float cs = 1.0f;
+  if (!kW4) cs = f16_bits_to_f32(scales8[n]);
+#pragma unroll
+  for (int i = 0; i < kLive; ++i) {
+    const int m = 4 * kc + i;
+    if (m < M) {
+      const float v = sum[i] * cs;
+      if (out_f32)
+        reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
+      else
+        reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+    }
+  }
+}
+
+// LDS bytes of one workgroup: activation slices, reduction slots, partial sums of squares
+constexpr size_t gemv_pro_lds_bytes(int waves, int tpw, int mrows) {
+  return gemv_lds_bytes(waves, tpw, mrows) + (size_t)mrows * waves * 4;
+}
+
+}  // namespace ajq

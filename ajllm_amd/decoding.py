@@ -122,9 +122,36 @@ class _FusedLinear:
         self.wq = torch.cat([m.wq for m in layers], dim=0).contiguous()
         self.meta = torch.cat([m.meta for m in layers], dim=0).contiguous()
 
+        self.in_features = layers[0].in_features
+        self.rows16 = self.wq.shape[0] * 16
+
     def __call__(self, x_bf16: torch.Tensor) -> torch.Tensor:
         fn = w8a16_matmul if self.scheme == "w8a16" else w4a16_matmul
         return fn(x_bf16, self.wq, self.meta, torch.float32)
+
+    def fusable(self, batch: int) -> bool:
+        """Whether the GEMV with a norm / gate prologue is built for this batch and input width."""
+        return bool(_lib.load().ajq_gemv_fused_supported(batch, self.in_features))
+
+    def after_norm(self, h_in: torch.Tensor, delta: torch.Tensor | None, gain: torch.Tensor, eps: float,
+                   h_out: torch.Tensor) -> torch.Tensor:
+        """``self(bf16(RMSNorm(h_in + delta) * gain))`` with ``h_out = h_in + delta``, one launch."""
+        lib = _lib.load()
+        y = torch.empty((h_in.shape[0], self.rows16), dtype=torch.float32, device=h_in.device)
+        fn = lib.ajq_w8a16_gemv_norm if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_norm
+        _lib.check(fn(h_in.data_ptr(), delta.data_ptr() if delta is not None else None, gain.data_ptr(), eps,
+                      h_out.data_ptr(), h_in.shape[0], self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, y.data_ptr(), _lib.AJQ_OUT_F32, _stream()), "gemv_norm")
+        return y
+
+    def after_gate(self, ab: torch.Tensor) -> torch.Tensor:
+        """``self(bf16(silu(a) * u))`` for ``ab = (a | u)``, one launch."""
+        lib = _lib.load()
+        y = torch.empty((ab.shape[0], self.rows16), dtype=torch.float32, device=ab.device)
+        fn = lib.ajq_w8a16_gemv_gate if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_gate
+        _lib.check(fn(ab.data_ptr(), ab.shape[0], self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, y.data_ptr(), _lib.AJQ_OUT_F32, _stream()), "gemv_gate")
+        return y
 
 
 class FusedDecoder(GraphDecoder):
@@ -180,6 +207,15 @@ class FusedDecoder(GraphDecoder):
         self.vocab = model.lm_head.out_features
         self.embedding = model.token_embeddings.weight.detach()
         self.hidden = torch.zeros((batch, d), dtype=torch.float32, device=dev)
+        self.hidden2 = torch.zeros((batch, d), dtype=torch.float32, device=dev)
+        # GEMVs that form their own input (residual add + RMSNorm, SwiGLU gate) where they are built
+        # (the gate reads w1|w3's output as rows of 2 * d_ff: no padding rows between the halves)
+        # Every workgroup of such a GEMV re-reads the fp32 sources of all batch rows, so the saved
+        # launch only pays for small batches (measured on the 12-layer model: the norm up to batch
+        # 4, the gate at batch 1).
+        self.fuse_norm = batch <= 4 and self.head.fusable(batch)
+        self.fuse_gate = (batch == 1 and self.layers[0]["w2"].fusable(batch)
+                          and self.layers[0]["w13"].rows16 == 2 * self.d_ff)
         self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)
@@ -191,26 +227,36 @@ class FusedDecoder(GraphDecoder):
         lib, st = _lib.load(), _stream()
         b, d = self.batch, self.model.d_model
         pos = self.cache.position
-        torch.index_select(self.embedding, 0, self.token.view(-1), out=self.hidden)
+        cur, other = self.hidden, self.hidden2  # the residual stream and the buffer its next update goes to
+        torch.index_select(self.embedding, 0, self.token.view(-1), out=cur)
         delta = None
+
+        def normed_linear(linear, gain, eps):
+            """linear(RMSNorm(cur + delta) * gain); afterwards ``cur`` holds cur + delta."""
+            nonlocal cur, other
+            if self.fuse_norm:
+                out = linear.after_norm(cur, delta, gain, eps, other)
+                cur, other = other, cur
+                return out
+            _lib.check(lib.ajq_add_rmsnorm(cur.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                           gain.data_ptr(), eps, self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+            return linear(self.normed)
+
         for index, w in enumerate(self.layers):
-            _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), delta.data_ptr() if delta is not None else None,
-                                           w["g1"].data_ptr(), w["eps1"], self.normed.data_ptr(), b, d, st), "add_rmsnorm")
-            qkv = w["qkv"](self.normed)
+            qkv = normed_linear(w["qkv"], w["g1"], w["eps1"])
             _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
                                          self.cache.keys[index].data_ptr(), self.cache.values[index].data_ptr(),
                                          self.kv_flag, b, self.heads, self.kv_heads, 128, self.max_len,
                                          self.attended.data_ptr(), self.attn_ws.data_ptr(), self.attn_ws_bytes, st),
                        "attn_step")
-            attn_out = w["o"](self.attended)
-            _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), attn_out.data_ptr(), w["g2"].data_ptr(), w["eps2"],
-                                           self.normed.data_ptr(), b, d, st), "add_rmsnorm")
-            ab = w["w13"](self.normed)
-            _lib.check(lib.ajq_swiglu(ab.data_ptr(), self.gated.data_ptr(), b, self.d_ff, st), "swiglu")
-            delta = w["w2"](self.gated)
-        _lib.check(lib.ajq_add_rmsnorm(self.hidden.data_ptr(), delta.data_ptr(), self.final_gain.data_ptr(),
-                                       self.final_eps, self.normed.data_ptr(), b, d, st), "add_rmsnorm")
-        return self.head(self.normed)[:, : self.vocab]
+            delta = w["o"](self.attended)
+            ab = normed_linear(w["w13"], w["g2"], w["eps2"])
+            if self.fuse_gate:
+                delta = w["w2"].after_gate(ab)
+            else:
+                _lib.check(lib.ajq_swiglu(ab.data_ptr(), self.gated.data_ptr(), b, self.d_ff, st), "swiglu")
+                delta = w["w2"](self.gated)
+        return normed_linear(self.head, self.final_gain, self.final_eps)[:, : self.vocab]
 
 
 @torch.no_grad()

@@ -97,6 +97,26 @@ int ajq_w4a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
+/* The same GEMV with its activations produced on the way in (one launch less per use):
+ *   _norm: x = bf16(RMSNorm(h_in + delta) * gain) and h_out = h_in + delta (delta may be NULL;
+ *          h_out must not be h_in) -- the residual add and RMSNorm of TransformerBlock.forward
+ *          (src/ajllm/modeling/transformer.py:45-50, layers.py:70-74) in front of q|k|v or w1|w3;
+ *   _gate: x = bf16(silu(a) * u) for ab[M, 2K] = (a | u) -- SwiGLU.forward's product
+ *          (src/ajllm/modeling/activations.py:24-25) in front of w2.
+ * Built for the (M, K) that ajq_gemv_fused_supported reports: K = 1024 and 2048 (M <= 16), 4096
+ * and 5632 (M <= 8); AJQ_ERR_UNSUPPORTED otherwise (use the separate operators below). */
+int ajq_gemv_fused_supported(int M, int K);
+int ajq_w4a16_gemv_norm(const float* h_in, const float* delta, const float* gain, float eps, float* h_out,
+                        int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                        int out_dtype, void* stream);
+int ajq_w8a16_gemv_norm(const float* h_in, const float* delta, const float* gain, float eps, float* h_out,
+                        int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                        int out_dtype, void* stream);
+int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                        void* y, int out_dtype, void* stream);
+int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                        void* y, int out_dtype, void* stream);
+
 /* any M >= 1; bf16 MFMA.  M >= 256 (prefill) runs the 256 x 128 tile kernel, 17 <= M < 256
  * (several sequences decoded together) a weight-streaming kernel with 32-row activation
  * blocks, M <= 16 the GEMV above.

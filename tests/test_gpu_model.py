@@ -272,6 +272,74 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
     assert rel <= 1e-3, (max_abs, rel)
 
 
+@pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
+@pytest.mark.parametrize("m,k", [(1, 1024), (3, 2048), (16, 2048), (1, 4096), (8, 4096), (2, 5632), (8, 5632)])
+def test_gemv_with_norm_or_gate_prologue(cuda, scheme, m, k):
+    """ajq_w*a16_gemv_norm / _gate against the separate operators (add + RMSNorm, SwiGLU gate) followed by
+    the plain GEMV: same bf16 activations up to the rounding of a differently ordered sum of squares."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(5 + m + k)
+    n = 272
+    layer = QuantLinear.from_weight((torch.randn((n, k), generator=g) * 0.02).to(cuda), scheme)
+    fused = decoding._FusedLinear([layer])
+    assert fused.fusable(m) and not fused.fusable(17)
+    h = torch.randn((m, k), generator=g).to(cuda)
+    d = torch.randn((m, k), generator=g).to(cuda)
+    gain = (torch.rand(k, generator=g) + 0.5).to(cuda)
+    for delta in (d, None):
+        h_out = torch.zeros_like(h)
+        y = fused.after_norm(h, delta, gain, 1e-5, h_out)
+        h_ref = h.clone()
+        normed = torch.empty((m, k), dtype=torch.bfloat16, device=cuda)
+        _lib.check(lib.ajq_add_rmsnorm(h_ref.data_ptr(), delta.data_ptr() if delta is not None else None, gain.data_ptr(),
+                                       1e-5, normed.data_ptr(), m, k, st), "add_rmsnorm")
+        assert torch.equal(h_out, h_ref)
+        want = fused(normed)
+        assert errors(y, want.cpu())[1] <= 1e-3 and (y - want).abs().max() <= 2e-2
+    ab = (torch.randn((m, 2 * k), generator=g) * 2).to(cuda)
+    y = fused.after_gate(ab)
+    gated = torch.empty((m, k), dtype=torch.bfloat16, device=cuda)
+    _lib.check(lib.ajq_swiglu(ab.data_ptr(), gated.data_ptr(), m, k, st), "swiglu")
+    want = fused(gated)
+    assert torch.equal(y, want)  # same expression per element: identical activations, identical GEMV order
+
+
+@pytest.mark.parametrize("scheme,batch", [("w4a16_g128", 1), ("w8a16", 4), ("w4a16_g128", 16)])
+def test_fused_decoder_with_gemv_prologues(cuda, scheme, batch):
+    """A model whose widths the prologue GEMVs are built for (d_model 1024, d_ff 2048): the decoder
+    folds both norms and the gate into the following GEMVs; tokens against the eager loop."""
+    torch.manual_seed(14)
+    model = modeling.TransformerLM(vocab_size=512, context_length=96, d_model=1024, num_layers=2, num_heads=8,
+                                   d_ff=2048, num_kv_heads=4).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(11)).to(cuda)
+    eager, margins = modeling.greedy_decode(fast, prompt, 30, return_margins=True)
+    dec = decoding.FusedDecoder(fast, batch, 60)
+    assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
+    dec.fuse_norm = dec.fuse_gate = True  # also at the batches where the decoder would not choose them
+    dec.prefill(prompt)
+    got = dec.generate(30)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 20, noise=2e-3)
+    print(scheme, batch, report)
+    for row, step, margin in report["unexplained"]:
+        dec.prefill(prompt)
+        dec.generate(step)
+        with torch.no_grad():
+            fused_logits = dec._logits()[row].float()
+            eager_logits = fast(eager[row:row + 1, : 20 + step], fast.new_cache(1, 60))[0, -1].float()
+        gap = float((fused_logits - eager_logits).abs().max())
+        assert gap <= 1e-2 and margin <= 2 * gap, (row, step, margin, gap)
+    dec.prefill(prompt)
+    with torch.no_grad():
+        logits_fused = dec._logits()
+        cache = fast.new_cache(batch, 60)
+        fast(prompt, cache)
+        logits_eager = fast(dec.token, cache)[:, -1, :]
+    assert errors(logits_fused, logits_eager.cpu())[1] <= REL_FRO_TOL
+
+
 def test_fused_decoder_tokens_match_the_oracle_model(cuda):
     """The all-kernel, graph-replayed decode against the CPU oracle model (the restated Transformer
     with the oracle's QuantLinearRef in every linear slot), batch 4, head_dim 128, GQA off: the
