@@ -639,6 +639,20 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
   return check_launch("ajq_attn_step");
 }
 
+int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embedding, int D, float* hidden,
+                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, void* stream) {
+  if (!logits || !embedding || !hidden || !token || !out || !step)
+    return fail(AJQ_ERR_NULL, "ajq_greedy_pick: null pointer argument");
+  if (B < 1 || V < 1 || ld < V || D < 4 || D % 4 != 0 || out_ld < 1)
+    return fail(AJQ_ERR_SHAPE, "ajq_greedy_pick: unsupported shape (B=%d V=%d ld=%d D=%d out_ld=%d)", B, V, ld, D, out_ld);
+  if (!aligned16(embedding) || !aligned16(hidden))
+    return fail(AJQ_ERR_ALIGN, "ajq_greedy_pick: embedding and hidden must be 16-byte aligned");
+  hipLaunchKernelGGL(greedy_pick_kernel, dim3(B), dim3(1024), 0, (hipStream_t)stream, logits, V, ld, embedding, D, hidden,
+                     reinterpret_cast<long long*>(token), reinterpret_cast<long long*>(out), out_ld,
+                     reinterpret_cast<const long long*>(step));
+  return check_launch("ajq_greedy_pick");
+}
+
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream) {
   if (!ab || !out) return fail(AJQ_ERR_NULL, "ajq_swiglu: null pointer argument");
   if (B < 1 || F < 2 || F % 2 != 0) return fail(AJQ_ERR_SHAPE, "ajq_swiglu: need B >= 1 and even F (got %d, %d)", B, F);

@@ -277,26 +277,81 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   }
 }
 
-// merge of the S partial results of attn_decode_kernel: one wave per (b, h)
+// merge of the S <= 16 partial results of attn_decode_kernel: one wave per (b, h).  Lane s
+// fetches chunk s's maximum and denominator and every lane its two dimensions of all chunks
+// at once, so the kernel is one memory round trip, not one per chunk.
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, int S,
                                                         uint16_t* __restrict__ out) {
   constexpr int hd = 128;
   const int bh = blockIdx.x, lane = threadIdx.x;
   const float* src = partial + (size_t)bh * S * (hd + 2);
-  float M = -INFINITY;
-  for (int s = 0; s < S; ++s) M = fmaxf(M, src[s * (hd + 2)]);
+  const int sl = min(lane & 15, S - 1);
+  const float2 ml = *reinterpret_cast<const float2*>(src + sl * (hd + 2));  // (max, denominator) of chunk lane % 16
+  float2 a[16];
+#pragma unroll
+  for (int s = 0; s < 16; ++s) a[s] = *reinterpret_cast<const float2*>(src + min(s, S - 1) * (hd + 2) + 2 + 2 * lane);
+  float M = ml.x;
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+  const float mine = ml.x == -INFINITY ? 0.f : expf(ml.x - M);  // weight of chunk lane % 16
   float L = 0.f;
   float2 A = float2{0.f, 0.f};
-  for (int s = 0; s < S; ++s) {
-    const float ms = src[s * (hd + 2)];
-    const float c = ms == -INFINITY ? 0.f : expf(ms - M);
-    L += src[s * (hd + 2) + 1] * c;
-    const float2 a = *reinterpret_cast<const float2*>(src + s * (hd + 2) + 2 + 2 * lane);
-    A.x += a.x * c;
-    A.y += a.y * c;
+#pragma unroll
+  for (int s = 0; s < 16; ++s) {
+    const float c = __shfl(mine, s), l = __shfl(ml.y, s);
+    if (s < S) {
+      L += l * c;
+      A.x += a[s].x * c;
+      A.y += a[s].y * c;
+    }
   }
   const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
   reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
+}
+
+// Greedy choice at the end of a decode step, one workgroup of 1024 threads per sequence:
+// token = argmax(logits[b, 0..V)) (the lowest index among equal maxima, as torch.argmax),
+// written to token[b] and to out[b, *step]; then hidden[b, :] = embedding[token, :], the next
+// step's input.  `step` is only read.
+__global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restrict__ logits, int V, int ld,
+                                                           const float* __restrict__ embedding, int D,
+                                                           float* __restrict__ hidden, long long* __restrict__ token,
+                                                           long long* __restrict__ out, int out_ld,
+                                                           const long long* __restrict__ step) {
+  const int b = blockIdx.x, t = threadIdx.x;
+  const float* row = logits + (size_t)b * ld;
+  float best = -INFINITY;
+  int best_i = 0x7FFFFFFF;
+  for (int i = t; i < V; i += 1024) {  // ascending i per thread: a strict > keeps the first maximum
+    const float v = row[i];
+    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+  }
+  auto better = [](float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); };
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best, off);
+    const int oi = __shfl_xor(best_i, off);
+    if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
+  }
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  __shared__ int chosen;
+  if ((t & 63) == 0) { sv[t >> 6] = best; si[t >> 6] = best_i; }
+  __syncthreads();
+  if (t == 0) {
+    float bv = sv[0];
+    int bi = si[0];
+    for (int w = 1; w < 16; ++w)
+      if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
+    if (bi == 0x7FFFFFFF) bi = 0;  // a row of NaNs: torch picks the NaN; here index 0
+    chosen = bi;
+    token[b] = bi;
+    out[(size_t)b * out_ld + *step] = bi;
+  }
+  __syncthreads();
+  const float4* e4 = reinterpret_cast<const float4*>(embedding + (size_t)chosen * D);
+  float4* h4 = reinterpret_cast<float4*>(hidden + (size_t)b * D);
+  for (int i = t; i < D / 4; i += 1024) h4[i] = e4[i];
 }
 
 // ab [B, 2F] fp32 (gate projection, then up projection) -> out[b, f] = bf16( silu(a) * u ),

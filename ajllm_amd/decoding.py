@@ -205,9 +205,15 @@ class FusedDecoder(GraphDecoder):
         self.final_eps = model.final_norm.epsilon
         self.head = _FusedLinear([model.lm_head])
         self.vocab = model.lm_head.out_features
-        self.embedding = model.token_embeddings.weight.detach()
+        self.embedding = model.token_embeddings.weight.detach().float().contiguous()
+        self.embedded = torch.zeros((batch, d), dtype=torch.float32, device=dev)  # embedding row of self.token
         self.hidden = torch.zeros((batch, d), dtype=torch.float32, device=dev)
         self.hidden2 = torch.zeros((batch, d), dtype=torch.float32, device=dev)
+        # write position and output column advance together: one tensor, one increment per step
+        self.counters = torch.zeros(2, dtype=torch.long, device=dev)
+        self.cache.position = self.counters[0:1]
+        self.step_index = self.counters[1:2]
+        self.logits_full: torch.Tensor | None = None
         # GEMVs that form their own input (residual add + RMSNorm, SwiGLU gate) where they are built
         # (the gate reads w1|w3's output as rows of 2 * d_ff: no padding rows between the halves)
         # Every workgroup of such a GEMV re-reads the fp32 sources of all batch rows, so the saved
@@ -223,12 +229,35 @@ class FusedDecoder(GraphDecoder):
         self.attn_ws_bytes = int(lib.ajq_attn_step_workspace_bytes(batch, self.heads))
         self.attn_ws = torch.zeros(max(self.attn_ws_bytes, 16), dtype=torch.uint8, device=dev)
 
+    @torch.no_grad()
+    def prefill(self, prompt: torch.Tensor, rows_per_pass: int | None = None) -> None:
+        super().prefill(prompt, rows_per_pass)
+        torch.index_select(self.embedding, 0, self.token.view(-1), out=self.embedded)
+
+    @torch.no_grad()
+    def _step(self) -> None:
+        """One token: the layer stack, then the greedy choice, its embedding row (the next step's
+        input) and the two counters, in two launches."""
+        self._logits()
+        full = self.logits_full
+        _lib.check(_lib.load().ajq_greedy_pick(full.data_ptr(), self.batch, self.vocab, full.shape[1],
+                                               self.embedding.data_ptr(), self.model.d_model, self.embedded.data_ptr(),
+                                               self.token.data_ptr(), self.out.data_ptr(), self.out.shape[1],
+                                               self.step_index.data_ptr(), _stream()), "greedy_pick")
+        self.counters.add_(1)
+
     def _logits(self) -> torch.Tensor:
+        """Logits ``[B, V]`` of the token whose embedding row is in ``self.embedded`` (``prefill`` and
+        every step leave it there), at cache row ``cache.position``; the decoding state is untouched."""
         lib, st = _lib.load(), _stream()
         b, d = self.batch, self.model.d_model
         pos = self.cache.position
-        cur, other = self.hidden, self.hidden2  # the residual stream and the buffer its next update goes to
-        torch.index_select(self.embedding, 0, self.token.view(-1), out=cur)
+        if self.fuse_norm:
+            # the first norm reads the embedding row where it is; the updated stream goes to `other`
+            cur, other = self.embedded, self.hidden
+        else:
+            cur, other = self.hidden, self.hidden2
+            cur.copy_(self.embedded)
         delta = None
 
         def normed_linear(linear, gain, eps):
@@ -236,7 +265,7 @@ class FusedDecoder(GraphDecoder):
             nonlocal cur, other
             if self.fuse_norm:
                 out = linear.after_norm(cur, delta, gain, eps, other)
-                cur, other = other, cur
+                cur, other = other, (self.hidden2 if cur is self.embedded else cur)
                 return out
             _lib.check(lib.ajq_add_rmsnorm(cur.data_ptr(), delta.data_ptr() if delta is not None else None,
                                            gain.data_ptr(), eps, self.normed.data_ptr(), b, d, st), "add_rmsnorm")
@@ -256,7 +285,8 @@ class FusedDecoder(GraphDecoder):
             else:
                 _lib.check(lib.ajq_swiglu(ab.data_ptr(), self.gated.data_ptr(), b, self.d_ff, st), "swiglu")
                 delta = w["w2"](self.gated)
-        return normed_linear(self.head, self.final_gain, self.final_eps)[:, : self.vocab]
+        self.logits_full = normed_linear(self.head, self.final_gain, self.final_eps)
+        return self.logits_full[:, : self.vocab]
 
 
 @torch.no_grad()

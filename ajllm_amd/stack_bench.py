@@ -99,6 +99,7 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     first = torch.argmax(torch.cat(logits, dim=0), dim=-1, keepdim=True)
     dec.out.index_copy_(1, dec.step_index, first)
     dec.token.copy_(first)
+    torch.index_select(dec.embedding, 0, first.view(-1), out=dec.embedded)
     dec.step_index.add_(1)
     dec.produced, dec.prompt_len = 1, context
 

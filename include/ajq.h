@@ -167,6 +167,14 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
  * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
 
+/* Greedy choice at the end of a decode step: token[b] = argmax(logits[b, 0..V)) (row stride ld;
+ * the lowest index among equal maxima: next = argmax(logits[:, -1]) of generate,
+ * src/ajllm/generation/generator.py:20-27, sampling.py:9-10), also stored at out[b, *step] (row
+ * stride out_ld), and hidden[b, :] = embedding[token[b], :] (Embedding.forward,
+ * src/ajllm/modeling/layers.py:52-53), the next step's input.  token, out, step: int64. */
+int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embedding, int D, float* hidden,
+                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

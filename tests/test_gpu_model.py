@@ -272,6 +272,30 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
     assert rel <= 1e-3, (max_abs, rel)
 
 
+def test_greedy_pick(cuda):
+    """ajq_greedy_pick against torch.argmax (first maximum wins), the output column and the embedding row."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(3)
+    for b, v, ld, d in ((1, 32000, 32000, 2048), (5, 1000, 1008, 256), (32, 128256, 128256, 64)):
+        logits = torch.randn((b, ld), generator=g).to(cuda)
+        logits[:, v:] = 100.0                      # padding columns must not be looked at
+        logits[0, 7] = logits[0, 900] = 50.0       # equal maxima: the lower index
+        if b > 1:
+            logits[1, v - 1] = 60.0                # the last valid column
+        emb = torch.randn((v, d), generator=g).to(cuda)
+        hidden = torch.zeros((b, d), device=cuda)
+        token = torch.zeros((b, 1), dtype=torch.long, device=cuda)
+        out = torch.full((b, 9), -1, dtype=torch.long, device=cuda)
+        step = torch.tensor([4], device=cuda)
+        _lib.check(lib.ajq_greedy_pick(logits.data_ptr(), b, v, ld, emb.data_ptr(), d, hidden.data_ptr(), token.data_ptr(),
+                                       out.data_ptr(), 9, step.data_ptr(), st), "greedy_pick")
+        want = torch.argmax(logits[:, :v], dim=-1)
+        assert want[0] == 7 and torch.equal(token.view(-1), want) and torch.equal(out[:, 4], want)
+        assert (out[:, :4] == -1).all() and (out[:, 5:] == -1).all() and torch.equal(hidden, emb[want])
+
+
 @pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
 @pytest.mark.parametrize("m,k", [(1, 1024), (3, 2048), (16, 2048), (1, 4096), (8, 4096), (2, 5632), (8, 5632)])
 def test_gemv_with_norm_or_gate_prologue(cuda, scheme, m, k):
