@@ -1,0 +1,40 @@
+"""Host side of the library's causal prefill attention (``ajq_attn_prefill``).
+
+Stands where the reference switches to its FlashAttention under ``use_flash_attention``
+(src/ajllm/modeling/attention.py:106-117; its own kernels, flash_attention.py:44-108,194-298, need
+CUDA/Triton).  Same contract as there: the arithmetic is flash attention's (bf16 products, fp32
+online softmax), not bit-for-bit the eager fp32 one, so it is opt-in.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def flash_prefill(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, start: int) -> torch.Tensor:
+    """Causal attention of the ``T`` new positions ``start .. start + T - 1``.
+
+    ``q`` fp32 ``[B, H, T, 128]`` (rotated); ``keys`` / ``values`` ``[B, Hkv, max_len, 128]`` fp32 or
+    bf16 whose rows ``0 .. start + T - 1`` are filled (a KV cache, or the keys and values themselves
+    with ``start == 0``).  Returns fp32 ``[B, T, H * 128]``."""
+    if not q.is_cuda:
+        raise ValueError("flash_prefill needs tensors on a ROCm device (there is no CPU path)")
+    batch, heads, seq, hd = q.shape
+    kv_heads, max_len = keys.shape[1], keys.shape[2]
+    if hd != 128 or keys.shape != values.shape or keys.shape[0] != batch or keys.shape[3] != 128:
+        raise ValueError("flash_prefill: q [B, H, T, 128] and caches [B, Hkv, max_len, 128] expected")
+    if keys.dtype not in (torch.float32, torch.bfloat16) or values.dtype != keys.dtype:
+        raise ValueError("flash_prefill: the caches must be float32 or bfloat16")
+    if not (keys.is_contiguous() and values.is_contiguous()):
+        raise ValueError("flash_prefill: the caches must be contiguous")
+    q = q.float().contiguous()
+    out = torch.empty((batch, seq, heads * hd), dtype=torch.float32, device=q.device)
+    flag = _lib.AJQ_KV_F32 if keys.dtype == torch.float32 else _lib.AJQ_KV_BF16
+    with torch.cuda.device(q.device):
+        status = _lib.load().ajq_attn_prefill(q.data_ptr(), keys.data_ptr(), values.data_ptr(), flag, batch, heads,
+                                              kv_heads, seq, start, max_len, hd, out.data_ptr(),
+                                              torch.cuda.current_stream().cuda_stream)
+    _lib.check(status, "attn_prefill")
+    return out

@@ -10,6 +10,7 @@
 #include "gemm_kernels.h"
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
+#include "prefill_attention.h"
 
 using namespace ajq;
 
@@ -651,6 +652,30 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
                      reinterpret_cast<long long*>(token), reinterpret_cast<long long*>(out), out_ld,
                      reinterpret_cast<const long long*>(step));
   return check_launch("ajq_greedy_pick");
+}
+
+int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H, int Hkv,
+                     int T, int start, int max_len, int head_dim, float* out, void* stream) {
+  if (!q || !kcache || !vcache || !out) return fail(AJQ_ERR_NULL, "ajq_attn_prefill: null pointer argument");
+  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (only 128 is built)", head_dim);
+  if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || T < 1 || start < 0 || (long long)start + T > max_len ||
+      (long long)B * H > 65535)
+    return fail(AJQ_ERR_SHAPE, "ajq_attn_prefill: unsupported shape (B=%d H=%d Hkv=%d T=%d start=%d max_len=%d)", B, H,
+                Hkv, T, start, max_len);
+  if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+  if (!aligned16(q) || !aligned16(kcache) || !aligned16(vcache) || !aligned16(out))
+    return fail(AJQ_ERR_ALIGN, "ajq_attn_prefill: q, the caches and out must be 16-byte aligned");
+  const dim3 grid((T + kPfBQ - 1) / kPfBQ, B * H);
+  if (cache_dtype == AJQ_KV_F32)
+    hipLaunchKernelGGL(attn_prefill_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, q,
+                       reinterpret_cast<const float*>(kcache), reinterpret_cast<const float*>(vcache), H, Hkv, T, start,
+                       max_len, out);
+  else
+    hipLaunchKernelGGL(attn_prefill_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, q,
+                       reinterpret_cast<const uint16_t*>(kcache), reinterpret_cast<const uint16_t*>(vcache), H, Hkv, T,
+                       start, max_len, out);
+  return check_launch("ajq_attn_prefill");
 }
 
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream) {

@@ -69,6 +69,8 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     model = build_quantized_model(device, scheme, seed=4321, config=config)
     torch.cuda.synchronize()
     build_s = time.perf_counter() - t0
+    for layer in model.layers:  # prefill attention through the library's flash-attention kernel
+        layer.attention.use_flash_attention = True
     quant = [m for m in model.modules() if isinstance(m, QuantLinear)]
     packed = sum(m.wq.numel() * 4 + m.meta.numel() * m.meta.element_size() for m in quant)
     g = torch.Generator().manual_seed(77)
@@ -143,7 +145,7 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     result = {
         "scheme": scheme, "config": config, "batch": batch, "context": context, "build_s": build_s,
         "packed_weight_bytes": packed,
-        "prefill": {"tokens_per_pass": PREFILL_ROWS * context, "s_per_pass": t_pass,
+        "prefill": {"tokens_per_pass": PREFILL_ROWS * context, "s_per_pass": t_pass, "attention": "ajq_attn_prefill",
                     "tok/s": PREFILL_ROWS * context / t_pass,
                     "quant_linear_s_per_pass": t_pass_linear, "quant_linear_share": t_pass_linear / t_pass,
                     "quant_linear_TFLOP/s": 2 * PREFILL_ROWS * context * sum(

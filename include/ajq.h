@@ -167,6 +167,15 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
  * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
 
+/* Causal attention of T new positions (absolute positions start .. start + T - 1) over cache
+ * rows 0 .. start + T - 1, which the caller has already written; q fp32 [B, H, T, head_dim]
+ * (rotated), out fp32 [B, T, H * head_dim].  Flash-attention arithmetic: bf16 MFMA products,
+ * fp32 online softmax, no T x T matrix (scaled_dot_product_attention under a causal mask,
+ * src/ajllm/modeling/attention.py:20-33,106-117; the reference's own tiled and Triton variants,
+ * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128 only. */
+int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H,
+                     int Hkv, int T, int start, int max_len, int head_dim, float* out, void* stream);
+
 /* Greedy choice at the end of a decode step: token[b] = argmax(logits[b, 0..V)) (row stride ld;
  * the lowest index among equal maxima: next = argmax(logits[:, -1]) of generate,
  * src/ajllm/generation/generator.py:20-27, sampling.py:9-10), also stored at out[b, *step] (row

@@ -272,6 +272,60 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
     assert rel <= 1e-3, (max_abs, rel)
 
 
+@pytest.mark.parametrize("b,heads,kv_heads,t,start,cache_dtype", [
+    (2, 4, 2, 100, 0, torch.float32), (1, 2, 2, 64, 0, torch.float32), (1, 4, 1, 130, 37, torch.float32),
+    (3, 2, 1, 257, 5, torch.bfloat16), (1, 1, 1, 1, 9, torch.float32), (1, 8, 2, 512, 0, torch.bfloat16)])
+def test_flash_prefill_attention(cuda, b, heads, kv_heads, t, start, cache_dtype):
+    """ajq_attn_prefill against the model code's masked softmax attention.  The kernel rounds q, k, v
+    and the probabilities to bf16 (flash-attention arithmetic): compared with the fp32 statement on the
+    same bf16-rounded inputs within 4e-3 relative Frobenius, and with the unrounded one within 1e-2."""
+    from ajllm_amd.attention import flash_prefill
+    g = torch.Generator().manual_seed(b * 1000 + t)
+    hd, max_len = 128, start + t + 3
+    q = torch.randn((b, heads, t, hd), generator=g).to(cuda)
+    keys = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
+    values = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
+    got = flash_prefill(q, keys, values, start)
+    assert got.shape == (b, t, heads * hd) and bool(torch.isfinite(got).all())
+    total = start + t
+    rep = heads // kv_heads
+    k32 = keys[:, :, :total].float().repeat_interleave(rep, dim=1)
+    v32 = values[:, :, :total].float().repeat_interleave(rep, dim=1)
+    mask = torch.ones(t, total, dtype=torch.bool, device=cuda).tril_(diagonal=start)
+    def statement(qq, kk, vv):
+        return modeling.scaled_dot_product_attention(qq, kk, vv, mask).transpose(1, 2).reshape(b, t, heads * hd)
+    rounded = lambda x: x.to(torch.bfloat16).float()
+    want_rounded = statement(rounded(q), rounded(k32), rounded(v32))
+    want = statement(q, k32, v32)
+    assert errors(got, want_rounded.cpu())[1] <= 4e-3, errors(got, want_rounded.cpu())
+    assert errors(got, want.cpu())[1] <= 1e-2, errors(got, want.cpu())
+
+
+def test_model_with_flash_attention_flag(cuda):
+    """use_flash_attention on every attention layer: prefill logits stay within flash-attention noise of
+    the eager model, with and without a KV cache, and a following cached step agrees as well."""
+    torch.manual_seed(2)
+    model = modeling.TransformerLM(vocab_size=512, context_length=160, d_model=512, num_layers=2, num_heads=4,
+                                   d_ff=1408, num_kv_heads=2).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w8a16")
+    tokens = torch.randint(0, 512, (2, 150), generator=torch.Generator().manual_seed(4)).to(cuda)
+    with torch.no_grad():
+        eager = fast(tokens)
+        cache_e = fast.new_cache(2, 160)
+        fast(tokens[:, :149], cache_e)
+        step_e = fast(tokens[:, 149:], cache_e)
+        for layer in fast.layers:
+            layer.attention.use_flash_attention = True
+        flash = fast(tokens)
+        cache_f = fast.new_cache(2, 160)
+        first = fast(tokens[:, :100], cache_f)      # two chunks: the second starts at row 100
+        second = fast(tokens[:, 100:149], cache_f)
+        step_f = fast(tokens[:, 149:], cache_f)
+    assert errors(flash, eager.cpu())[1] <= 1e-2
+    assert errors(torch.cat((first, second), 1), eager[:, :149].cpu())[1] <= 1e-2
+    assert errors(step_f, step_e.cpu())[1] <= 1e-2
+
+
 def test_greedy_pick(cuda):
     """ajq_greedy_pick against torch.argmax (first maximum wins), the output column and the embedding row."""
     from ajllm_amd import _lib
