@@ -33,19 +33,20 @@ def build_quantized_model(device, scheme: str = "w4a16_g128", seed: int = 1234, 
     return model
 
 
-def _linear_seconds_per_step(model, batch: int, device) -> float:
-    """Time of the quantized linears of one decode step on their own: every QuantLinear once, with
-    ``[batch, in_features]`` inputs, replayed from a HIP graph."""
-    layers = [m for m in model.modules() if isinstance(m, QuantLinear)]
-    inputs = [torch.randn((batch, m.in_features), device=device).to(torch.bfloat16) for m in layers]
+def _linear_seconds_per_step(dec: "decoding.FusedDecoder", batch: int, device) -> float:
+    """Time of the quantized linears of one decode step on their own, as the decoder launches them
+    (fused q|k|v and w1|w3, output projection, w2, lm_head; plain GEMVs on ``[batch, in_features]``
+    inputs), replayed from a HIP graph."""
+    linears = [w[name] for w in dec.layers for name in ("qkv", "o", "w13", "w2")] + [dec.head]
+    inputs = [torch.randn((batch, m.in_features), device=device).to(torch.bfloat16) for m in linears]
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream), torch.no_grad():
-        for m, x in zip(layers, inputs):
+        for m, x in zip(linears, inputs):
             m(x)
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            for m, x in zip(layers, inputs):
+            for m, x in zip(linears, inputs):
                 m(x)
         graph.replay()
         stream.synchronize()
@@ -114,7 +115,7 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
                 step_i = int(diff[0])
                 diverged.append({"row": row, "step": step_i, "eager_margin": float(margins[row, step_i])})
         same = min([d["step"] for d in diverged], default=NEW_TOKENS)
-        t_linear = _linear_seconds_per_step(model, batch, device)
+        t_linear = _linear_seconds_per_step(dec, batch, device)
         step = t_graph / graph_steps
         r = {
             "scheme": scheme, "batch": batch, "prompt": PROMPT_LEN, "new_tokens": NEW_TOKENS,
@@ -130,9 +131,12 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
             "quant_linear_share_of_step": t_linear / step,
             "quant_linear_GB/s": packed / t_linear / 1e9,
             "packed_weight_bytes": packed,
-            "loop": "one-token step replayed from a HIP graph, token fed back on the device; the step is "
-                    "this library's kernels (fused q|k|v and w1|w3 GEMVs, add+RMSNorm, RoPE+cache write, "
-                    "single-query attention, SwiGLU gate) plus PyTorch's embedding lookup and argmax",
+            "launches_per_layer": 6 if (dec.fuse_norm and dec.fuse_gate) else 7 if dec.fuse_norm else 9,
+            "loop": "one-token step replayed from a HIP graph, token fed back on the device; the step is this "
+                    "library's kernels only (fused q|k|v and w1|w3 GEMVs with the residual add + RMSNorm formed on "
+                    "their way in at small batch, RoPE + cache write + single-query attention in one kernel, merge "
+                    "of its row chunks, output projection, w2 with the SwiGLU gate on its way in at batch 1, greedy "
+                    "pick + embedding row) plus one counter increment",
         }
         log("decode", r)
         results.append(r)
