@@ -515,10 +515,16 @@ namespace {
 #ifndef AJQ_ATTN_WGS
 #define AJQ_ATTN_WGS 256
 #endif
+#ifndef AJQ_ATTN_ROWS_PER_CHUNK
+#define AJQ_ATTN_ROWS_PER_CHUNK 128
+#endif
 constexpr int kAttnMaxSplits = 16;
-// row chunks per cache head: enough workgroups to cover the CUs
-int attn_splits(int B, int Hkv) {
+// row chunks per cache head: enough workgroups to cover the CUs, and few enough rows per chunk
+// that a 16-lane team (two rows in flight) makes only a handful of dependent round trips
+int attn_splits(int B, int Hkv, int max_len) {
   int s = AJQ_ATTN_WGS / (B * Hkv);
+  const int by_rows = max_len / AJQ_ATTN_ROWS_PER_CHUNK;
+  if (by_rows > s) s = by_rows;
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
 }
 
@@ -594,7 +600,7 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
   const int R = H / Hkv;
   if (R != 1 && R != 2 && R != 4)
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: %d query heads per cache head (1, 2 and 4 are built)", R);
-  const int S = attn_splits(B, Hkv);
+  const int S = attn_splits(B, Hkv, max_len);
   if (S > 1 && (!workspace || workspace_bytes < ajq_attn_decode_workspace_bytes(B, H)))
     return fail(AJQ_ERR_WORKSPACE, "ajq_attn_decode: workspace of %zu bytes needed, %zu given",
                 ajq_attn_decode_workspace_bytes(B, H), workspace_bytes);
@@ -629,7 +635,7 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
   if (!aligned16(qkv) || !aligned16(cosine) || !aligned16(sine) || !aligned16(kcache) || !aligned16(vcache))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_step: qkv, the tables and the caches must be 16-byte aligned");
-  const int S = attn_splits(B, Hkv);
+  const int S = attn_splits(B, Hkv, max_len);
   if (S > 1 && (!workspace || workspace_bytes < ajq_attn_step_workspace_bytes(B, H) || !aligned16(workspace)))
     return fail(AJQ_ERR_WORKSPACE, "ajq_attn_step: 16-byte aligned workspace of %zu bytes needed, %zu given",
                 ajq_attn_step_workspace_bytes(B, H), workspace_bytes);
@@ -644,10 +650,10 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
                     int64_t* token, int64_t* out, int out_ld, const int64_t* step, void* stream) {
   if (!logits || !embedding || !hidden || !token || !out || !step)
     return fail(AJQ_ERR_NULL, "ajq_greedy_pick: null pointer argument");
-  if (B < 1 || V < 1 || ld < V || D < 4 || D % 4 != 0 || out_ld < 1)
+  if (B < 1 || V < 1 || ld < V || ld % 4 != 0 || D < 4 || D % 4 != 0 || out_ld < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_greedy_pick: unsupported shape (B=%d V=%d ld=%d D=%d out_ld=%d)", B, V, ld, D, out_ld);
-  if (!aligned16(embedding) || !aligned16(hidden))
-    return fail(AJQ_ERR_ALIGN, "ajq_greedy_pick: embedding and hidden must be 16-byte aligned");
+  if (!aligned16(logits) || !aligned16(embedding) || !aligned16(hidden))
+    return fail(AJQ_ERR_ALIGN, "ajq_greedy_pick: logits, embedding and hidden must be 16-byte aligned");
   hipLaunchKernelGGL(greedy_pick_kernel, dim3(B), dim3(1024), 0, (hipStream_t)stream, logits, V, ld, embedding, D, hidden,
                      reinterpret_cast<long long*>(token), reinterpret_cast<long long*>(out), out_ld,
                      reinterpret_cast<const long long*>(step));

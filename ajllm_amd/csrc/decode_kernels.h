@@ -322,9 +322,29 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
   const float* row = logits + (size_t)b * ld;
   float best = -INFINITY;
   int best_i = 0x7FFFFFFF;
-  for (int i = t; i < V; i += 1024) {  // ascending i per thread: a strict > keeps the first maximum
-    const float v = row[i];
-    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+  // four 128-bit loads per thread in flight; a thread meets its elements in ascending index
+  // order, so a strict > keeps the first maximum
+  const float4* row4 = reinterpret_cast<const float4*>(row);
+  const int nvec = V >> 2;
+  for (int base = 0; base < nvec; base += 4 * 1024) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int idx = base + u * 1024 + t;
+      v[u] = idx < nvec ? row4[idx] : float4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i0 = 4 * (base + u * 1024 + t);
+      if (v[u].x > best) { best = v[u].x; best_i = i0; }
+      if (v[u].y > best) { best = v[u].y; best_i = i0 + 1; }
+      if (v[u].z > best) { best = v[u].z; best_i = i0 + 2; }
+      if (v[u].w > best) { best = v[u].w; best_i = i0 + 3; }
+    }
+  }
+  if (4 * nvec + t < V) {  // the last V % 4 columns
+    const float v = row[4 * nvec + t];
+    if (v > best) { best = v; best_i = 4 * nvec + t; }
   }
   auto better = [](float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); };
 #pragma unroll
