@@ -163,6 +163,52 @@ def test_static_cache_steps_equal_dynamic_decoding():
         model(prompt, cache)  # a static cache takes one token per call
 
 
+def test_cache_rows_view_prefills_a_few_sequences_at_a_time():
+    """KVCache.rows(): prompts pushed through the model two sequences at a time into views of one
+    cache leave it exactly as one pass over all sequences does, and give the same logits."""
+    torch.manual_seed(12)
+    model = _model(num_layers=2)
+    prompt = torch.randint(0, model.vocab_size, (5, 9))
+    whole = model.new_cache(5, 12)
+    want = model(prompt, whole, last_token_only=True)
+    parts = model.new_cache(5, 12)
+    got = torch.cat([model(prompt[i:i + 2], parts.rows(i, min(i + 2, 5)), last_token_only=True) for i in (0, 2, 4)])
+    assert torch.allclose(got, want, atol=1e-6, rtol=1e-5)
+    for a, b in zip(parts.keys + parts.values, whole.keys + whole.values):
+        assert torch.allclose(a, b, atol=1e-6, rtol=1e-5)
+    assert parts.length == 0  # the views keep their own length; the owner's is set by the caller
+
+
+def test_narrower_kv_cache_rounds_keys_and_values_only():
+    """A bf16 KV cache: keys and values are rounded on write and widened on read; decoding with it
+    equals decoding where k and v are rounded by hand, and stays close to the fp32 cache."""
+    torch.manual_seed(13)
+    model = _model(num_layers=2)
+    prompt = torch.randint(0, model.vocab_size, (2, 8))
+    cache16 = model.new_cache(2, 10, dtype=torch.bfloat16)
+    cache32 = model.new_cache(2, 10)
+    a = model(prompt, cache16)
+    b = model(prompt, cache32)
+    assert cache16.keys[0].dtype == torch.bfloat16 and a.dtype == b.dtype == torch.float32
+    assert torch.equal(cache16.keys[0][:, :, :8], cache32.keys[0][:, :, :8].to(torch.bfloat16))
+    assert (a - b).abs().max() < 5e-2 and not torch.equal(a, b)
+    step16 = model(prompt[:, :1], cache16)
+    assert torch.isfinite(step16).all() and cache16.length == 9
+
+
+def test_flash_attention_flag_is_off_by_default_and_ignored_on_the_host():
+    """use_flash_attention mirrors the reference's flag: off by default, and a CPU call keeps the
+    masked-softmax path whatever it says (the kernel is a GPU one; no CPU fallback of it exists)."""
+    torch.manual_seed(14)
+    model = _model(num_layers=1)
+    tokens = torch.randint(0, model.vocab_size, (1, 7))
+    want = model(tokens)
+    assert all(not layer.attention.use_flash_attention for layer in model.layers)
+    for layer in model.layers:
+        layer.attention.use_flash_attention = True
+    assert torch.equal(model(tokens), want)
+
+
 def test_quantized_checkpoint_manifest_and_foreign_files(tmp_path):
     """The checkpoint reader refuses files that are not its own format (no GPU needed)."""
     from safetensors.torch import save_file
