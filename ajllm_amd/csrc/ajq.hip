@@ -269,6 +269,11 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
     if (M <= 4) return launch_gemv_cfg<11, 4, 4, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
     return launch_gemv_cfg<11, 4, 8, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   }
+  if (K == 16 * 7 * kGroup && M <= 4) {  // K = 14336 (112 groups): sixteen waves of seven groups, straight-line kernel
+    if (M <= 1) return launch_gemv_cfg<16, 7, 1, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    if (M <= 2) return launch_gemv_cfg<16, 7, 2, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+    return launch_gemv_cfg<16, 7, 4, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
+  }
   if (M <= 1) return launch_gemv_rows<8, 4, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 2) return launch_gemv_rows<8, 4, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (M <= 4) return launch_gemv_rows<8, 4, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);

@@ -187,6 +187,8 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
         part = mfma16(a, w4_unpack(w[p][0][j], mask, magic), part);
         asum = mfma16(a, ones, asum);
       }
+      // all four components stay live for the compiler (see dequant_gemv_kernel)
+      asm volatile("" : "+v"(part), "+v"(asum));
 #pragma unroll
       for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
     }

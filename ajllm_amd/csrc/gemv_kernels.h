@@ -166,6 +166,10 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
             part = mfma16(a, w4_unpack(b.w[p][0][j], mask, magic), part);
             asum = mfma16(a, ones, asum);
           }
+          // All four components stay live for the compiler.  With the components of unused
+          // rows dead (MROWS < 4) it reuses their registers while the MFMAs that still write
+          // them are in flight: the 16-wave configuration returned garbage that way.
+          asm volatile("" : "+v"(part), "+v"(asum));
           // (128+q) and (128+z) cancel in fp32 before the scale is applied
 #pragma unroll
           for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
@@ -358,6 +362,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_mt_kernel(
           const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
           part = mfma16(a, w4_unpack(b.w[p][0][j], mask, magic), part);
         }
+        asm volatile("" : "+v"(part));  // all four components live: see dequant_gemv_kernel
 #pragma unroll
         for (int i = 0; i < kLive; ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[p][i]);
       }
