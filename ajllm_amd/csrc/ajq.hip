@@ -589,6 +589,31 @@ int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, con
   return check_launch("ajq_rope_cache");
 }
 
+int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, float* q_out, void* kcache, void* vcache,
+                     int cache_dtype, int B, int T, int H, int Hkv, int head_dim, int start, int max_len, void* stream) {
+  if (!qkv || !cosine || !sine || !q_out || !kcache || !vcache)
+    return fail(AJQ_ERR_NULL, "ajq_rope_prefill: null pointer argument");
+  if (B < 1 || T < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || head_dim < 2 || head_dim % 2 != 0 || start < 0 ||
+      (long long)start + T > max_len)
+    return fail(AJQ_ERR_SHAPE, "ajq_rope_prefill: unsupported shape (B=%d T=%d H=%d Hkv=%d head_dim=%d start=%d max_len=%d)",
+                B, T, H, Hkv, head_dim, start, max_len);
+  if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_rope_prefill: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+  const long long pairs = (long long)B * T * (H + 2 * Hkv) * (head_dim / 2);
+  const long long blocks = (pairs + 255) / 256;
+  if (blocks > 0x7FFFFFFFLL) return fail(AJQ_ERR_SHAPE, "ajq_rope_prefill: too many elements");
+  const dim3 grid((unsigned)blocks);
+  if (cache_dtype == AJQ_KV_F32)
+    hipLaunchKernelGGL(rope_prefill_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, qkv, cosine, sine, q_out,
+                       reinterpret_cast<float*>(kcache), reinterpret_cast<float*>(vcache), B, T, H, Hkv, head_dim, start,
+                       max_len);
+  else
+    hipLaunchKernelGGL(rope_prefill_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, qkv, cosine, sine, q_out,
+                       reinterpret_cast<uint16_t*>(kcache), reinterpret_cast<uint16_t*>(vcache), B, T, H, Hkv, head_dim,
+                       start, max_len);
+  return check_launch("ajq_rope_prefill");
+}
+
 size_t ajq_attn_decode_workspace_bytes(int B, int H) {
   if (B < 1 || H < 1) return 0;
   // sized for the largest split count: the number of cache heads is not known here

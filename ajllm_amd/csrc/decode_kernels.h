@@ -95,6 +95,37 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
     store_pair(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i, r);
 }
 
+// Prefill form of the rotation: qkv [B * T, (H + 2 Hkv) * hd] fp32, row b * T + t at absolute
+// position start + t.  Rotated queries go to q_out [B, H, T, hd] (the layout the prefill
+// attention reads), rotated keys and plain values to rows start + t of the caches
+// [B, Hkv, max_len, hd].  One thread per pair.
+template <typename CacheT>
+__global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restrict__ qkv, const float* __restrict__ cosine,
+                                                           const float* __restrict__ sine, float* __restrict__ q_out,
+                                                           CacheT* __restrict__ kcache, CacheT* __restrict__ vcache,
+                                                           int B, int T, int H, int Hkv, int hd, int start, int max_len) {
+  const int half = hd >> 1;
+  const int heads = H + 2 * Hkv;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)B * T * heads * half) return;
+  const int i = (int)(idx % half);
+  const int head = (int)((idx / half) % heads);
+  const long long row = idx / ((long long)half * heads);  // b * T + t
+  const int b = (int)(row / T), t = (int)(row % T);
+  const long long p = (long long)start + t;
+  const float2 v = *reinterpret_cast<const float2*>(qkv + ((size_t)row * heads + head) * hd + 2 * i);
+  if (head >= H + Hkv) {
+    store_pair(vcache + (((size_t)b * Hkv + (head - H - Hkv)) * max_len + p) * hd + 2 * i, v);
+    return;
+  }
+  const float c = cosine[p * half + i], s = sine[p * half + i];
+  const float2 r = float2{v.x * c - v.y * s, v.x * s + v.y * c};
+  if (head < H)
+    *reinterpret_cast<float2*>(q_out + (((size_t)b * H + head) * T + t) * hd + 2 * i) = r;
+  else
+    store_pair(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i, r);
+}
+
 // Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * Hkv, S): a
 // workgroup of 4 waves takes chunk s of the rows of one cache head and serves the R = H / Hkv
 // query heads that share it, so a cache row is read once whatever R is.  Sixteen lanes share

@@ -230,9 +230,68 @@ class FusedDecoder(GraphDecoder):
         self.attn_ws = torch.zeros(max(self.attn_ws_bytes, 16), dtype=torch.uint8, device=dev)
 
     @torch.no_grad()
-    def prefill(self, prompt: torch.Tensor, rows_per_pass: int | None = None) -> None:
-        super().prefill(prompt, rows_per_pass)
+    def prefill(self, prompt: torch.Tensor, rows_per_pass: int | None = None, fused: bool = False) -> None:
+        """``fused``: the prompt goes through this library's kernels as well (GEMMs, add + RMSNorm,
+        RoPE + cache write, flash attention, SwiGLU gate) instead of the model's PyTorch code; the
+        attention then has flash-attention arithmetic, as with the model's ``use_flash_attention``."""
+        if not fused:
+            super().prefill(prompt, rows_per_pass)
+        else:
+            if prompt.shape[0] != self.batch or prompt.shape[1] >= self.max_len:
+                raise ValueError("prompt must be [batch, T] with T < max_len")
+            prompt = prompt.to(self.device)
+            step = rows_per_pass or self.batch
+            logits = torch.cat([self._prefill_rows(prompt[i:i + step], i) for i in range(0, self.batch, step)], dim=0)
+            self.cache.length = prompt.shape[1]
+            self.cache.static = True
+            self.cache.position.fill_(prompt.shape[1])
+            self.step_index.zero_()
+            nxt = torch.argmax(logits, dim=-1, keepdim=True)
+            self.out.index_copy_(1, self.step_index, nxt)
+            self.token.copy_(nxt)
+            self.step_index.add_(1)
+            self.produced = 1
+            self.prompt_len = prompt.shape[1]
         torch.index_select(self.embedding, 0, self.token.view(-1), out=self.embedded)
+
+    def _prefill_rows(self, prompt: torch.Tensor, first: int) -> torch.Tensor:
+        """Sequences ``first .. first + rows - 1`` of the batch through the layer stack on library
+        kernels, from an empty cache; returns the last position's logits ``[rows, V]``."""
+        lib, st = _lib.load(), _stream()
+        rows, seq = prompt.shape
+        d, m = self.model.d_model, rows * seq
+        hidden = self.embedding[prompt.reshape(-1)]  # [rows * seq, d] fp32, row b * seq + t
+        normed = torch.empty((m, d), dtype=torch.bfloat16, device=self.device)
+        q_rot = torch.empty((rows, self.heads, seq, 128), dtype=torch.float32, device=self.device)
+        gated = torch.empty((m, self.d_ff), dtype=torch.bfloat16, device=self.device)
+        delta = None
+        for index, w in enumerate(self.layers):
+            _lib.check(lib.ajq_add_rmsnorm(hidden.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                           w["g1"].data_ptr(), w["eps1"], normed.data_ptr(), m, d, st), "add_rmsnorm")
+            qkv = w["qkv"](normed)
+            keys, values = self.cache.keys[index][first:first + rows], self.cache.values[index][first:first + rows]
+            _lib.check(lib.ajq_rope_prefill(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), q_rot.data_ptr(),
+                                            keys.data_ptr(), values.data_ptr(), self.kv_flag, rows, seq, self.heads,
+                                            self.kv_heads, 128, 0, self.max_len, st), "rope_prefill")
+            del qkv
+            attended = torch.empty((m, d), dtype=torch.float32, device=self.device)
+            _lib.check(lib.ajq_attn_prefill(q_rot.data_ptr(), keys.data_ptr(), values.data_ptr(), self.kv_flag, rows,
+                                            self.heads, self.kv_heads, seq, 0, self.max_len, 128, attended.data_ptr(),
+                                            st), "attn_prefill")
+            delta = w["o"](attended.to(torch.bfloat16))
+            del attended
+            _lib.check(lib.ajq_add_rmsnorm(hidden.data_ptr(), delta.data_ptr(), w["g2"].data_ptr(), w["eps2"],
+                                           normed.data_ptr(), m, d, st), "add_rmsnorm")
+            ab = w["w13"](normed)
+            _lib.check(lib.ajq_swiglu(ab.data_ptr(), gated.data_ptr(), m, self.d_ff, st), "swiglu")
+            del ab
+            delta = w["w2"](gated)
+        last = hidden.view(rows, seq, d)[:, -1, :].contiguous()
+        last_delta = delta.view(rows, seq, -1)[:, -1, :d].contiguous()
+        last_normed = torch.empty((rows, d), dtype=torch.bfloat16, device=self.device)
+        _lib.check(lib.ajq_add_rmsnorm(last.data_ptr(), last_delta.data_ptr(), self.final_gain.data_ptr(), self.final_eps,
+                                       last_normed.data_ptr(), rows, d, st), "add_rmsnorm")
+        return self.head(last_normed)[:, : self.vocab]
 
     @torch.no_grad()
     def _step(self) -> None:

@@ -78,21 +78,33 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
 
     # ---- prefill, PREFILL_ROWS sequences (PREFILL_ROWS * context tokens) per pass, into the decoder's cache
     dec = decoding.FusedDecoder(model, batch, context + decode_steps + 8, kv_dtype)
-    dec.prefill(prompt[:, :64], rows_per_pass=PREFILL_ROWS)  # warm-up: library load, allocator
+    dec.prefill(prompt[:, :64], rows_per_pass=PREFILL_ROWS, fused=True)  # warm-up: library load, allocator
+    dec.prefill(prompt[:, :64], rows_per_pass=PREFILL_ROWS)
     torch.cuda.synchronize()
-    pass_times = []
+    # (a) the model's own PyTorch code around the library's GEMMs and flash attention, one pass
     dec.cache.static = False
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    eager_logits = model(prompt[:PREFILL_ROWS], dec.cache.rows(0, PREFILL_ROWS), last_token_only=True)[:, -1, :]
+    torch.cuda.synchronize()
+    t_pass_eager = time.perf_counter() - t0
+    # (b) library kernels only, every pass (this is what fills the cache the decode below starts from)
+    pass_times = []
     logits = []
     for start in range(0, batch, PREFILL_ROWS):
-        rows = dec.cache.rows(start, start + PREFILL_ROWS)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits.append(model(prompt[start:start + PREFILL_ROWS], rows, last_token_only=True)[:, -1, :])
+        logits.append(dec._prefill_rows(prompt[start:start + PREFILL_ROWS], start))
         torch.cuda.synchronize()
         pass_times.append(time.perf_counter() - t0)
     pass_times.sort()
     t_pass = pass_times[len(pass_times) // 2]
     t_pass_linear = _eager_linear_seconds(model, PREFILL_ROWS * context, device)
+    logits_rel = float((eager_logits.double() - logits[0].double()).norm() / eager_logits.double().norm())
+    top2 = torch.topk(eager_logits.float(), 2, dim=-1).values
+    first_match = {"rows_with_equal_argmax": int((torch.argmax(eager_logits, -1) == torch.argmax(logits[0], -1)).sum()),
+                   "rows": PREFILL_ROWS, "smallest_top2_margin": float((top2[:, 0] - top2[:, 1]).min()),
+                   "largest_logit_difference": float((eager_logits.float() - logits[0].float()).abs().max())}
     # hand the prefilled cache to the decoder (what FusedDecoder.prefill does after its passes)
     dec.cache.length = context
     dec.cache.static = True
@@ -145,7 +157,11 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     result = {
         "scheme": scheme, "config": config, "batch": batch, "context": context, "build_s": build_s,
         "packed_weight_bytes": packed,
-        "prefill": {"tokens_per_pass": PREFILL_ROWS * context, "s_per_pass": t_pass, "attention": "ajq_attn_prefill",
+        "prefill": {"tokens_per_pass": PREFILL_ROWS * context, "s_per_pass": t_pass,
+                    "path": "library kernels only: GEMMs, add + RMSNorm, RoPE + cache write, flash attention, gate",
+                    "s_per_pass_model_code_with_library_gemm_and_attention": t_pass_eager,
+                    "last_position_logits_relative_difference_between_the_two": logits_rel,
+                    "first_token_choice_between_the_two": first_match,
                     "tok/s": PREFILL_ROWS * context / t_pass,
                     "quant_linear_s_per_pass": t_pass_linear, "quant_linear_share": t_pass_linear / t_pass,
                     "quant_linear_TFLOP/s": 2 * PREFILL_ROWS * context * sum(

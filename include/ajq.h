@@ -147,6 +147,13 @@ int ajq_rope_cache(const float* qkv, const float* cosine, const float* sine, con
                    float* q_out, void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv,
                    int head_dim, int max_len, void* stream);
 
+/* The same rotation for T new positions per sequence (prefill): qkv[B * T, (H + 2 Hkv) * head_dim],
+ * row b * T + t at absolute position start + t; rotated queries to q_out[B, H, T, head_dim] (what
+ * ajq_attn_prefill reads), rotated keys and values to rows start + t of the caches. */
+int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, float* q_out, void* kcache,
+                     void* vcache, int cache_dtype, int B, int T, int H, int Hkv, int head_dim, int start,
+                     int max_len, void* stream);
+
 /* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
  * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
  * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of

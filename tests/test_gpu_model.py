@@ -326,6 +326,35 @@ def test_model_with_flash_attention_flag(cuda):
     assert errors(step_f, step_e.cpu())[1] <= 1e-2
 
 
+@pytest.mark.parametrize("scheme,kv_dtype", [("w4a16_g128", None), ("w8a16", torch.bfloat16)])
+def test_fused_prefill_matches_the_model_with_flash_attention(cuda, scheme, kv_dtype):
+    """FusedDecoder.prefill(fused=True): the prompt on library kernels only (GEMMs, add + RMSNorm, RoPE +
+    cache write, flash attention, gate), sequences a few at a time, against the model's own PyTorch
+    prefill with use_flash_attention: same caches, same first tokens, logits within flash-attention noise;
+    decoding continues from either state alike."""
+    torch.manual_seed(21)
+    model = modeling.TransformerLM(vocab_size=512, context_length=200, d_model=512, num_layers=2, num_heads=4,
+                                   d_ff=1408, num_kv_heads=2).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    for layer in fast.layers:
+        layer.attention.use_flash_attention = True
+    prompt = torch.randint(0, 512, (5, 150), generator=torch.Generator().manual_seed(3)).to(cuda)
+    a = decoding.FusedDecoder(fast, 5, 180, kv_dtype)
+    b = decoding.FusedDecoder(fast, 5, 180, kv_dtype)
+    a.prefill(prompt)
+    b.prefill(prompt, rows_per_pass=2, fused=True)
+    for x, y in zip(a.cache.keys + a.cache.values, b.cache.keys + b.cache.values):
+        # later layers see the earlier layers' flash-attention noise: bf16-level agreement
+        assert errors(y[:, :, :150].float(), x[:, :, :150].float().cpu())[1] <= 1e-2
+    # the first layer's keys see no attention at all: equal up to the rotation's fp32 rounding
+    assert errors(b.cache.keys[0][:, :, :150].float(), a.cache.keys[0][:, :, :150].float().cpu())[1] <= 2e-3
+    la, lb = a._logits(), b._logits()
+    assert errors(lb, la.cpu())[1] <= 2e-2
+    assert int(a.cache.position) == int(b.cache.position) == 150
+    ta, tb = a.generate(12), b.generate(12)
+    assert ta.shape == tb.shape == (5, 12) and (ta == tb).float().mean() >= 0.8
+
+
 def test_greedy_pick(cuda):
     """ajq_greedy_pick against torch.argmax (first maximum wins), the output column and the embedding row."""
     from ajllm_amd import _lib
