@@ -18,7 +18,8 @@
 //                  (contraction slot 8g + e <-> key 4g + e, or 16 + 4g + e - 4 for e >= 4), and
 //                  the A fragment takes the same keys of V^T, which is how V is laid down in
 //                  LDS (transposed on the way in, 2-byte stores).
-// Row maxima and sums need only the 4 lanes that share a query row (two shuffles).  bf16
+// Row maxima and sums need only the 4 lanes that share a query row (two shuffles).  The next
+// block of keys and values is fetched into registers while the current one is computed.  bf16
 // inputs, fp32 scores, probabilities rounded to bf16 for the second product, fp32 output
 // accumulators: the usual flash-attention arithmetic, not the eager fp32 one.
 #pragma once
@@ -38,13 +39,20 @@ __device__ __forceinline__ u32x4_t pack8_bf16(const float* v) {
   r.w = f32_to_bf16_rne(v[6]) | ((uint32_t)f32_to_bf16_rne(v[7]) << 16);
   return r;
 }
-// 8 consecutive cache elements as bf16
-__device__ __forceinline__ u32x4_t load8_bf16(const float* p) {
-  const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
-  const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+// 8 consecutive cache elements as loaded, and their bf16 form (made when they are needed, so
+// that the loads can stay in flight meanwhile)
+struct Raw8F32 {
+  float4 a, b;
+};
+__device__ __forceinline__ Raw8F32 load8_raw(const float* p) {
+  return Raw8F32{reinterpret_cast<const float4*>(p)[0], reinterpret_cast<const float4*>(p)[1]};
+}
+__device__ __forceinline__ u32x4_t load8_raw(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+__device__ __forceinline__ u32x4_t to_bf16x8(const Raw8F32& r) {
+  const float v[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
   return pack8_bf16(v);
 }
-__device__ __forceinline__ u32x4_t load8_bf16(const uint16_t* p) { return *reinterpret_cast<const u32x4_t*>(p); }
+__device__ __forceinline__ u32x4_t to_bf16x8(const u32x4_t& r) { return r; }
 
 template <typename CacheT>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
@@ -84,28 +92,37 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restri
 #pragma unroll
   for (int t = 0; t < 8; ++t) o[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (int kb0 = 0; kb0 < kv_end; kb0 += kPfBK) {
-    __syncthreads();  // the previous block's fragments have been read
-    // ---- K block row-major (16-byte stores), V block transposed (2-byte stores, keys fastest across lanes)
+  // One block of keys and values in registers, as loaded (8 elements per chunk, two chunks per
+  // thread and operand): chunk c of K is (key c / 16, dims 8 (c % 16) ..), of V (key c % 32,
+  // dims 8 (c / 32) ..): keys vary fastest across the lanes that store V transposed.
+  typedef decltype(load8_raw(kbase)) raw8_t;
+  raw8_t kraw[2], vraw[2];
+  auto fetch = [&](int kb0) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int c = threadIdx.x + 256 * u;  // 512 chunks of 8 elements
-      {
-        const int key = c >> 4, hd8 = c & 15;
-        const u32x4_t kv8 = load8_bf16(kbase + (size_t)min(kb0 + key, kv_len - 1) * kPfHD + 8 * hd8);
-        *reinterpret_cast<u32x4_t*>(Ks + key * kPfKStride + 8 * hd8) = kv8;
-      }
-      {
-        const int key = c & 31, hd8 = c >> 5;
-        const u32x4_t vv8 = load8_bf16(vbase + (size_t)min(kb0 + key, kv_len - 1) * kPfHD + 8 * hd8);
-        uint16_t* dst = Vt + (8 * hd8) * kPfVStride + key;
-        dst[0 * kPfVStride] = (uint16_t)(vv8.x & 0xFFFFu); dst[1 * kPfVStride] = (uint16_t)(vv8.x >> 16);
-        dst[2 * kPfVStride] = (uint16_t)(vv8.y & 0xFFFFu); dst[3 * kPfVStride] = (uint16_t)(vv8.y >> 16);
-        dst[4 * kPfVStride] = (uint16_t)(vv8.z & 0xFFFFu); dst[5 * kPfVStride] = (uint16_t)(vv8.z >> 16);
-        dst[6 * kPfVStride] = (uint16_t)(vv8.w & 0xFFFFu); dst[7 * kPfVStride] = (uint16_t)(vv8.w >> 16);
-      }
+      const int c = threadIdx.x + 256 * u;
+      kraw[u] = load8_raw(kbase + (size_t)min(kb0 + (c >> 4), kv_len - 1) * kPfHD + 8 * (c & 15));
+      vraw[u] = load8_raw(vbase + (size_t)min(kb0 + (c & 31), kv_len - 1) * kPfHD + 8 * (c >> 5));
+    }
+  };
+  fetch(0);
+  for (int kb0 = 0; kb0 < kv_end; kb0 += kPfBK) {
+    __syncthreads();  // the previous block's fragments have been read
+    // ---- K block row-major (16-byte stores), V block transposed (2-byte stores)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      *reinterpret_cast<u32x4_t*>(Ks + (c >> 4) * kPfKStride + 8 * (c & 15)) = to_bf16x8(kraw[u]);
+      const u32x4_t vv8 = to_bf16x8(vraw[u]);
+      uint16_t* dst = Vt + (8 * (c >> 5)) * kPfVStride + (c & 31);
+      dst[0 * kPfVStride] = (uint16_t)(vv8.x & 0xFFFFu); dst[1 * kPfVStride] = (uint16_t)(vv8.x >> 16);
+      dst[2 * kPfVStride] = (uint16_t)(vv8.y & 0xFFFFu); dst[3 * kPfVStride] = (uint16_t)(vv8.y >> 16);
+      dst[4 * kPfVStride] = (uint16_t)(vv8.z & 0xFFFFu); dst[5 * kPfVStride] = (uint16_t)(vv8.z >> 16);
+      dst[6 * kPfVStride] = (uint16_t)(vv8.w & 0xFFFFu); dst[7 * kPfVStride] = (uint16_t)(vv8.w >> 16);
     }
     __syncthreads();
+    // the next block's loads fly while this one is computed
+    if (kb0 + kPfBK < kv_end) fetch(kb0 + kPfBK);
     // ---- scores of the two 16-key halves: sc[jb][i] = S[qrow r][key kb0 + 16 jb + 4 g + i] (log2 units)
     f32x4_t sc[2];
 #pragma unroll
