@@ -61,4 +61,12 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
+// two fp32 -> one dword holding two bf16 (lo in bits 0..15), round to nearest even: a single
+// v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+
 }  // namespace ajq

@@ -51,8 +51,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
   for (int i = threadIdx.x; i < n4; i += 256) {
     const float4 v = h4[i];  // own writes above: same thread, same addresses
     const float4 g = g4[i];
-    const uint32_t lo = f32_to_bf16_rne((v.x / rms) * g.x) | ((uint32_t)f32_to_bf16_rne((v.y / rms) * g.y) << 16);
-    const uint32_t hi = f32_to_bf16_rne((v.z / rms) * g.z) | ((uint32_t)f32_to_bf16_rne((v.w / rms) * g.w) << 16);
+    const uint32_t lo = pack2_bf16((v.x / rms) * g.x, (v.y / rms) * g.y);
+    const uint32_t hi = pack2_bf16((v.z / rms) * g.z, (v.w / rms) * g.w);
     o2[i] = uint2{lo, hi};
   }
 }
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
 // The caches hold fp32 or (kBf16) bf16, rounded to nearest even.
 __device__ __forceinline__ void store_pair(float* p, float2 v) { *reinterpret_cast<float2*>(p) = v; }
 __device__ __forceinline__ void store_pair(uint16_t* p, float2 v) {
-  *reinterpret_cast<uint32_t*>(p) = f32_to_bf16_rne(v.x) | ((uint32_t)f32_to_bf16_rne(v.y) << 16);
+  *reinterpret_cast<uint32_t*>(p) = pack2_bf16(v.x, v.y);
 }
 
 template <typename CacheT>
@@ -171,10 +171,10 @@ __device__ __forceinline__ void store_row8(float* p, float4& a, float4& b) {
 __device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
   // rounds to bf16 and hands the rounded values back: what a later read of the cache would give
   u32x4_t v;
-  v.x = f32_to_bf16_rne(a.x) | ((uint32_t)f32_to_bf16_rne(a.y) << 16);
-  v.y = f32_to_bf16_rne(a.z) | ((uint32_t)f32_to_bf16_rne(a.w) << 16);
-  v.z = f32_to_bf16_rne(b.x) | ((uint32_t)f32_to_bf16_rne(b.y) << 16);
-  v.w = f32_to_bf16_rne(b.z) | ((uint32_t)f32_to_bf16_rne(b.w) << 16);
+  v.x = pack2_bf16(a.x, a.y);
+  v.y = pack2_bf16(a.z, a.w);
+  v.z = pack2_bf16(b.x, b.y);
+  v.w = pack2_bf16(b.z, b.w);
   *reinterpret_cast<u32x4_t*>(p) = v;
   a = float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u), __uint_as_float(v.y << 16),
              __uint_as_float(v.y & 0xFFFF0000u)};
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
       A.y += sacc[r][w][2 * lane + 1] * cw;
     }
     if (S == 1) {
-      const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
+      const uint32_t o = pack2_bf16(A.x / L, A.y / L);
       reinterpret_cast<uint32_t*>(out + (size_t)(bh0 + r) * hd)[lane] = o;
     } else {
       float* dst = partial + ((size_t)(bh0 + r) * S + s) * (hd + 2);
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
       A.y += a[s].y * c;
     }
   }
-  const uint32_t o = f32_to_bf16_rne(A.x / L) | ((uint32_t)f32_to_bf16_rne(A.y / L) << 16);
+  const uint32_t o = pack2_bf16(A.x / L, A.y / L);
   reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
 }
 
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ a
   const float2 u = *reinterpret_cast<const float2*>(ab + (size_t)b * 2 * F + F + 2 * i);
   const float x0 = a.x * (1.0f / (1.0f + expf(-a.x))) * u.x;
   const float x1 = a.y * (1.0f / (1.0f + expf(-a.y))) * u.y;
-  reinterpret_cast<uint32_t*>(out + (size_t)b * F)[i] = f32_to_bf16_rne(x0) | ((uint32_t)f32_to_bf16_rne(x1) << 16);
+  reinterpret_cast<uint32_t*>(out + (size_t)b * F)[i] = pack2_bf16(x0, x1);
 }
 
 }  // namespace ajq

@@ -162,10 +162,10 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   for (int i = 0; i < kXLoads; ++i) {
     const int v = lane + 64 * i;
     u32x4_t pk;
-    pk.x = f32_to_bf16_rne(xv[i][0]) | ((uint32_t)f32_to_bf16_rne(xv[i][1]) << 16);
-    pk.y = f32_to_bf16_rne(xv[i][2]) | ((uint32_t)f32_to_bf16_rne(xv[i][3]) << 16);
-    pk.z = f32_to_bf16_rne(xv[i][4]) | ((uint32_t)f32_to_bf16_rne(xv[i][5]) << 16);
-    pk.w = f32_to_bf16_rne(xv[i][6]) | ((uint32_t)f32_to_bf16_rne(xv[i][7]) << 16);
+    pk.x = pack2_bf16(xv[i][0], xv[i][1]);
+    pk.y = pack2_bf16(xv[i][2], xv[i][3]);
+    pk.z = pack2_bf16(xv[i][4], xv[i][5]);
+    pk.w = pack2_bf16(xv[i][6], xv[i][7]);
     if ((i + 1) * 64 <= kVecs || v < kVecs)
       *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = pk;
   }

@@ -36,12 +36,6 @@ constexpr int kPfBQ = 64 * kPfQG, kPfBK = 32, kPfHD = 128;
 constexpr int kPfKStride = kPfHD + 8;   // bf16 elements per K row in LDS
 constexpr int kPfVStride = kPfBK + 8;   // bf16 elements per V^T row in LDS (80 B: conflict-free 8-byte reads)
 
-// two fp32 -> one dword of two bf16 (round to nearest even): a single v_cvt_pk_bf16_f32
-__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
-  typedef float f32x2_t __attribute__((ext_vector_type(2)));
-  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
-}
 __device__ __forceinline__ u32x4_t pack8_bf16(const float* v) {
   return u32x4_t{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
 }
