@@ -498,3 +498,42 @@ def test_quantized_checkpoint_round_trip(cuda, tmp_path):
     (tmp_path / "bad.safetensors").write_bytes(bytes(raw))
     with pytest.raises(ValueError):
         checkpoint.read_quantized(tmp_path / "bad.safetensors")
+
+
+def test_quantization_report_against_the_oracle_model(cuda, tmp_path):
+    """Held-out loss of the quantized model (reference evaluate_model, evaluator.py:14-31) equals the
+    loss of the oracle model on the same windows, both schemes cost little, and the
+    caller's dense model is left untouched."""
+    import numpy as np
+
+    from ajllm_amd import evaluation
+    torch.manual_seed(21)
+    cfg = dict(vocab_size=512, context_length=64, d_model=256, num_layers=2, num_heads=2, d_ff=640)
+    dense = modeling.TransformerLM(**cfg).eval()
+    with torch.no_grad():  # sharpen the random-init model so its own samples are predictable to it
+        dense.lm_head.weight.mul_(6.0)
+        sample = torch.randint(0, 512, (1, 1))
+        gen = torch.Generator().manual_seed(3)
+        stream = [int(sample)]
+        cache = dense.new_cache(1, 64)
+        for _ in range(63):
+            probs = torch.softmax(dense(sample, cache)[0, -1], -1)
+            sample = torch.multinomial(probs, 1, generator=gen).view(1, 1)
+            stream.append(int(sample))
+    path = tmp_path / "heldout.bin"
+    np.asarray(stream * 8, dtype=np.uint32).tofile(path)
+    data = evaluation.TokenFile(path)
+    args = dict(batches=2, batch_size=4, context_length=32, seed=17)
+    deltas = {}
+    for scheme in ("w8a16", "w4a16_g128"):
+        report = evaluation.quantization_report(dense, data, scheme, device=cuda, **args)
+        oracle = evaluation.evaluate_model(_oracle_model(dense, scheme), data, device="cpu", **args)
+        print(scheme, report, oracle)
+        assert abs(report["quantized"]["loss"] - oracle["loss"]) < 2e-3
+        assert report["dense"]["loss"] < 6.0  # below ln(512) = 6.24: the stream is the model's own
+        deltas[scheme] = abs(report["loss_delta"])
+        assert abs(report["perplexity_ratio"] - np.exp(report["loss_delta"])) < 1e-6
+    # W8's delta is mostly the bf16 rounding of the activations at every linear, not the weights
+    assert deltas["w8a16"] < 0.05 and deltas["w4a16_g128"] < 0.25
+    assert all(isinstance(m, modeling.Linear) for m in (dense.lm_head, dense.layers[0].attention.q_proj))
+    dense.cpu()

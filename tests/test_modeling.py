@@ -222,3 +222,56 @@ def test_quantized_checkpoint_manifest_and_foreign_files(tmp_path):
     assert M.TransformerLM(**cfg).state_dict().keys() == model.state_dict().keys()
     with pytest.raises(ValueError):
         checkpoint.save_quantized(tmp_path / "dense.safetensors", model, "w4a16_g128")  # nothing quantized
+
+
+def _token_file(tmp_path, tokens):
+    import numpy as np
+    path = tmp_path / "tokens.bin"
+    np.asarray(tokens, dtype=np.uint32).tofile(path)
+    return path
+
+
+def test_cross_entropy_matches_library_and_closed_forms():
+    from ajllm_amd import evaluation
+    logits = torch.randn(3, 5, 37) * 4
+    targets = torch.randint(0, 37, (3, 5))
+    want = F.cross_entropy(logits.reshape(-1, 37), targets.reshape(-1))
+    assert torch.allclose(evaluation.cross_entropy(logits, targets), want, atol=1e-6)
+    assert abs(float(evaluation.cross_entropy(torch.zeros(4, 37), targets[0, :4])) - math.log(37)) < 1e-6
+    big = torch.full((2, 37), -1e4)
+    big[0, 3] = big[1, 9] = 1e4  # no overflow, certain prediction -> zero loss
+    assert float(evaluation.cross_entropy(big, torch.tensor([3, 9]))) == 0.0
+
+
+def test_token_file_windows_and_evaluation(tmp_path):
+    """Reference evaluate_model (evaluator.py:14-31): windows at generator.integers starts, targets one
+    token on, mean of per-batch losses, perplexity = exp(min(loss, 50))."""
+    import numpy as np
+
+    from ajllm_amd import evaluation
+    stream = np.arange(100) % 37
+    data = evaluation.TokenFile(_token_file(tmp_path, stream))
+    assert len(data) == 100
+    inputs, targets = data.batch(4, 8, "cpu", np.random.default_rng(5))
+    starts = np.random.default_rng(5).integers(0, 100 - 8 - 1 + 1, size=4)
+    assert inputs.dtype == torch.int64 and inputs.shape == targets.shape == (4, 8)
+    for row, s in enumerate(starts):
+        assert inputs[row].tolist() == stream[s:s + 8].tolist()
+        assert targets[row].tolist() == stream[s + 1:s + 9].tolist()
+    with pytest.raises(ValueError):
+        data.batch(1, 100, "cpu", np.random.default_rng(0))
+    (tmp_path / "odd.bin").write_bytes(b"\0" * 6)
+    with pytest.raises(ValueError):
+        evaluation.TokenFile(tmp_path / "odd.bin")
+
+    model = _model()
+    got = evaluation.evaluate_model(model, data, batches=3, batch_size=2, context_length=8, device="cpu", seed=9)
+    rng = np.random.default_rng(9)
+    losses = []
+    for _ in range(3):
+        x, y = data.batch(2, 8, "cpu", rng)
+        losses.append(float(F.cross_entropy(model(x).reshape(-1, 37), y.reshape(-1))))
+    assert abs(got["loss"] - sum(losses) / 3) < 1e-6 and got["batches"] == 3
+    assert abs(got["perplexity"] - math.exp(got["loss"])) < 1e-9
+    with pytest.raises(ValueError):
+        evaluation.evaluate_model(model, data, 0, 2, 8, "cpu", 9)
