@@ -28,6 +28,7 @@
 //  * The last row tile is shifted up to end at row M (M >= 256), so no row is
 //    clamped or masked; rows it shares with its neighbour are computed twice
 //    with identical results.
+//  * bf16 output leaves through LDS in whole 256-byte rows.
 #pragma once
 #include "ajq_common.h"
 
@@ -336,23 +337,51 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     __syncthreads();
   }
 
-  // ---- epilogue: accumulator register r of lane (col, kh) is row (r & 3) + 8 * (r >> 2) + 4 * kh
+  // ---- epilogue: accumulator register r of lane (col, kh) is row (r & 3) + 8 * (r >> 2) + 4 * kh.
+  // bf16 output: the tile is laid out row-major in LDS (the activation buffers are free: every
+  // wave has passed the loop's last barrier) and leaves in whole 256-byte rows, four rows per
+  // wave-wide 128-bit store; 2-byte stores straight from the accumulators took 2-3 times as long.
+  // Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart) use different banks.
+  constexpr int kOutStride = 272;
+  float cs[2] = {1.0f, 1.0f};
+  if (!kW4) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(n0 + wn * 64 + t * 32 + col, N - 1)]);
+  }
+  if (!out_f32) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          *reinterpret_cast<uint16_t*>(lds + row * kOutStride + (wn * 64 + t * 32 + col) * 2) =
+              f32_to_bf16_rne(acc[i][t][r] * cs[t]);
+        }
+    __syncthreads();
+    // lane -> (row within a group of 4, 16-byte piece of the 256-byte row); columns past N are dropped
+    const int piece = lane & 15, rsub = lane >> 4;
+    const bool live = n0 + piece * 8 < N;
+#pragma unroll
+    for (int j = 0; j < kLoadRows / 4; ++j) {
+      const int row = wave * kLoadRows + j * 4 + rsub;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kOutStride + piece * 16);
+      if (live)
+        *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * N + n0 + piece * 8) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int n = n0 + wn * 64 + t * 32 + col;
     if (n >= N) continue;
-    float cs = 1.0f;
-    if (!kW4) cs = f16_bits_to_f32(scales8[n]);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-        const float v = acc[i][t][r] * cs;
-        if (out_f32)
-          reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
-        else
-          reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+        reinterpret_cast<float*>(y)[(size_t)m * N + n] = acc[i][t][r] * cs[t];
       }
     }
   }
