@@ -27,6 +27,7 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_version": (c_int, []),
     "ajq_last_error": (c_char_p, []),
     "ajq_status_string": (c_char_p, [c_int]),
+    "ajq_probe_mfma_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w8": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w4_g128": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ajq_repack_w4": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),

@@ -156,6 +156,59 @@ def bench_gemm(scheme: str, m: int, n: int, k: int, steps: int, warmup: int, dev
             "TFLOP/s": tflops, "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS}
 
 
+# ------------------------------------------------------------------ yardsticks
+def bench_dense_library_gemm(m: int, n: int, k: int, steps: int, warmup: int, device, copies: int = 4) -> dict:
+    """The vendor library's plain bf16 GEMM (``torch.matmul`` on weights already expanded to bf16) on
+    the same shape, launch pattern and activations: what a GEMM with no dequantization work reaches."""
+    gen = torch.Generator(device=device).manual_seed(4321)
+    weights = [(torch.randn((n, k), generator=gen, device=device) * 0.02).to(torch.bfloat16) for _ in range(copies)]
+    x = make_x(m, k, device, 98, outliers=True)
+    outs = []
+
+    def step():
+        outs.clear()
+        for w in weights:
+            outs.append(torch.matmul(x, w.t()))
+
+    seconds = time_graph_steps(step, steps, warmup)
+    launches = steps * copies
+    tflops = gemm_flops(m, n, k) / (seconds / launches) / 1e12
+    return {"M": m, "N": n, "K": k, "us_per_launch": seconds / launches * 1e6, "TFLOP/s": tflops,
+            "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS}
+
+
+def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launches: int = 4) -> dict:
+    """bf16 MFMA rate the GPU sustains from registers alone (no memory traffic): with constant
+    operands and with random mantissas, where the power limit lowers the shader clock."""
+    import ctypes
+
+    from ajllm_amd import _lib
+
+    lib = _lib.load()
+    sink = torch.empty(workgroups * 512, dtype=torch.float32, device=device)
+    clocks = torch.zeros(2, dtype=torch.int64, device=device)
+    flops = ctypes.c_double(0.0)
+    stream = torch.cuda.current_stream()
+    out = {}
+    for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        def launch():
+            _lib.check(lib.ajq_probe_mfma_rate(rnd, iters, workgroups, sink.data_ptr(), clocks.data_ptr(),
+                                               ctypes.addressof(flops), stream.cuda_stream), "ajq_probe_mfma_rate")
+        launch()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(stream)
+        for _ in range(launches):
+            launch()
+        stop.record(stream)
+        stop.synchronize()
+        seconds = start.elapsed_time(stop) / 1e3 / launches
+        cycles, ticks = (int(v) for v in clocks.tolist())
+        out[name] = {"TFLOP/s": flops.value / seconds / 1e12, "ms_per_launch": seconds * 1e3,
+                     "shader_clock_GHz": cycles / max(ticks, 1) * 0.1}
+    return out
+
+
 # ------------------------------------------------------------------ CPU baseline
 def cpu_baseline(m: int, n: int, k: int, budget_s: float = 15.0) -> dict:
     """The oracle's quantized linear (dequantize -> matmul, fp32) on the host cores, same shape
@@ -236,6 +289,17 @@ def main() -> int:
             log("gemm", json.dumps(r))
             gemm.append(r)
         extras["prefill_gemm"] = gemm
+        dense = bench_dense_library_gemm(2048, 4096, 4096, steps=10, warmup=3, device=device)
+        log("dense library gemm", json.dumps(dense))
+        rate = bench_mfma_rate(device)
+        log("mfma rate", json.dumps(rate))
+        extras["yardsticks"] = {
+            "dense_bf16_library_gemm": [dense],
+            "mfma_from_registers": rate,
+            "note": "not part of the product path: the vendor library's plain bf16 GEMM on weights already "
+                    "expanded to bf16, and the MFMA rate sustained with no memory traffic (random operands "
+                    "reach the power limit and the shader clock drops)",
+        }
     if args.sweep:
         sweep = []
         for scheme in ("w4", "w8"):
@@ -254,6 +318,13 @@ def main() -> int:
                     log("gemm", json.dumps(r))
                     gemm.append(r)
         extras["prefill_sweep"] = gemm
+        dense = []
+        for sm in (256, 2048, 8192):
+            for sn in (4096, 14336):
+                r = bench_dense_library_gemm(sm, sn, 4096, steps=5, warmup=2, device=device, copies=2)
+                log("dense library gemm", json.dumps(r))
+                dense.append(r)
+        extras.setdefault("yardsticks", {})["dense_bf16_library_gemm_sweep"] = dense
     if args.decode:
         from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
 

@@ -186,3 +186,27 @@ def test_linearity_at_full_size(cuda):
     y1 = _run("w4", x1, wq, meta, torch.float32, "gemm")
     y2 = _run("w4", x2, wq, meta, torch.float32, "gemm")
     assert errors(y2, 2 * y1)[0] <= 1e-3
+
+
+def test_mfma_rate_probe_runs_and_reports_clocks(cuda):
+    """The device yardstick entry point: a short launch finishes, counts its flops and reports a
+    plausible shader clock (the rate itself is a measurement, not a pass criterion); bad arguments
+    are refused."""
+    import ctypes
+
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    sink = torch.zeros(8 * 512, dtype=torch.float32, device=cuda)
+    clocks = torch.zeros(2, dtype=torch.int64, device=cuda)
+    flops = ctypes.c_double(0.0)
+    for random_operands in (0, 1):
+        status = lib.ajq_probe_mfma_rate(random_operands, 2000, 8, sink.data_ptr(), clocks.data_ptr(),
+                                         ctypes.addressof(flops), torch.cuda.current_stream().cuda_stream)
+        assert status == 0
+        torch.cuda.synchronize()
+        assert flops.value == 8 * 8 * 2000 * 4 * 32768.0
+        cycles, ticks = (int(v) for v in clocks.tolist())
+        assert ticks > 0 and 0.3 < cycles / ticks * 0.1 < 3.5  # GHz
+        assert cycles >= 2000 * 4 * 32 * 0.9  # four 32-cycle MFMAs per iteration, issued in order
+    assert lib.ajq_probe_mfma_rate(0, 0, 8, sink.data_ptr(), clocks.data_ptr(), None, None) == -2
+    assert lib.ajq_probe_mfma_rate(0, 10, 8, None, clocks.data_ptr(), None, None) == -1
