@@ -531,18 +531,17 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 // --------------------------------------------------- decode-step operators -----
 namespace {
 #ifndef AJQ_ATTN_WGS
-#define AJQ_ATTN_WGS 256
-#endif
-#ifndef AJQ_ATTN_ROWS_PER_CHUNK
-#define AJQ_ATTN_ROWS_PER_CHUNK 128
+#define AJQ_ATTN_WGS 640
 #endif
 constexpr int kAttnMaxSplits = 16;
-// row chunks per cache head: enough workgroups to cover the CUs, and few enough rows per chunk
-// that a 16-lane team (two rows in flight) makes only a handful of dependent round trips
+// Row chunks per cache head.  Measured on (batch x cache heads) = 32 ... 256 at contexts 640 ... 4096: the
+// kernel is fastest with 500-800 workgroups in all (two to three per CU); more chunks only add start-up,
+// in-workgroup merges and partial results.  A chunk keeps at least 32 rows.
 int attn_splits(int B, int Hkv, int max_len) {
-  int s = AJQ_ATTN_WGS / (B * Hkv);
-  const int by_rows = max_len / AJQ_ATTN_ROWS_PER_CHUNK;
-  if (by_rows > s) s = by_rows;
+  const int pairs = B * Hkv;
+  int s = (AJQ_ATTN_WGS + pairs / 2) / pairs;
+  const int by_rows = max_len / 32;
+  if (s > by_rows) s = by_rows;
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
 }
 

@@ -80,7 +80,9 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(const float* __restrict
   const int i = (int)(idx % half);
   const int head = (int)((idx / half) % heads);
   const int b = (int)(idx / ((long long)half * heads));
-  const long long p = *pos;
+  // the position is device data the host cannot check: held inside the cache so that a stale or
+  // unwritten value gives a wrong row, never a wild address
+  const long long p = min(max(*pos, 0LL), (long long)max_len - 1);
   const float2 v = *reinterpret_cast<const float2*>(qkv + ((size_t)b * heads + head) * hd + 2 * i);
   if (head >= H + Hkv) {  // value head: stored as it is
     const int hv = head - H - Hkv;
@@ -182,6 +184,24 @@ __device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
              __uint_as_float(v.w & 0xFFFF0000u)};
 }
 
+// Sum over the 16 lanes of a team, result in every lane: four adds whose second operand comes
+// through the DPP row rotate (a "row" is 16 lanes), no LDS crossbar round trips.
+template <int kRor>
+__device__ __forceinline__ float row_ror(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + kRor, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float team_sum16(float v) {
+  v += row_ror<8>(v);
+  v += row_ror<4>(v);
+  v += row_ror<2>(v);
+  v += row_ror<1>(v);
+  return v;
+}
+// 2^x by the hardware instruction (1 ulp); the softmax below keeps its running maximum and
+// scores in the base-2 domain, scores pre-multiplied by log2(e)
+__device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
+constexpr float kLog2e = 1.4426950408889634f;
+
 template <int R, typename CacheT, bool kStep>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, CacheT* __restrict__ kcache,
                                                           CacheT* __restrict__ vcache,
@@ -194,7 +214,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   const int b = bk / Hkv, hk = bk % Hkv;
   const int bh0 = b * H + hk * R;  // first of the R query heads
   const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // 16 teams of 16 lanes
-  const long long p = *pos;
+  const long long p = min(max(*pos, 0LL), (long long)max_len - 1);  // held inside the cache (device data, unchecked by the host)
   const int rows = (int)p + 1;
   const int per = (rows + S - 1) / S;
   const int t_begin = s * per;
@@ -221,6 +241,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   }
   const CacheT* kbase = kcache + (size_t)bk * max_len * hd + 8 * c;
   const CacheT* vbase = vcache + (size_t)bk * max_len * hd + 8 * c;
+  const float scale2 = scale * kLog2e;  // maxima and the partial results' maxima are base-2 exponents
   float m[R], l[R], acc[R][8];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -235,11 +256,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     for (int r = 0; r < R; ++r) {
       float d = qa[r].x * ka.x + qa[r].y * ka.y + qa[r].z * ka.z + qa[r].w * ka.w + qb[r].x * kb.x + qb[r].y * kb.y +
                 qb[r].z * kb.z + qb[r].w * kb.w;
-#pragma unroll
-      for (int off = 8; off > 0; off >>= 1) d += __shfl_xor(d, off);
-      const float sc = d * scale;
+      const float sc = team_sum16(d) * scale2;
       const float m_new = fmaxf(m[r], sc);
-      const float corr = expf(m[r] - m_new), w = expf(sc - m_new);
+      const float corr = exp2_hw(m[r] - m_new), w = exp2_hw(sc - m_new);
       l[r] = l[r] * corr + w;
       acc[r][0] = acc[r][0] * corr + w * va.x; acc[r][1] = acc[r][1] * corr + w * va.y;
       acc[r][2] = acc[r][2] * corr + w * va.z; acc[r][3] = acc[r][3] * corr + w * va.w;
@@ -292,7 +311,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     float2 A = float2{0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
-      const float cw = sm[r][w] == -INFINITY ? 0.f : expf(sm[r][w] - M16);
+      const float cw = sm[r][w] == -INFINITY ? 0.f : exp2_hw(sm[r][w] - M16);
       L += sl[r][w] * cw;
       A.x += sacc[r][w][2 * lane] * cw;
       A.y += sacc[r][w][2 * lane + 1] * cw;
@@ -324,7 +343,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
   float M = ml.x;
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
-  const float mine = ml.x == -INFINITY ? 0.f : expf(ml.x - M);  // weight of chunk lane % 16
+  const float mine = ml.x == -INFINITY ? 0.f : exp2_hw(ml.x - M);  // weight of chunk lane % 16 (base-2 maxima)
   float L = 0.f;
   float2 A = float2{0.f, 0.f};
 #pragma unroll
@@ -397,7 +416,7 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
     if (bi == 0x7FFFFFFF) bi = 0;  // a row of NaNs: torch picks the NaN; here index 0
     chosen = bi;
     token[b] = bi;
-    out[(size_t)b * out_ld + *step] = bi;
+    out[(size_t)b * out_ld + min(max(*step, 0LL), (long long)out_ld - 1)] = bi;  // device data: held inside the row
   }
   __syncthreads();
   const float4* e4 = reinterpret_cast<const float4*>(embedding + (size_t)chosen * D);

@@ -40,6 +40,7 @@ def _linear_seconds_per_step(dec: "decoding.FusedDecoder", batch: int, device) -
     linears = [w[name] for w in dec.layers for name in ("qkv", "o", "w13", "w2")] + [dec.head]
     inputs = [torch.randn((batch, m.in_features), device=device).to(torch.bfloat16) for m in linears]
     stream = torch.cuda.Stream()
+    torch.cuda.synchronize()  # the inputs above are complete before ``stream`` reads them
     with torch.cuda.stream(stream), torch.no_grad():
         for m, x in zip(linears, inputs):
             m(x)

@@ -28,6 +28,7 @@ PREFILL_ROWS = 4
 
 def _graph_seconds(fn, stream, reps: int = 10) -> float:
     """Seconds per call of ``fn`` replayed from a HIP graph on ``stream``."""
+    torch.cuda.synchronize()  # inputs made on the default stream are complete before ``stream`` reads them
     with torch.cuda.stream(stream), torch.no_grad():
         fn()
         stream.synchronize()

@@ -91,6 +91,7 @@ def time_graph_steps(step_fn, steps: int, warmup: int) -> float:
     ``warmup`` times untimed, then time exactly ``steps`` replays with HIP events on the same
     stream.  Returns seconds for the ``steps`` replays."""
     stream = torch.cuda.Stream()
+    torch.cuda.synchronize()  # inputs made on the default stream are complete before ``stream`` reads them
     with torch.cuda.stream(stream):
         step_fn()  # eager once: sets function attributes, fills caches
         stream.synchronize()
