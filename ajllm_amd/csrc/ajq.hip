@@ -316,17 +316,28 @@ int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
 
-// M >= 17.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup: as
-// many as still leave a workgroup for every CU.  (Wider row blocks lose to more row tiles: a
-// workgroup's traffic is K * (2 * rows + bytes per weight * 16 * tiles) for rows * 16 * tiles
-// outputs.)
+// M >= 17.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup.  A workgroup
+// moves K * (2 * 32 + bytes per weight * 16 * tiles) bytes (the activations come from L2 once per
+// workgroup, so more row tiles mean less traffic per output) and the CUs take the workgroups in
+// rounds: the tile count with the smallest rounds x bytes wins (384 row tiles as 192 workgroups of
+// two run in one round instead of two: 14.7 -> 11.2 us at M = 32, K = 4096).  Wider row blocks
+// lose to more row tiles on the same count.
 template <bool kW4>
 int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   const int ntiles = N / kTileN;
   const int mblocks = (M + 31) / 32;
   int nt = 1;
-  while (nt < 4 && (ntiles / (2 * nt)) * mblocks >= 256) nt *= 2;
+  long long best = 0;
+  for (int c = 1; c <= 4; c *= 2) {
+    const long long wgs = (long long)((ntiles + c - 1) / c) * mblocks;
+    const int slots = (c == 4 && (ntiles / 4) * mblocks >= 512) ? 512 : 256;  // four-wave workgroups share a CU
+    const long long cost = ((wgs + slots - 1) / slots) * (64 + (kW4 ? 8 : 16) * c);
+    if (c == 1 || cost < best) {
+      best = cost;
+      nt = c;
+    }
+  }
   if (AJQ_SKINNY_FORCE_NT) nt = AJQ_SKINNY_FORCE_NT;
   if (nt == 1) return launch_skinny_cfg<8, 2, 32, 1, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   if (nt == 2) return launch_skinny_cfg<8, 1, 32, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
