@@ -8,6 +8,7 @@
 #include "gemv_kernels.h"
 #include "gemv_fused_kernels.h"
 #include "gemm_kernels.h"
+#include "gemm128_kernels.h"
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
 #include "prefill_attention.h"
@@ -88,6 +89,20 @@ int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
   const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
   hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
+                     reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
+  return AJQ_OK;
+}
+
+// 128 x 128 tiles, tiles requested two k-blocks ahead; M >= 128
+template <bool kW4>
+int launch_gemm128(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                   const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
+  auto kernel = dequant_gemm128_kernel<kW4>;
+  constexpr size_t lds = kW4 ? kG1LdsBytesW4 : kG1LdsBytesW8;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  const int tiles = ((M + kG1BM - 1) / kG1BM) * ((N + kG1BN - 1) / kG1BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(256), lds, stream, x, M, K,
                      reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
                      reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
   return AJQ_OK;
@@ -409,17 +424,32 @@ int check_pro(const char* name, int M, int K, const void* a, const void* b) {
   return AJQ_OK;
 }
 
-// M >= 256: the 256 x 128 tile kernel needs about a workgroup per CU to be worth its long K
-// loop; below that the weight-streaming kernel is faster.  Both times are modelled from
-// measurements: a k-block of the tile kernel takes about 1.8 us per round of 256 workgroups,
-// the streaming kernel sustains about 400 TFLOP/s for M >= 256.
-bool streaming_kernel_is_faster(int M, int N, int K) {
-  if (M < kGemm256MinM) return true;
-  const double tiles = (double)((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
-  const double rounds = (double)(long long)((tiles + 255) / 256);
-  const double us_tiles = rounds * (K / kGroup) * 1.8 + 3.0;
+// Which kernel runs a matmul of M >= 17 rows.  All three times are modelled from measurements
+// at K = 4096 (microseconds per k-block of 128 and round of 256 workgroups, one workgroup per CU).
+//  * 256 x 128 tiles: about 1.8 us.
+//  * 128 x 128 tiles (M >= 128): about 1.45 us (W4) / 1.25 us (W8): they win where the big tiles
+//    leave CUs idle (M = 1024 on N = 4096 is 128 big tiles or 256 small ones).
+//  * the weight-streaming kernel sustains about 400 TFLOP/s for M >= 256 and is the only one below
+//    M = 128.
+#ifndef AJQ_GEMM_TILE
+#define AJQ_GEMM_TILE 0  // 0: by the estimate; 128 or 256: that tile kernel for every M it can run
+#endif
+enum MatmulKernel { kStreaming, kTiles256, kTiles128 };
+MatmulKernel pick_matmul_kernel(int M, int N, int K, bool w4) {
+  if (AJQ_GEMM_TILE == 128 && M >= kG1BM) return kTiles128;
+  if (AJQ_GEMM_TILE == 256 && M >= kG2BM) return kTiles256;
+  if (M < kG1BM) return kStreaming;
+  const double G = (double)(K / kGroup);
   const double us_stream = 2.0 * M * N * (double)K / 400e6;
-  return us_stream < us_tiles;
+  double us_big = 1e30;
+  if (M >= kGemm256MinM) {
+    const long long tiles = (long long)((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
+    us_big = (double)((tiles + 255) / 256) * G * 1.8 + 3.0;
+  }
+  const long long small_ = (long long)((M + kG1BM - 1) / kG1BM) * ((N + kG1BN - 1) / kG1BN);
+  const double us_small = (double)((small_ + 255) / 256) * G * (w4 ? 1.45 : 1.25) + 5.0;
+  if (us_stream <= us_big && us_stream <= us_small) return kStreaming;
+  return us_small < us_big ? kTiles128 : kTiles256;
 }
 
 }  // namespace
@@ -492,7 +522,7 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
 
 // --------------------------------------------------------------- GEMM -----
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K) {
-  if (M < kGemm256MinM || K < kGroup) return 0;  // only the large-M kernel needs the group sums
+  if (M < kG1BM || K < kGroup) return 0;  // only the tile kernels need the group sums
   return (size_t)(K / kGroup) * M * 16;
 }
 
@@ -500,7 +530,8 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                    int out_dtype, void* workspace, size_t workspace_bytes, void* stream) {
   if (int s = check_matmul_args("ajq_w4a16_gemm", x, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
   const bool out_f32 = out_dtype == AJQ_OUT_F32;
-  if (streaming_kernel_is_faster(M, N, K)) {
+  const MatmulKernel which = M <= kMaxGemvM ? kStreaming : pick_matmul_kernel(M, N, K, true);
+  if (which == kStreaming) {
     const int s = M <= kMaxGemvM ? launch_gemv<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream)
                                  : launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream);
     return s ? s : check_launch("ajq_w4a16_gemm");
@@ -514,8 +545,10 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
   const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
   hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
                      K, reinterpret_cast<u32x4_t*>(workspace));
-  if (int s = launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32,
-                                                 (hipStream_t)stream))
+  if (int s = which == kTiles128
+                  ? launch_gemm128<true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32, (hipStream_t)stream)
+                  : launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32,
+                                                       (hipStream_t)stream))
     return s;
   return check_launch("ajq_w4a16_gemm");
 }
@@ -524,15 +557,18 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                    int out_dtype, void* stream) {
   if (int s = check_matmul_args("ajq_w8a16_gemm", x, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
   const bool out_f32 = out_dtype == AJQ_OUT_F32;
-  if (streaming_kernel_is_faster(M, N, K)) {
+  const MatmulKernel which = M <= kMaxGemvM ? kStreaming : pick_matmul_kernel(M, N, K, false);
+  if (which == kStreaming) {
     const int s = M <= kMaxGemvM ? launch_gemv<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream)
                                  : launch_skinny<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream);
     return s ? s : check_launch("ajq_w8a16_gemm");
   }
   if ((long long)M * K * 2 >= (1LL << 32))
     return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
-  if (int s = launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32,
-                                                  (hipStream_t)stream))
+  if (int s = which == kTiles128
+                  ? launch_gemm128<false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32, (hipStream_t)stream)
+                  : launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32,
+                                                        (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemm");
 }

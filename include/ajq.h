@@ -126,11 +126,13 @@ int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
 int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                         void* y, int out_dtype, void* stream);
 
-/* any M >= 1; bf16 MFMA.  M >= 256 (prefill) runs the 256 x 128 tile kernel, 17 <= M < 256
- * (several sequences decoded together) a weight-streaming kernel with 32-row activation
- * blocks, M <= 16 the GEMV above.
+/* any M >= 1; bf16 MFMA.  M <= 16 runs the GEMV above, 17 <= M < 128 (several sequences decoded
+ * together) a weight-streaming kernel with 32-row activation blocks, and from M = 128 on the
+ * fastest by a measured cost model of that kernel, a 128 x 128 tile kernel (shapes with few
+ * tiles) and a 256 x 128 tile kernel (M >= 256, prefill).
  * The W4 GEMM needs a workspace of ajq_w4a16_gemm_workspace_bytes(M, K) bytes (per-row,
- * per-group activation sums; 0 bytes below M = 256, where workspace may be NULL). */
+ * per-group activation sums for the tile kernels; 0 bytes below M = 128, where workspace may
+ * be NULL). */
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K);
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                    void* y, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);

@@ -62,13 +62,13 @@ def test_shape_alignment_and_option_errors():
     assert lib.ajq_w8a16_gemm(p, 1, 192, p, p, 16, p, 0, None) == -2
     assert lib.ajq_add_rmsnorm(p, None, p, 1e-5, p, 1, 6, None) == -2            # D not a multiple of 4
     assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 64, 8, p, p, 1 << 20, None) == -4  # head_dim 64 is not built
-    assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 128, 8, p, None, 0, None) == -6   # split attention needs its workspace
+    assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 128, 1024, p, None, 0, None) == -6  # split attention needs its workspace
     assert lib.ajq_attn_decode(p, p, p, 5, p, 1, 16, 16, 128, 8, p, p, 1 << 20, None) == -4  # unknown cache dtype
     assert lib.ajq_swiglu(p, p, 1, 3, None) == -2
     assert lib.ajq_rope_cache(p, p, p, p, p, p, p, 0, 1, 16, 3, 128, 8, None) == -2   # 16 query heads over 3 cache heads
     need = lib.ajq_w4a16_gemm_workspace_bytes(300, 512)
     assert need == 4 * 300 * 16                                             # G=4 groups x 300 rows x 16 bytes
-    assert lib.ajq_w4a16_gemm_workspace_bytes(255, 512) == 0                 # below 256 rows no workspace is used
+    assert lib.ajq_w4a16_gemm_workspace_bytes(127, 512) == 0                 # below 128 rows no tile kernel runs: no workspace
     assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 2, 128, 8, p, p, 1 << 20, None) == -4  # 8 query heads per cache head
     need = lib.ajq_w4a16_gemm_workspace_bytes(2048, 4096)                    # a shape the tile kernel takes
     assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, None, 0, None) == -6

@@ -140,6 +140,15 @@ def test_prefill_gemm(cuda, scheme, m, n, k):
     _check(scheme, "gemm", m, n, k, seed=31, cuda=cuda, outliers=True, max_rows=256)
 
 
+@pytest.mark.parametrize("m,n,k", [(1024, 4096, 4096), (1000, 3088, 4096), (640, 6144, 4096)])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_prefill_gemm_few_tiles(cuda, scheme, m, n, k):
+    """Shapes with fewer 256 x 128 tiles than CUs: the library's cost model takes the 128 x 128 tile
+    kernel (ring of three tile buffers); ragged M (last row tile shifted up) and an N whose last
+    column tile is partly outside the matrix."""
+    _check(scheme, "gemm", m, n, k, seed=33, cuda=cuda, outliers=True, max_rows=192)
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 @pytest.mark.parametrize("n", [4096, 14336])
 def test_prefill_gemm_m8192(cuda, scheme, n):
