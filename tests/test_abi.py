@@ -94,3 +94,13 @@ def test_python_layer_refuses_cpu_tensors():
     with pytest.raises(RuntimeError):
         QuantLinear(128, 16)(torch.zeros(1, 128))
     assert w4a16_matmul.__module__ == "ajllm_amd.quant"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The quantized linear is a one-GPU path: bench.py says so and exits non-zero for --gpus 2."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    proc = subprocess.run([sys.executable, str(Path(__file__).resolve().parents[1] / "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0 and "one GPU" in (proc.stderr + proc.stdout)
