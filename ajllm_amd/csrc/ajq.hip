@@ -95,14 +95,17 @@ int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 }
 
 // 128 x 128 tiles, tiles requested two k-blocks ahead; M >= 128
+#ifndef AJQ_G1_WN
+#define AJQ_G1_WN 4
+#endif
 template <bool kW4>
 int launch_gemm128(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                    const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
-  auto kernel = dequant_gemm128_kernel<kW4>;
+  auto kernel = dequant_gemm128_kernel<kW4, AJQ_G1_WN>;
   constexpr size_t lds = kW4 ? kG1LdsBytesW4 : kG1LdsBytesW8;
   if (int s = allow_big_lds(kernel, lds)) return s;
   const int tiles = ((M + kG1BM - 1) / kG1BM) * ((N + kG1BN - 1) / kG1BN);
-  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(256), lds, stream, x, M, K,
+  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(128 * AJQ_G1_WN), lds, stream, x, M, K,
                      reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
                      reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
   return AJQ_OK;
@@ -427,7 +430,7 @@ int check_pro(const char* name, int M, int K, const void* a, const void* b) {
 // Which kernel runs a matmul of M >= 17 rows.  All three times are modelled from measurements
 // at K = 4096 (microseconds per k-block of 128 and round of 256 workgroups, one workgroup per CU).
 //  * 256 x 128 tiles: about 1.8 us.
-//  * 128 x 128 tiles (M >= 128): about 1.45 us (W4) / 1.25 us (W8): they win where the big tiles
+//  * 128 x 128 tiles (M >= 128): about 1.25 us (W4) / 1.15 us (W8): they win where the big tiles
 //    leave CUs idle (M = 1024 on N = 4096 is 128 big tiles or 256 small ones).
 //  * the weight-streaming kernel sustains about 400 TFLOP/s for M >= 256 and is the only one below
 //    M = 128.
@@ -447,7 +450,7 @@ MatmulKernel pick_matmul_kernel(int M, int N, int K, bool w4) {
     us_big = (double)((tiles + 255) / 256) * G * 1.8 + 3.0;
   }
   const long long small_ = (long long)((M + kG1BM - 1) / kG1BM) * ((N + kG1BN - 1) / kG1BN);
-  const double us_small = (double)((small_ + 255) / 256) * G * (w4 ? 1.45 : 1.25) + 5.0;
+  const double us_small = (double)((small_ + 255) / 256) * G * (w4 ? 1.25 : 1.15) + 5.0;
   if (us_stream <= us_big && us_stream <= us_small) return kStreaming;
   return us_small < us_big ? kTiles128 : kTiles256;
 }

@@ -4,10 +4,10 @@
 //
 // Same arithmetic and operand paths as dequant_gemm256_kernel (everything enters LDS by DMA;
 // exact integers in bf16 through v_mfma_f32_32x32x16_bf16, scales in fp32, the W4 zero-point as
-// a ninth k-step against the three bf16 pieces of the activations' group sums), four waves as
-// 2 x 2 with 64 x 64 wave tiles, K walked in blocks of 128.  What differs: a workgroup has a CU
-// to itself and only one wave per SIMD, and a k-block is 36 MFMAs per wave, about half a
-// microsecond: less than a trip to memory.  So the tiles travel in a ring of THREE buffers and
+// a ninth k-step against the three bf16 pieces of the activations' group sums), eight waves as
+// 2 x 4 with 64 x 32 wave tiles, K walked in blocks of 128.  What differs: a workgroup has a CU
+// to itself, and a k-block is 36 MFMAs per SIMD, about half a microsecond: less than a trip to
+// memory.  So the tiles travel in a ring of THREE buffers and
 // are requested two k-blocks ahead; at the end of a block a wave waits only for the loads it
 // issued one block earlier (s_waitcnt vmcnt(loads per block)).
 #pragma once
@@ -27,8 +27,11 @@ constexpr int kG1MetaBase = kG1SideBase + kG1Ring * kG1SideSlot, kG1MetaSlot = 5
 constexpr size_t kG1LdsBytesW4 = kG1MetaBase + kG1Ring * kG1MetaSlot;  // 127.5 KiB
 constexpr size_t kG1LdsBytesW8 = kG1WBase + kG1Ring * kG1W8Slot;       // 144 KiB
 
-template <bool kW4>
-__global__ __launch_bounds__(256) void dequant_gemm128_kernel(
+// kWN = waves along N: 2 -> four waves with 64 x 64 wave tiles, 4 -> eight waves with 64 x 32
+// wave tiles (two waves per SIMD: each fetches twice the activation fragments per MFMA, but the
+// SIMD always has a second instruction stream to issue from).
+template <bool kW4, int kWN>
+__global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
     const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
@@ -36,9 +39,10 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
     int N, void* __restrict__ y, int out_f32) {
   constexpr int MT = 2;
   constexpr int kSteps = kW4 ? 9 : 8;  // MFMA k-steps per 128-k block
-  constexpr int kWaves = 4;
+  constexpr int kWaves = 2 * kWN;
+  constexpr int TB = 4 / kWN;          // 32-column blocks per wave
   constexpr int kWaveRows = 32 * MT;   // rows of the tile one wave computes
-  constexpr int kLoadRows = 32;        // rows of the tile one wave loads
+  constexpr int kLoadRows = kG1BM / kWaves;  // rows of the tile one wave loads
   constexpr int kBTiles = kW4 ? 8 : 16;  // 1 KiB private weight tiles per k-block and workgroup
   constexpr int kWSlot = kW4 ? kG1W4Slot : kG1W8Slot;
 
@@ -47,7 +51,7 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / kWN, wn = wave % kWN;
   const int col = lane & 31, kh = lane >> 5;
 
   // column-major walk over output tiles: consecutive workgroups share a column block of W
@@ -57,8 +61,8 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
   const int G = K >> 7;
   const int ntiles16 = N / kTileN;
 
-  // ---- global -> LDS.  Activations: wave w fills rows 32 w .. 32 w + 31 with eight wave-wide
-  // loads of 4 rows; chunk c of row r lives in slot c ^ (r & 15) of its row.  Every wave issues
+  // ---- global -> LDS.  Activations: wave w fills kLoadRows rows (128 / waves) with wave-wide
+  // loads of 4 rows (wave w: rows kLoadRows w ...); chunk c of row r lives in slot c ^ (r & 15) of its row.  Every wave issues
   // the same number of loads per k-block (the count the end-of-block wait relies on): where a
   // piece needs fewer loads than there are waves, two waves fetch the same bytes to the same place.
   const int row_in = lane >> 4, slot16 = lane & 15;
@@ -95,11 +99,11 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
     }
   };
 
-  f32x16_t acc[MT][2];
+  f32x16_t acc[MT][TB];
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < TB; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][t][r] = 0.f;
 
@@ -110,7 +114,7 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
   for (int v = 0; v < 8; ++v)
     a_off[v] = (uint32_t)((wm * kWaveRows + col) * 256 + (((v ^ ((col >> 1) & 7)) << 5) | ((kh ^ (col & 1)) << 4)));
   uint32_t g_off = (uint32_t)(kG1SideBase + (wm * kWaveRows + col) * 16);
-  const int c16 = wn * 4 + (col >> 4), nl = col & 15;
+  const int c16 = wn * (2 * TB) + (col >> 4), nl = col & 15;
   uint32_t b_off = (uint32_t)(kG1WBase + (kW4 ? c16 : 2 * c16) * 1024 + (kh * 16 + nl) * 16);
   uint32_t m_off = (uint32_t)(kG1MetaBase + (c16 * 16 + nl) * 4);
 
@@ -133,11 +137,11 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
     const int kb_load = min(kb + 2, G - 1);
     const int ring_load = ring == 0 ? 2 : ring - 1;  // (ring + 2) % 3: the slot read one block ago
 
-    u32x4_t raw[2][kW4 ? 2 : 4];
-    uint32_t mraw[2];
+    u32x4_t raw[TB][kW4 ? 2 : 4];
+    uint32_t mraw[TB];
     auto read_raw = [&](int first, int count) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < TB; ++t) {
         const int tb = t * (kW4 ? 2048 : 4096);
 #pragma unroll
         for (int q = first; q < first + count; ++q)
@@ -147,16 +151,16 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
     read_raw(0, 2);
     if (kW4) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
+      for (int t = 0; t < TB; ++t) mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
     }
 
     // ---- B fragments, unpacked one k-step ahead of their first use inside the wave's first
     // 32-row block, so the unpacking (VALU) runs under the MFMAs
-    u32x4_t bf[2][kSteps];
-    float sc[2];
+    u32x4_t bf[TB][kSteps];
+    float sc[TB];
     auto unpack_step = [&](int s) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
+      for (int t = 0; t < TB; ++t) {
         if (kW4) {
           if (s < 8) {
             bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], mask, magic);
@@ -193,7 +197,7 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
 #pragma unroll
     for (int p = 0; p < kAhead; ++p) afr[p] = *a_addr(p);
     unpack_step(0);
-    f32x16_t part[2];
+    f32x16_t part[TB];
 #pragma unroll
     for (int p = 0; p < kPos; ++p) {
       const int i = p / kSteps, s = p % kSteps;
@@ -203,21 +207,21 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
       if (kW4) {
         if (s == 0) {
 #pragma unroll
-          for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < TB; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) part[t][r] = 0.f;
         }
 #pragma unroll
-        for (int t = 0; t < 2; ++t) part[t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], part[t]);
+        for (int t = 0; t < TB; ++t) part[t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], part[t]);
         if (s == kSteps - 1) {
 #pragma unroll
-          for (int t = 0; t < 2; ++t)
+          for (int t = 0; t < TB; ++t)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][t][r] += sc[t] * part[t][r];
         }
       } else {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) acc[i][t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], acc[i][t]);
+        for (int t = 0; t < TB; ++t) acc[i][t] = mfma32(afr[p % (kAhead + 1)], bf[t][s], acc[i][t]);
       }
       __builtin_amdgcn_sched_barrier(0x2 | 0x4);  // VALU and SALU may cross
     }
@@ -248,20 +252,22 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
   // 128-bit store.  Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart)
   // use different banks.
   constexpr int kOutStride = 272;
-  float cs[2] = {1.0f, 1.0f};
+  float cs[TB];
+#pragma unroll
+  for (int t = 0; t < TB; ++t) cs[t] = 1.0f;
   if (!kW4) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(n0 + wn * 64 + t * 32 + col, N - 1)]);
+    for (int t = 0; t < TB; ++t) cs[t] = f16_bits_to_f32(scales8[min(n0 + wn * (32 * TB) + t * 32 + col, N - 1)]);
   }
   if (!out_f32) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < TB; ++t)
 #pragma unroll
       for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-          *reinterpret_cast<uint16_t*>(lds + row * kOutStride + (wn * 64 + t * 32 + col) * 2) =
+          *reinterpret_cast<uint16_t*>(lds + row * kOutStride + (wn * (32 * TB) + t * 32 + col) * 2) =
               f32_to_bf16_rne(acc[i][t][r] * cs[t]);
         }
     __syncthreads();
@@ -278,8 +284,8 @@ __global__ __launch_bounds__(256) void dequant_gemm128_kernel(
     return;
   }
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int n = n0 + wn * 64 + t * 32 + col;
+  for (int t = 0; t < TB; ++t) {
+    const int n = n0 + wn * (32 * TB) + t * 32 + col;
     if (n >= N) continue;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
