@@ -145,13 +145,13 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
         const int tb = t * (kW4 ? 2048 : 4096);
 #pragma unroll
         for (int q = first; q < first + count; ++q)
-          raw[t][q] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + q * 512);
+          raw[t][q] = lds_read128(b_off + tb + q * 512);
       }
     };
     read_raw(0, 2);
     if (kW4) {
 #pragma unroll
-      for (int t = 0; t < TB; ++t) mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
+      for (int t = 0; t < TB; ++t) mraw[t] = lds_read32(m_off + t * 128);
     }
 
     // ---- B fragments, unpacked one k-step ahead of their first use inside the wave's first
@@ -188,20 +188,19 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
     constexpr int kPos = MT * kSteps;
     constexpr int kAhead = 4;
     static_assert(kLoads <= kPos, "one load per position");
-    auto a_addr = [&](int p) -> const u32x4_t* {
+    auto a_frag = [&](int p) -> u32x4_t {
       const int i = p / kSteps, s = p % kSteps;
-      const uint32_t off = s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16;
-      return reinterpret_cast<const u32x4_t*>(lds + off);
+      return lds_read128(s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16);
     };
     u32x4_t afr[kAhead + 1];
 #pragma unroll
-    for (int p = 0; p < kAhead; ++p) afr[p] = *a_addr(p);
+    for (int p = 0; p < kAhead; ++p) afr[p] = a_frag(p);
     unpack_step(0);
     f32x16_t part[TB];
 #pragma unroll
     for (int p = 0; p < kPos; ++p) {
       const int i = p / kSteps, s = p % kSteps;
-      if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = *a_addr(p + kAhead);
+      if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = a_frag(p + kAhead);
       if (i == 0 && s + 1 < kSteps) unpack_step(s + 1);
       if (p < kLoads) issue_load(p, kb_load, ring_load);  // one load per position
       if (kW4) {

@@ -80,6 +80,16 @@ __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
 }
 
 typedef __attribute__((address_space(3))) void lds_void_t;
+// LDS reads by byte address.  The tile kernels declare no static LDS, so their dynamic LDS starts
+// at address 0 (the DMA destinations below are absolute addresses too); a read through
+// "pointer to the dynamic array + offset" costs a VALU add of that zero per read.
+typedef __attribute__((address_space(3))) const u32x4_t lds_u32x4_t;
+typedef __attribute__((address_space(3))) const uint32_t lds_u32_t;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wint-to-pointer-cast"  // the host pass sees 64-bit pointers
+__device__ __forceinline__ u32x4_t lds_read128(uint32_t address) { return *(lds_u32x4_t*)address; }
+__device__ __forceinline__ uint32_t lds_read32(uint32_t address) { return *(lds_u32_t*)address; }
+#pragma clang diagnostic pop
 typedef __attribute__((address_space(1))) const void global_void_t;
 
 // One wave-wide global -> LDS load of 16 bytes per lane: lane l reads base + voff(l) and
@@ -244,13 +254,13 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
         const int tb = t * (kW4 ? 2048 : 4096);
 #pragma unroll
         for (int q = first; q < first + count; ++q)
-          raw[t][q] = *reinterpret_cast<const u32x4_t*>(lds + b_off + tb + q * 512);
+          raw[t][q] = lds_read128(b_off + tb + q * 512);
       }
     };
     read_raw(0, 2);
     if (kW4) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) mraw[t] = *reinterpret_cast<const uint32_t*>(lds + m_off + t * 128);
+      for (int t = 0; t < 2; ++t) mraw[t] = lds_read32(m_off + t * 128);
     }
 
     // ---- B fragments.  They are unpacked one k-step ahead of their first use, inside the
@@ -289,20 +299,19 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
 #define AJQ_AHEAD 4
 #endif
     constexpr int kAhead = AJQ_AHEAD;
-    auto a_addr = [&](int p) -> const u32x4_t* {
+    auto a_frag = [&](int p) -> u32x4_t {
       const int i = p / kSteps, s = p % kSteps;
-      const uint32_t off = s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16;
-      return reinterpret_cast<const u32x4_t*>(lds + off);
+      return lds_read128(s < 8 ? a_off[s & 7] + i * 32 * 256 : g_off + i * 32 * 16);
     };
     u32x4_t afr[kAhead + 1];
 #pragma unroll
-    for (int p = 0; p < kAhead; ++p) afr[p] = *a_addr(p);
+    for (int p = 0; p < kAhead; ++p) afr[p] = a_frag(p);
     unpack_step(0);
     f32x16_t part[2];
 #pragma unroll
     for (int p = 0; p < kPos; ++p) {
       const int i = p / kSteps, s = p % kSteps;
-      if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = *a_addr(p + kAhead);
+      if (p + kAhead < kPos) afr[(p + kAhead) % (kAhead + 1)] = a_frag(p + kAhead);
       if (i == 0 && s + 1 < kSteps) unpack_step(s + 1);
       if (p < kLoads) issue_load(p, kb_next, (kb + 1) & 1);  // one load per position
       if (kW4) {
