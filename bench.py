@@ -290,6 +290,11 @@ def main() -> int:
             log("gemm", json.dumps(r))
             gemm.append(r)
         extras["prefill_gemm"] = gemm
+        # the headline kernel with 64 times the rows per launch: what it streams once the cost of
+        # launching is spread over 559 MB instead of 8.7 MB
+        tall = bench_gemv("w4", 1, 64 * 4096, 4096, 2, 10, 3, device)
+        log("tall gemv", json.dumps(tall))
+        extras["gemv_same_kernel_64x_rows_per_launch"] = tall
         dense = bench_dense_library_gemm(2048, 4096, 4096, steps=10, warmup=3, device=device)
         log("dense library gemm", json.dumps(dense))
         rate = bench_mfma_rate(device)
