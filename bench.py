@@ -361,10 +361,11 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 activations x uint4 weights, fp32 accumulate",
+        "dtype": "bf16",
         "data": "synthetic (seeded N(0,0.02) weights quantized on the GPU, N(0,1) bf16 activations)",
         "config": {
             "workload": "W4A16-g128 decode GEMV, K=N=4096, M=1 (decode sweep headline shape)",
+            "arithmetic": "bf16 activations x uint4 weights (exact integers in bf16) on MFMA, fp32 accumulate, fp16 scales applied in fp32",
             "launches_per_step": args.copies,
             "distinct_weight_bytes": args.copies * (n * k // 2 + n * k // 128 * 4),
             "launch": "HIP graph replay of one step",
