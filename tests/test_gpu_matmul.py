@@ -219,3 +219,37 @@ def test_mfma_rate_probe_runs_and_reports_clocks(cuda):
         assert cycles >= 2000 * 4 * 32 * 0.9  # four 32-cycle MFMAs per iteration, issued in order
     assert lib.ajq_probe_mfma_rate(0, 0, 8, sink.data_ptr(), clocks.data_ptr(), None, None) == -2
     assert lib.ajq_probe_mfma_rate(0, 10, 8, None, clocks.data_ptr(), None, None) == -1
+
+
+def _random_shapes(count: int, seed: int):
+    """Seeded (M, N, K) with N a multiple of 16 and K of 128, spread over the ranges where the
+    dispatch changes kernel (M = 16 / 17, 127 / 128, 255 / 256; few and many tiles)."""
+    gen = torch.Generator().manual_seed(seed)
+    pick = lambda values: values[int(torch.randint(0, len(values), (1,), generator=gen))]
+    shapes = []
+    for _ in range(count):
+        m = pick([1, 5, 16, 17, 31, 33, 64, 127, 128, 129, 200, 255, 256, 257, 384, 500, 640, 1000, 1100])
+        n = 16 * int(torch.randint(1, 400, (1,), generator=gen))
+        k = 128 * pick([1, 2, 3, 5, 8, 16, 24, 32])
+        shapes.append((m, n, k))
+    return shapes
+
+
+# three more whose size sends them to the tile kernels with ragged M and a partial last column tile
+_TILE_SHAPES = [(1000, 3088, 1024), (640, 4112, 2048), (1100, 6400, 640)]
+
+
+@pytest.mark.parametrize("m,n,k", _random_shapes(14, seed=2024) + _TILE_SHAPES)
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_matmul_random_shapes(cuda, scheme, m, n, k):
+    """Whatever kernel the library picks for the shape (GEMV, weight-streaming, 128 x 128 or 256 x 128
+    tiles), the result is the oracle's within fp32 accumulation noise; all rows are checked, the
+    reference product is formed in fp64 on the GPU from the oracle's dequantized weight."""
+    w_hat, wq, meta = _quantized(scheme, n, k, 900 + n + k, cuda)
+    x = make_activations(m, k, 7 * m + n, True).to(cuda)
+    y32 = _run(scheme, x, wq, meta, torch.float32, "auto")
+    y16 = _run(scheme, x, wq, meta, torch.bfloat16, "auto")
+    want = x.double() @ w_hat.to(cuda).double().t()
+    max_abs, rel_fro = errors(y32.double().cpu(), want.cpu())
+    assert max_abs <= 2e-3 and rel_fro <= 1e-5, (max_abs, rel_fro)
+    assert torch.equal(y16, y32.to(torch.bfloat16))
