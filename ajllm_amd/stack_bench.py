@@ -175,5 +175,19 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
                    "kv_cache_dtype": str(dec.cache.keys[0].dtype).replace("torch.", ""),
                    "first_tokens_row0": tokens[0, :8].tolist()},
     }
+    if kv_dtype is None:
+        # the same decode with a bf16 KV cache (keys and values rounded on write; arithmetic fp32):
+        # the attention's bytes halve
+        del dec
+        torch.cuda.empty_cache()
+        dec16 = decoding.FusedDecoder(model, batch, context + decode_steps + 8, torch.bfloat16)
+        dec16.prefill(prompt, rows_per_pass=PREFILL_ROWS, fused=True)
+        dec16.generate(4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec16.generate(4 + decode_steps)
+        torch.cuda.synchronize()
+        t16 = (time.perf_counter() - t0) / decode_steps
+        result["decode_bf16_kv_cache"] = {"ms_per_step": t16 * 1e3, "tok/s": batch / t16}
     log("stack", result)
     return result
