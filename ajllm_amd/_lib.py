@@ -27,6 +27,10 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_version": (c_int, []),
     "ajq_last_error": (c_char_p, []),
     "ajq_status_string": (c_char_p, [c_int]),
+    "ajq_gemm_gate_supported": (c_int, [c_int, c_int, c_int, c_int]),
+    "ajq_w4a16_gemm_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t,
+                                    c_void_p]),
+    "ajq_w8a16_gemm_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
     "ajq_probe_mfma_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w8": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w4_g128": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),

@@ -82,10 +82,10 @@ int check_matmul_args(const char* name, const void* x, int M, int K, const void*
 }
 
 // 256 x 128 tiles on 32x32x16 MFMA; M >= 256 (the last row tile is shifted, not masked)
-template <int MT, bool kW4>
+template <int MT, bool kW4, bool kGate = false>
 int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                    const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
-  auto kernel = dequant_gemm256_kernel<MT, kW4>;
+  auto kernel = dequant_gemm256_kernel<MT, kW4, kGate>;
   if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
   const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
   hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,
@@ -98,10 +98,10 @@ int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 #ifndef AJQ_G1_WN
 #define AJQ_G1_WN 4
 #endif
-template <bool kW4>
+template <bool kW4, bool kGate = false>
 int launch_gemm128(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                    const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
-  auto kernel = dequant_gemm128_kernel<kW4, AJQ_G1_WN>;
+  auto kernel = dequant_gemm128_kernel<kW4, AJQ_G1_WN, kGate>;
   constexpr size_t lds = kW4 ? kG1LdsBytesW4 : kG1LdsBytesW8;
   if (int s = allow_big_lds(kernel, lds)) return s;
   const int tiles = ((M + kG1BM - 1) / kG1BM) * ((N + kG1BN - 1) / kG1BN);
@@ -574,6 +574,52 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                                                         (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemm");
+}
+
+// ---- w1 | w3 GEMM with the SwiGLU gate formed in the epilogue (tile kernels only)
+int ajq_gemm_gate_supported(int M, int N2, int K, int w4) {
+  if (M < kG1BM || N2 < 2 * 64 || N2 % 128 != 0 || K < kGroup || K % kGroup != 0) return 0;
+  if (AJQ_G1_WN != 4) return 0;
+  return pick_matmul_kernel(M, N2, K, w4 != 0) != kStreaming;
+}
+
+int ajq_w4a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N2, uint16_t* y,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemm_gate", x, M, K, wq, meta, N2, y, AJQ_OUT_BF16, kGroup)) return s;
+  if (!ajq_gemm_gate_supported(M, N2, K, 1))
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_w4a16_gemm_gate: M=%d, N=%d, K=%d is not a tile-kernel shape with N %% 128 == 0", M,
+                N2, K);
+  const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
+  if (!workspace || workspace_bytes < need)
+    return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm_gate: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm_gate: workspace must be 16-byte aligned");
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_gate: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
+  hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
+                     K, reinterpret_cast<u32x4_t*>(workspace));
+  if (int s = pick_matmul_kernel(M, N2, K, true) == kTiles128
+                  ? launch_gemm128<true, true>(x, M, K, wq, meta, nullptr, workspace, N2, y, 0, (hipStream_t)stream)
+                  : launch_gemm256<AJQ_G2_MT_W4, true, true>(x, M, K, wq, meta, nullptr, workspace, N2, y, 0,
+                                                             (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w4a16_gemm_gate");
+}
+
+int ajq_w8a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N2, uint16_t* y,
+                        void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemm_gate", x, M, K, wq, scales, N2, y, AJQ_OUT_BF16, kGroup)) return s;
+  if (!ajq_gemm_gate_supported(M, N2, K, 0))
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_w8a16_gemm_gate: M=%d, N=%d, K=%d is not a tile-kernel shape with N %% 128 == 0", M,
+                N2, K);
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm_gate: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  if (int s = pick_matmul_kernel(M, N2, K, false) == kTiles128
+                  ? launch_gemm128<false, true>(x, M, K, wq, nullptr, scales, nullptr, N2, y, 0, (hipStream_t)stream)
+                  : launch_gemm256<AJQ_G2_MT_W8, false, true>(x, M, K, wq, nullptr, scales, nullptr, N2, y, 0,
+                                                              (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w8a16_gemm_gate");
 }
 
 }  // extern "C"

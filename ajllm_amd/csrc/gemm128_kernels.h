@@ -30,7 +30,10 @@ constexpr size_t kG1LdsBytesW8 = kG1WBase + kG1Ring * kG1W8Slot;       // 144 Ki
 // kWN = waves along N: 2 -> four waves with 64 x 64 wave tiles, 4 -> eight waves with 64 x 32
 // wave tiles (two waves per SIMD: each fetches twice the activation fragments per MFMA, but the
 // SIMD always has a second instruction stream to issue from).
-template <bool kW4, int kWN>
+// kGate (kWN = 4 only): w1 | w3 weights of a SwiGLU feed-forward, output bf16( silu(a) * u ),
+// [M, N / 2]; the workgroup's four 32-column blocks alternate between the two halves as in
+// dequant_gemm256_kernel, here one block per wave, so the pairs meet in an fp32 staging tile.
+template <bool kW4, int kWN, bool kGate = false>
 __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
     const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -57,7 +60,9 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
   // column-major walk over output tiles: consecutive workgroups share a column block of W
   const int tiles_m = (M + kG1BM - 1) / kG1BM;
   const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
-  const int m0 = min(tile_m * kG1BM, M - kG1BM), n0 = tile_n * kG1BN;  // M >= 128: the last row tile is shifted up
+  static_assert(!kGate || kWN == 4, "the gate epilogue pairs the blocks of waves 2 j and 2 j + 1");
+  const int m0 = min(tile_m * kG1BM, M - kG1BM);  // M >= 128: the last row tile is shifted up
+  const int n0 = tile_n * (kGate ? kG1BN / 2 : kG1BN);  // kGate: first of the workgroup's 64 columns of each half
   const int G = K >> 7;
   const int ntiles16 = N / kTileN;
 
@@ -72,12 +77,18 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
     a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)((slot16 ^ (4 * v + row_in)) * 16);
   const char* a_base = reinterpret_cast<const char*>(x) + (size_t)(m0 + kLoadRows * wave) * K * 2;
   const int nt16_0 = n0 / kTileN;
+  // the workgroup's T-th private 16-column tile (T = 0 .. 7) in the weight tensor; tiles past the
+  // matrix repeat the last one (their columns are never stored)
+  auto col_tile = [&](int T) -> int {
+    if (kGate) return ((T >> 1) & 1) * (ntiles16 >> 1) + nt16_0 + (T >> 2) * 2 + (T & 1);
+    return min(nt16_0 + T, ntiles16 - 1);
+  };
   constexpr int kALoads = kLoadRows / 4;
   constexpr int kBLoads = kBTiles / kWaves;
   constexpr int kLoads = kALoads + kBLoads + (kW4 ? 2 : 0);
   const uint32_t lane16 = (uint32_t)lane * 16u;
   const uint32_t meta_voff =
-      (uint32_t)((min(nt16_0 + (wave & 1) * 4 + (lane >> 4), ntiles16 - 1) * G * 16 + (lane & 15)) * 4);
+      (uint32_t)((col_tile((wave & 1) * 4 + (lane >> 4)) * G * 16 + (lane & 15)) * 4);
   auto issue_load = [&](int j, int kb, int ring) {
     if (j < kALoads) {
       const char* src = a_base + (size_t)kb * 256 + (size_t)j * 4 * K * 2;
@@ -86,9 +97,9 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
       const int T = wave * kBLoads + (j - kALoads);
       const u32x4_t* tile;
       if (kW4)
-        tile = wq + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 64;
+        tile = wq + ((size_t)col_tile(T) * G + kb) * 64;
       else
-        tile = wq + ((size_t)min(nt16_0 + (T >> 1), ntiles16 - 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
+        tile = wq + ((size_t)col_tile(T >> 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
       dma16(tile, lane16, (uint32_t)(kG1WBase + ring * kWSlot + T * 1024));
     } else if (j == kALoads + kBLoads) {
       const int e = wave & 1;  // group-sum pieces of 64 rows
@@ -251,12 +262,46 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
   // 128-bit store.  Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart)
   // use different banks.
   constexpr int kOutStride = 272;
+  // column of the weight tensor behind the wave's 32-column block t
+  auto column = [&](int t) -> int {
+    if (kGate) return (wn & 1) * (N >> 1) + n0 + (wn >> 1) * 32 + col;
+    return n0 + wn * (32 * TB) + t * 32 + col;
+  };
   float cs[TB];
 #pragma unroll
-  for (int t = 0; t < TB; ++t) cs[t] = 1.0f;
-  if (!kW4) {
+  for (int t = 0; t < TB; ++t) cs[t] = kW4 ? 1.0f : f16_bits_to_f32(scales8[min(column(t), N - 1)]);
+  if (kGate) {
+    // fp32 staging, 128 x 128 (rows 528 bytes apart): wave (wm, wn) writes its block at columns
+    // 32 wn; then a lane forms eight outputs of one row from a (block 2 j) and u (block 2 j + 1)
+    // and stores 16 bytes: out = bf16( a * sigmoid(a) * u ), [M, N / 2]
+    constexpr int kGateStride = 528;
+    const int F = N >> 1;
 #pragma unroll
-    for (int t = 0; t < TB; ++t) cs[t] = f16_bits_to_f32(scales8[min(n0 + wn * (32 * TB) + t * 32 + col, N - 1)]);
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        *reinterpret_cast<float*>(lds + row * kGateStride + (wn * 32 + col) * 4) = acc[i][0][r] * cs[0];
+      }
+    __syncthreads();
+    const int piece = lane & 7, rsub = lane >> 3;  // eight 8-column pieces per row of 64 outputs
+    const int block = (piece >> 2) * 64 + (piece & 3) * 8;  // staging column of the piece's first a
+#pragma unroll
+    for (int j = 0; j < kLoadRows / 8; ++j) {
+      const int row = wave * kLoadRows + j * 8 + rsub;
+      const float* src = reinterpret_cast<const float*>(lds + row * kGateStride) + block;
+      const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(src), a1 = *reinterpret_cast<const f32x4_t*>(src + 4);
+      const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(src + 32), u1 = *reinterpret_cast<const f32x4_t*>(src + 36);
+      float g[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        g[e] = a0[e] * (1.0f / (1.0f + expf(-a0[e]))) * u0[e];
+        g[4 + e] = a1[e] * (1.0f / (1.0f + expf(-a1[e]))) * u1[e];
+      }
+      *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * F + n0 + piece * 8) =
+          u32x4_t{pack2_bf16(g[0], g[1]), pack2_bf16(g[2], g[3]), pack2_bf16(g[4], g[5]), pack2_bf16(g[6], g[7])};
+    }
+    return;
   }
   if (!out_f32) {
 #pragma unroll

@@ -131,7 +131,12 @@ constexpr size_t kG2LdsBytes = 160 * 1024;
 
 // MT = 32-row blocks per wave: 4 -> 4 waves (2 x 2, wave tile 128 x 64), 2 -> 8 waves
 // (4 x 2, wave tile 64 x 64, two waves per SIMD).
-template <int MT, bool kW4>
+// kGate: the weights are the w1 | w3 rows of a SwiGLU feed-forward (N = 2 F, F % 64 == 0).  A
+// workgroup then takes 64 gate-projection columns and the SAME 64 up-projection columns (its
+// eight private tiles come from two places: 32-column blocks alternate between the halves, so a
+// wave's two blocks are a matching pair) and writes bf16( silu(a) * u ), [M, F]: the 4-byte
+// intermediate [M, 2 F] never exists.
+template <int MT, bool kW4, bool kGate = false>
 __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -156,7 +161,8 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   // column-major walk over output tiles: consecutive workgroups share a column block of W
   const int tiles_m = (M + kG2BM - 1) / kG2BM;
   const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
-  const int m0 = min(tile_m * kG2BM, M - kG2BM), n0 = tile_n * kG2BN;
+  const int m0 = min(tile_m * kG2BM, M - kG2BM);
+  const int n0 = tile_n * (kGate ? kG2BN / 2 : kG2BN);  // kGate: first of the workgroup's 64 columns of each half
   const int G = K >> 7;
   const int ntiles16 = N / kTileN;
 
@@ -173,6 +179,12 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     a_voff[v] = (uint32_t)row_in * (uint32_t)K * 2u + (uint32_t)((slot ^ (4 * v + row_in)) * 16);
   const char* a_base = reinterpret_cast<const char*>(x) + (size_t)(m0 + kLoadRows * wave) * K * 2;
   const int nt16_0 = n0 / kTileN;
+  // the workgroup's T-th private 16-column tile (T = 0 .. 7) in the weight tensor; tiles past the
+  // matrix repeat the last one (their columns are never stored)
+  auto col_tile = [&](int T) -> int {
+    if (kGate) return ((T >> 1) & 1) * (ntiles16 >> 1) + nt16_0 + (T >> 2) * 2 + (T & 1);
+    return min(nt16_0 + T, ntiles16 - 1);
+  };
   // The loads of one k-block are numbered 0 .. kLoads - 1 so that the main loop can issue
   // them one at a time between its MFMAs.
   constexpr int kALoads = kLoadRows / 4;
@@ -182,7 +194,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   // meta words of tile (wave & 1) * 4 + (lane >> 4) of the workgroup's eight, word (lane & 15);
   // tiles past the matrix repeat the last one (their columns are never stored)
   const uint32_t meta_voff =
-      (uint32_t)((min(nt16_0 + (wave & 1) * 4 + (lane >> 4), ntiles16 - 1) * G * 16 + (lane & 15)) * 4);
+      (uint32_t)((col_tile((wave & 1) * 4 + (lane >> 4)) * G * 16 + (lane & 15)) * 4);
   auto issue_load = [&](int j, int kb, int buf) {
     if (j < kALoads) {
       const char* src = a_base + (size_t)kb * 256 + (size_t)j * 4 * K * 2;
@@ -192,9 +204,9 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
       const int T = wave * kBLoads + (j - kALoads);
       const u32x4_t* tile;
       if (kW4)
-        tile = wq + ((size_t)min(nt16_0 + T, ntiles16 - 1) * G + kb) * 64;
+        tile = wq + ((size_t)col_tile(T) * G + kb) * 64;
       else
-        tile = wq + ((size_t)min(nt16_0 + (T >> 1), ntiles16 - 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
+        tile = wq + ((size_t)col_tile(T >> 1) * (2 * G) + 2 * kb + (T & 1)) * 64;
       dma16(tile, lane16, (uint32_t)(kWBase + buf * kG2WStride + T * 1024));
     } else if (j == kALoads + kBLoads) {
       // group-sum pieces of 64 rows; with eight waves the upper four repeat the lower four
@@ -352,10 +364,40 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   // wave-wide 128-bit store; 2-byte stores straight from the accumulators took 2-3 times as long.
   // Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart) use different banks.
   constexpr int kOutStride = 272;
+  // column of the weight tensor behind the wave's 32-column block t
+  auto column = [&](int t) -> int {
+    if (kGate) return t * (N >> 1) + n0 + wn * 32 + col;
+    return n0 + wn * 64 + t * 32 + col;
+  };
   float cs[2] = {1.0f, 1.0f};
   if (!kW4) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(n0 + wn * 64 + t * 32 + col, N - 1)]);
+    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(column(t), N - 1)]);
+  }
+  if (kGate) {
+    // block 0 holds the gate projection a, block 1 the up projection u of the same columns:
+    // out = bf16( a * sigmoid(a) * u ), [M, N / 2], staged like the plain bf16 tile (64 columns:
+    // 128-byte rows 144 bytes apart) and stored eight rows per wave-wide 128-bit store
+    constexpr int kGateStride = 144;
+    const int F = N >> 1;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        const float a = acc[i][0][r] * cs[0], u = acc[i][1][r] * cs[1];
+        *reinterpret_cast<uint16_t*>(lds + row * kGateStride + (wn * 32 + col) * 2) =
+            f32_to_bf16_rne(a * (1.0f / (1.0f + expf(-a))) * u);
+      }
+    __syncthreads();
+    const int piece = lane & 7, rsub = lane >> 3;
+#pragma unroll
+    for (int j = 0; j < kLoadRows / 8; ++j) {
+      const int row = wave * kLoadRows + j * 8 + rsub;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kGateStride + piece * 16);
+      *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * F + n0 + piece * 8) = v;
+    }
+    return;
   }
   if (!out_f32) {
 #pragma unroll
@@ -383,7 +425,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   }
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const int n = n0 + wn * 64 + t * 32 + col;
+    const int n = column(t);
     if (n >= N) continue;
 #pragma unroll
     for (int i = 0; i < MT; ++i) {

@@ -129,6 +129,30 @@ class _FusedLinear:
         fn = w8a16_matmul if self.scheme == "w8a16" else w4a16_matmul
         return fn(x_bf16, self.wq, self.meta, torch.float32)
 
+    def gate_fusable(self, rows: int) -> bool:
+        """Whether the tile GEMM with the SwiGLU gate in its epilogue takes ``rows`` rows of this
+        (w1 | w3) pair."""
+        return bool(_lib.load().ajq_gemm_gate_supported(rows, self.rows16, self.in_features,
+                                                        0 if self.scheme == "w8a16" else 1))
+
+    def gated(self, x_bf16: torch.Tensor) -> torch.Tensor:
+        """``bf16(silu(x w1^T) * (x w3^T))`` for this (w1 | w3) pair, one matmul launch (plus the W4
+        group-sum kernel): the fp32 ``[rows, 2 F]`` intermediate is never written."""
+        lib = _lib.load()
+        rows = x_bf16.shape[0]
+        y = torch.empty((rows, self.rows16 // 2), dtype=torch.bfloat16, device=x_bf16.device)
+        if self.scheme == "w8a16":
+            status = lib.ajq_w8a16_gemm_gate(x_bf16.data_ptr(), rows, self.in_features, self.wq.data_ptr(),
+                                             self.meta.data_ptr(), self.rows16, y.data_ptr(), _stream())
+        else:
+            nbytes = lib.ajq_w4a16_gemm_workspace_bytes(rows, self.in_features)
+            workspace = torch.empty((nbytes,), dtype=torch.uint8, device=x_bf16.device)
+            status = lib.ajq_w4a16_gemm_gate(x_bf16.data_ptr(), rows, self.in_features, self.wq.data_ptr(),
+                                             self.meta.data_ptr(), self.rows16, y.data_ptr(), workspace.data_ptr(),
+                                             nbytes, _stream())
+        _lib.check(status, "gemm_gate")
+        return y
+
     def fusable(self, batch: int) -> bool:
         """Whether the GEMV with a norm / gate prologue is built for this batch and input width."""
         return bool(_lib.load().ajq_gemv_fused_supported(batch, self.in_features))
@@ -263,7 +287,9 @@ class FusedDecoder(GraphDecoder):
         hidden = self.embedding[prompt.reshape(-1)]  # [rows * seq, d] fp32, row b * seq + t
         normed = torch.empty((m, d), dtype=torch.bfloat16, device=self.device)
         q_rot = torch.empty((rows, self.heads, seq, 128), dtype=torch.float32, device=self.device)
-        gated = torch.empty((m, self.d_ff), dtype=torch.bfloat16, device=self.device)
+        w13 = self.layers[0]["w13"]
+        gate_in_gemm = w13.rows16 == 2 * self.d_ff and w13.gate_fusable(m)
+        gated = None if gate_in_gemm else torch.empty((m, self.d_ff), dtype=torch.bfloat16, device=self.device)
         delta = None
         for index, w in enumerate(self.layers):
             _lib.check(lib.ajq_add_rmsnorm(hidden.data_ptr(), delta.data_ptr() if delta is not None else None,
@@ -282,9 +308,12 @@ class FusedDecoder(GraphDecoder):
             del attended
             _lib.check(lib.ajq_add_rmsnorm(hidden.data_ptr(), delta.data_ptr(), w["g2"].data_ptr(), w["eps2"],
                                            normed.data_ptr(), m, d, st), "add_rmsnorm")
-            ab = w["w13"](normed)
-            _lib.check(lib.ajq_swiglu(ab.data_ptr(), gated.data_ptr(), m, self.d_ff, st), "swiglu")
-            del ab
+            if gate_in_gemm:
+                gated = w["w13"].gated(normed)
+            else:
+                ab = w["w13"](normed)
+                _lib.check(lib.ajq_swiglu(ab.data_ptr(), gated.data_ptr(), m, self.d_ff, st), "swiglu")
+                del ab
             delta = w["w2"](gated)
         last = hidden.view(rows, seq, d)[:, -1, :].contiguous()
         last_delta = delta.view(rows, seq, -1)[:, -1, :d].contiguous()

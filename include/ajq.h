@@ -61,6 +61,20 @@ typedef enum ajq_status {
 #define AJQ_KV_F32 0
 #define AJQ_KV_BF16 1 /* rounded to nearest even on write; attention still computes in fp32 */
 
+/* The w1 | w3 matmul of a SwiGLU feed-forward with the gate formed in its epilogue:
+ * wq / meta / scales are the private tensors of the 2 F rows (w1's F rows, then w3's: the
+ * concatenation of the two layers' tensors), y[M, F] = bf16( silu(x w1^T) * (x w3^T) )
+ * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, up to its down projection); equal bit
+ * for bit to ajq_w*a16_gemm with fp32 output followed by ajq_swiglu, without the [M, 2 F] fp32
+ * intermediate.  Tile kernels only: ajq_gemm_gate_supported(M, 2 F, K, w4) says whether the shape
+ * qualifies (M >= 128, F a multiple of 64, large enough for the tile kernels); the W4 form needs
+ * the workspace of ajq_w4a16_gemm_workspace_bytes(M, K). */
+int ajq_gemm_gate_supported(int M, int N2, int K, int w4);
+int ajq_w4a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N2,
+                        uint16_t* y, void* workspace, size_t workspace_bytes, void* stream);
+int ajq_w8a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N2,
+                        uint16_t* y, void* stream);
+
 /* Device yardstick, no counterpart in the reference: every wave issues bf16 MFMAs back to
  * back from registers (no memory traffic), so launches timed by the caller give the MFMA
  * rate the GPU sustains -- with constant operands (random_operands = 0: nominal clock) or

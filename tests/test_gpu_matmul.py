@@ -253,3 +253,30 @@ def test_matmul_random_shapes(cuda, scheme, m, n, k):
     max_abs, rel_fro = errors(y32.double().cpu(), want.cpu())
     assert max_abs <= 2e-3 and rel_fro <= 1e-5, (max_abs, rel_fro)
     assert torch.equal(y16, y32.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("m,f,k", [(256, 7168, 1024), (2048, 2048, 2048), (1000, 3072, 4096), (200, 14336, 4096)])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemm_with_gate_epilogue_equals_gemm_then_swiglu(cuda, scheme, m, f, k):
+    """ajq_w*a16_gemm_gate on the (w1 | w3) rows: bit for bit the fp32 GEMM followed by ajq_swiglu
+    (both tile kernels, ragged M), and the oracle's silu(a) * u within bf16 rounding; shapes the tile
+    kernels do not take are refused."""
+    from ajllm_amd import _lib
+    from ajllm_amd.decoding import _FusedLinear
+    lib = _lib.load()
+    w_hat, wq, meta = _quantized(scheme, 2 * f, k, 77 + f, cuda)
+    x = make_activations(m, k, 5, True).to(cuda)
+    fused = _FusedLinear.__new__(_FusedLinear)
+    fused.scheme, fused.wq, fused.meta = ("w4a16_g128" if scheme == "w4" else "w8a16"), wq, meta
+    fused.in_features, fused.rows16 = k, 2 * f
+    assert fused.gate_fusable(m)
+    got = fused.gated(x)
+    ab = _run(scheme, x, wq, meta, torch.float32, "gemm")
+    want = torch.empty((m, f), dtype=torch.bfloat16, device=cuda)
+    _lib.check(lib.ajq_swiglu(ab.data_ptr(), want.data_ptr(), m, f, torch.cuda.current_stream().cuda_stream), "swiglu")
+    torch.cuda.synchronize()
+    assert got.shape == (m, f) and torch.equal(got, want)
+    ref = x.double() @ w_hat.to(cuda).double().t()
+    gate = torch.nn.functional.silu(ref[:, :f]) * ref[:, f:]
+    assert errors(got.double().cpu(), gate.cpu())[1] <= 4e-3  # bf16 output
+    assert not fused.gate_fusable(64) and lib.ajq_gemm_gate_supported(m, 2 * f + 16, k, 1) == 0
