@@ -117,10 +117,21 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
                 diverged.append({"row": row, "step": step_i, "eager_margin": float(margins[row, step_i])})
         same = min([d["step"] for d in diverged], default=NEW_TOKENS)
         t_linear = _linear_seconds_per_step(dec, batch, device)
+        # the prompt through this library's kernels only (GEMMs, add + RMSNorm, RoPE + cache write,
+        # flash attention, the gate in the w1|w3 GEMM): flash-attention arithmetic, so not the path
+        # the token comparison above uses
+        dec.prefill(prompt, fused=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.prefill(prompt, fused=True)
+        torch.cuda.synchronize()
+        t_prefill_fused = time.perf_counter() - t0
         step = t_graph / graph_steps
         r = {
             "scheme": scheme, "batch": batch, "prompt": PROMPT_LEN, "new_tokens": NEW_TOKENS,
             "prefill_s": t_prefill, "prefill_tok/s": batch * PROMPT_LEN / t_prefill,
+            "prefill_library_kernels_s": t_prefill_fused,
+            "prefill_library_kernels_tok/s": batch * PROMPT_LEN / t_prefill_fused,
             "decode_tok/s": batch * graph_steps / t_graph,
             "ms_per_step": step * 1e3,
             "eager_decode_tok/s": batch * (NEW_TOKENS - 1) / t_decode,
