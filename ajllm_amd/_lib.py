@@ -60,7 +60,7 @@ SIGNATURES: dict[str, tuple] = {
     ),
     "ajq_attn_prefill": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     ),
     "ajq_greedy_pick": (
         c_int,

@@ -13,12 +13,13 @@ import torch
 from . import _lib
 
 
-def flash_prefill(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, start: int) -> torch.Tensor:
+def flash_prefill(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, start: int,
+                  out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Causal attention of the ``T`` new positions ``start .. start + T - 1``.
 
     ``q`` fp32 ``[B, H, T, 128]`` (rotated); ``keys`` / ``values`` ``[B, Hkv, max_len, 128]`` fp32 or
     bf16 whose rows ``0 .. start + T - 1`` are filled (a KV cache, or the keys and values themselves
-    with ``start == 0``).  Returns fp32 ``[B, T, H * 128]``."""
+    with ``start == 0``).  Returns ``[B, T, H * 128]`` in ``out_dtype`` (fp32, or bf16 = its rounding)."""
     if not q.is_cuda:
         raise ValueError("flash_prefill needs tensors on a ROCm device (there is no CPU path)")
     batch, heads, seq, hd = q.shape
@@ -29,12 +30,15 @@ def flash_prefill(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, sta
         raise ValueError("flash_prefill: the caches must be float32 or bfloat16")
     if not (keys.is_contiguous() and values.is_contiguous()):
         raise ValueError("flash_prefill: the caches must be contiguous")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("flash_prefill: out_dtype must be float32 or bfloat16")
     q = q.float().contiguous()
-    out = torch.empty((batch, seq, heads * hd), dtype=torch.float32, device=q.device)
+    out = torch.empty((batch, seq, heads * hd), dtype=out_dtype, device=q.device)
     flag = _lib.AJQ_KV_F32 if keys.dtype == torch.float32 else _lib.AJQ_KV_BF16
     with torch.cuda.device(q.device):
         status = _lib.load().ajq_attn_prefill(q.data_ptr(), keys.data_ptr(), values.data_ptr(), flag, batch, heads,
                                               kv_heads, seq, start, max_len, hd, out.data_ptr(),
+                                              _lib.AJQ_OUT_F32 if out_dtype == torch.float32 else _lib.AJQ_OUT_BF16,
                                               torch.cuda.current_stream().cuda_stream)
     _lib.check(status, "attn_prefill")
     return out

@@ -799,7 +799,7 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
 }
 
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H, int Hkv,
-                     int T, int start, int max_len, int head_dim, float* out, void* stream) {
+                     int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream) {
   if (!q || !kcache || !vcache || !out) return fail(AJQ_ERR_NULL, "ajq_attn_prefill: null pointer argument");
   if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (only 128 is built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || T < 1 || start < 0 || (long long)start + T > max_len ||
@@ -808,17 +808,20 @@ int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int
                 Hkv, T, start, max_len);
   if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+  if (out_dtype != AJQ_OUT_BF16 && out_dtype != AJQ_OUT_F32)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: out_dtype %d is neither AJQ_OUT_BF16 nor AJQ_OUT_F32", out_dtype);
+  const int out_bf16 = out_dtype == AJQ_OUT_BF16;
   if (!aligned16(q) || !aligned16(kcache) || !aligned16(vcache) || !aligned16(out))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_prefill: q, the caches and out must be 16-byte aligned");
   const dim3 grid((T + kPfBQ - 1) / kPfBQ, B * H);
   if (cache_dtype == AJQ_KV_F32)
     hipLaunchKernelGGL(attn_prefill_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, q,
                        reinterpret_cast<const float*>(kcache), reinterpret_cast<const float*>(vcache), H, Hkv, T, start,
-                       max_len, out);
+                       max_len, out, out_bf16);
   else
     hipLaunchKernelGGL(attn_prefill_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, q,
                        reinterpret_cast<const uint16_t*>(kcache), reinterpret_cast<const uint16_t*>(vcache), H, Hkv, T,
-                       start, max_len, out);
+                       start, max_len, out, out_bf16);
   return check_launch("ajq_attn_prefill");
 }
 

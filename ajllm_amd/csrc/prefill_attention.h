@@ -57,7 +57,7 @@ __device__ __forceinline__ u32x4_t to_bf16x8(const u32x4_t& r) { return r; }
 template <typename CacheT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
                                                            const CacheT* __restrict__ vcache, int H, int Hkv, int T,
-                                                           int start, int max_len, float* __restrict__ out) {
+                                                           int start, int max_len, void* __restrict__ out, int out_bf16) {
   // two buffers of each: a block is laid down while the previous one is still being read
   __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][kPfBK * kPfKStride];
   __shared__ __attribute__((aligned(16))) uint16_t Vt2[2][kPfHD * kPfVStride];
@@ -218,11 +218,20 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   for (int u = 0; u < kPfQG; ++u) {
     if (qrow[u] >= T) continue;
     const float inv = 1.0f / l_run[u];
-    float* dst = out + ((size_t)b * T + qrow[u]) * ((size_t)H * kPfHD) + (size_t)h * kPfHD + 4 * g;
+    const size_t at = ((size_t)b * T + qrow[u]) * ((size_t)H * kPfHD) + (size_t)h * kPfHD + 4 * g;
+    if (out_bf16) {
+      uint16_t* dst = reinterpret_cast<uint16_t*>(out) + at;
 #pragma unroll
-    for (int t = 0; t < 8; ++t)
-      *reinterpret_cast<float4*>(dst + 16 * t) =
-          float4{o[u][t][0] * inv, o[u][t][1] * inv, o[u][t][2] * inv, o[u][t][3] * inv};
+      for (int t = 0; t < 8; ++t)
+        *reinterpret_cast<u32x2_t*>(dst + 16 * t) =
+            u32x2_t{pack2_bf16(o[u][t][0] * inv, o[u][t][1] * inv), pack2_bf16(o[u][t][2] * inv, o[u][t][3] * inv)};
+    } else {
+      float* dst = reinterpret_cast<float*>(out) + at;
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        *reinterpret_cast<float4*>(dst + 16 * t) =
+            float4{o[u][t][0] * inv, o[u][t][1] * inv, o[u][t][2] * inv, o[u][t][3] * inv};
+    }
   }
 }
 

@@ -300,11 +300,11 @@ class FusedDecoder(GraphDecoder):
                                             keys.data_ptr(), values.data_ptr(), self.kv_flag, rows, seq, self.heads,
                                             self.kv_heads, 128, 0, self.max_len, st), "rope_prefill")
             del qkv
-            attended = torch.empty((m, d), dtype=torch.float32, device=self.device)
+            attended = torch.empty((m, d), dtype=torch.bfloat16, device=self.device)
             _lib.check(lib.ajq_attn_prefill(q_rot.data_ptr(), keys.data_ptr(), values.data_ptr(), self.kv_flag, rows,
                                             self.heads, self.kv_heads, seq, 0, self.max_len, 128, attended.data_ptr(),
-                                            st), "attn_prefill")
-            delta = w["o"](attended.to(torch.bfloat16))
+                                            _lib.AJQ_OUT_BF16, st), "attn_prefill")
+            delta = w["o"](attended)
             del attended
             _lib.check(lib.ajq_add_rmsnorm(hidden.data_ptr(), delta.data_ptr(), w["g2"].data_ptr(), w["eps2"],
                                            normed.data_ptr(), m, d, st), "add_rmsnorm")

@@ -201,12 +201,13 @@ int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
 
 /* Causal attention of T new positions (absolute positions start .. start + T - 1) over cache
  * rows 0 .. start + T - 1, which the caller has already written; q fp32 [B, H, T, head_dim]
- * (rotated), out fp32 [B, T, H * head_dim].  Flash-attention arithmetic: bf16 MFMA products,
+ * (rotated), out [B, T, H * head_dim] fp32 or bf16 (out_dtype: AJQ_OUT_F32 / AJQ_OUT_BF16, the
+ * rounding of the fp32 result).  Flash-attention arithmetic: bf16 MFMA products,
  * fp32 online softmax, no T x T matrix (scaled_dot_product_attention under a causal mask,
  * src/ajllm/modeling/attention.py:20-33,106-117; the reference's own tiled and Triton variants,
  * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128 only. */
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H,
-                     int Hkv, int T, int start, int max_len, int head_dim, float* out, void* stream);
+                     int Hkv, int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream);
 
 /* Greedy choice at the end of a decode step: token[b] = argmax(logits[b, 0..V)) (row stride ld;
  * the lowest index among equal maxima: next = argmax(logits[:, -1]) of generate,

@@ -287,6 +287,8 @@ def test_flash_prefill_attention(cuda, b, heads, kv_heads, t, start, cache_dtype
     values = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
     got = flash_prefill(q, keys, values, start)
     assert got.shape == (b, t, heads * hd) and bool(torch.isfinite(got).all())
+    got16 = flash_prefill(q, keys, values, start, out_dtype=torch.bfloat16)  # the rounding of the fp32 result
+    assert got16.dtype == torch.bfloat16 and torch.equal(got16, got.to(torch.bfloat16))
     total = start + t
     rep = heads // kv_heads
     k32 = keys[:, :, :total].float().repeat_interleave(rep, dim=1)
