@@ -257,13 +257,37 @@ class QuantLinear(nn.Module):
         else:
             self.wq, self.meta = repack_w4(self.qweight, self.scales, self.zeros)
 
-    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs):
+        """Takes the canonical tensors under ``prefix``; reports an absent one in ``missing_keys`` and
+        any other key directly under the prefix (e.g. a dense ``weight`` aimed at this slot) in
+        ``unexpected_keys``, so ``load_state_dict(strict=True)`` raises as it does for the reference
+        layer (training/checkpoint.py:35-45 loads strictly)."""
+        wanted = ("qweight", "scales") + (() if self.scheme == "w8a16" else ("zeros",))
+        found = {}
         for name in ("qweight", "scales", "zeros"):
             key = prefix + name
             if key in state_dict:
-                setattr(self, name, state_dict[key].clone())
-                state_dict = {k: v for k, v in state_dict.items() if k != key}
-        if self.qweight is not None and self.qweight.is_cuda:
+                found[name] = state_dict[key]
+            elif name in wanted:
+                missing_keys.append(key)
+        for key in state_dict:
+            if key.startswith(prefix) and "." not in key[len(prefix):] and key[len(prefix):] not in (
+                    "qweight", "scales", "zeros"):
+                unexpected_keys.append(key)
+        if any(name not in found for name in wanted):
+            return  # leave the layer as it was: a partial load must not leave mixed tensors behind
+        expect_q = ((self.out_features, self.in_features) if self.scheme == "w8a16"
+                    else (self.out_features, self.in_features // 8))
+        if tuple(found["qweight"].shape) != expect_q:
+            error_msgs.append(f"size mismatch for {prefix}qweight: checkpoint {tuple(found['qweight'].shape)}, "
+                              f"layer ({self.scheme}) expects {expect_q}")
+            return
+        for name, value in found.items():
+            setattr(self, name, value.clone())
+        if self.scheme == "w8a16" and "zeros" not in found:
+            self.zeros = torch.empty(0, dtype=torch.uint8, device=self.qweight.device)
+        if self.qweight.is_cuda:
             self.prepare()
 
     def forward(self, inputs: torch.Tensor, out_dtype: torch.dtype | None = None) -> torch.Tensor:

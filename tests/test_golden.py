@@ -31,6 +31,27 @@ def test_oracle_reproduces_fixture(gold):
     w_hat = qspec.dequantize_w4(gold["w4_qweight"], gold["w4_scales_bits"].view(np.float16), gold["w4_zeros"])
     y = qspec.quant_linear(_x(gold), torch.from_numpy(w_hat), accumulate=torch.float64, out_dtype=torch.float64)
     assert np.array_equal(y.numpy(), gold["y_w4_f64"])
+    w_hat8 = qspec.dequantize_w8(gold["w8_q"], gold["w8_scales_bits"].view(np.float16))
+    y8 = qspec.quant_linear(_x(gold), torch.from_numpy(w_hat8), accumulate=torch.float64, out_dtype=torch.float64)
+    assert np.array_equal(y8.numpy(), gold["y_w8_f64"])
+
+
+def test_fixture_outputs_follow_from_its_integers(gold):
+    """The stored fp64 outputs against a sum written out in Python floats from the stored integer
+    tensors (no oracle function involved), so the fixture cannot drift together with the oracle."""
+    x = _x(gold).double().numpy()
+    q8 = gold["w8_q"].astype(np.int64)
+    s8 = gold["w8_scales_bits"].view(np.float16).astype(np.float64)
+    w_hat8 = (q8 * s8[:, None]).astype(np.float32).astype(np.float64)   # fp32 product is exact: no rounding
+    assert np.array_equal(w_hat8, q8 * s8[:, None])
+    want8 = x @ w_hat8.T
+    assert np.allclose(gold["y_w8_f64"], want8, rtol=0, atol=1e-11)
+    words = gold["w4_qweight"].view(np.uint32)
+    q4 = np.stack([(words >> (4 * j)) & 15 for j in range(8)], axis=-1).reshape(words.shape[0], -1).astype(np.int64)
+    s4 = np.repeat(gold["w4_scales_bits"].view(np.float16).astype(np.float64), 128, axis=1)
+    z4 = np.repeat(gold["w4_zeros"].astype(np.int64), 128, axis=1)
+    want4 = x @ ((q4 - z4) * s4).T
+    assert np.allclose(gold["y_w4_f64"], want4, rtol=0, atol=1e-11)
 
 
 @pytest.mark.gpu

@@ -27,6 +27,43 @@ def test_one_hot_activation_reads_single_weights():
             assert float(y[row]) == np.float32(want)
 
 
+def test_w8_one_hot_activation_reads_single_weights():
+    """The W8 twin of the test above: x = e_k returns column k of W_hat, and each entry must equal
+    int(q) * float(scale) computed in Python floats (an fp32 product of an integer below 2^7 and an
+    fp16 value is exact, so any rounding inside dequantize_w8, e.g. a product formed in fp16, fails)."""
+    n, k = 8, 256
+    w = make_weight(n, k, 11).numpy()
+    w[2] *= 37.0   # rows of different magnitude: different fp16 exponents of the scale
+    w[5] *= 1e-3
+    q, s = qspec.quantize_w8(w)
+    w_hat_np = qspec.dequantize_w8(q, s)
+    assert w_hat_np.dtype == np.float32
+    for row in range(n):
+        for col in range(k):
+            assert float(w_hat_np[row, col]) == int(q[row, col]) * float(s[row])
+    w_hat = torch.from_numpy(w_hat_np)
+    for col in (0, 63, 64, 255, 131):
+        x = torch.zeros((1, k), dtype=torch.bfloat16)
+        x[0, col] = 1.0
+        y = qspec.quant_linear(x, w_hat, out_dtype=torch.float32)[0]
+        for row in range(n):
+            assert float(y[row]) == int(q[row, col]) * float(s[row])
+    # the product must differ from one formed in fp16 somewhere, or the test would pin nothing
+    in_fp16 = (q.astype(np.float16) * s[:, None]).astype(np.float32)
+    assert not np.array_equal(in_fp16, w_hat_np)
+
+
+def test_w8_all_ones_activation_gives_row_sums():
+    n, k = 16, 512
+    q, s = qspec.quantize_w8(make_weight(n, k, 12).numpy())
+    w_hat = torch.from_numpy(qspec.dequantize_w8(q, s))
+    y = qspec.quant_linear(torch.ones((1, k), dtype=torch.bfloat16), w_hat, accumulate=torch.float64,
+                           out_dtype=torch.float64)[0]
+    for row in range(n):
+        want = float(s[row]) * int(q[row].astype(np.int64).sum())
+        assert abs(float(y[row]) - want) <= 1e-9 * max(1.0, abs(want))
+
+
 def test_all_ones_activation_gives_row_sums():
     n, k = 16, 512
     q, s, z, packed = _w4(n, k, 2)
