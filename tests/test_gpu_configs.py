@@ -1,0 +1,286 @@
+"""The two assembled benchmark configurations at full size against the CPU oracle model (the
+restated Transformer with the oracle's ``QuantLinearRef`` in every linear slot):
+
+* the 12-layer W4A16 model (d_model 2048, 16 heads, d_ff 5632, vocab 32000), prompt 512 + 256
+  greedy tokens, batch 1 and 8, through ``FusedDecoder``;
+* one Llama-3-8B-shaped W8A16 layer (d_model 4096, 32 query / 8 key-value heads, d_ff 14336,
+  vocab 128256): a batch-32 decode step at context 2048 and a 2048-token prefill.
+
+"Identical greedy tokens" is judged in two ways.  Free-running: the fused decoder's token rows
+against the oracle's, compared up to the first difference, which must sit at a step where the
+oracle's own top-1 minus top-2 logit is below the measured logit error of the two runs.
+Teacher-forced: the decode kernels fed the oracle's tokens, so that every one of the 256 steps is
+compared on the same context; a differing choice is again accepted only below the measured error.
+The numbers (identical-prefix lengths, agreement rate, margins, logit error) go to
+``gpurun_out/config4_tokens_b<batch>.json``.
+
+The oracle side takes a minute or two of CPU work per case; a heartbeat line is appended to
+``gpurun_out/config_tests_progress.log`` while it runs.
+"""
+
+import copy
+import json
+import os
+import time
+from pathlib import Path
+
+import pytest
+import torch
+
+from ajllm_amd import decoding, modeling, quantize_model_
+from oracle import qspec
+from tests.helpers import errors
+
+pytestmark = [pytest.mark.gpu, pytest.mark.timeout(900)]
+
+OUT_DIR = Path("gpurun_out")
+_t0 = time.time()
+
+
+def _beat(message: str) -> None:
+    OUT_DIR.mkdir(exist_ok=True)
+    with open(OUT_DIR / "config_tests_progress.log", "a") as fh:
+        fh.write(f"{time.time() - _t0:8.1f}s {message}\n")
+
+
+def _oracle_model_(ref: modeling.TransformerLM, scheme: str) -> modeling.TransformerLM:
+    """Swap every dense Linear of ``ref`` (a CPU model) for the oracle's QuantLinearRef, in place."""
+    for parent in list(ref.modules()):
+        for name, child in list(parent.named_children()):
+            if isinstance(child, modeling.Linear):
+                twin = qspec.QuantLinearRef.from_linear(child, scheme)
+                twin.dequantized()  # form the fp32 weight now, not inside the first timed forward
+                setattr(parent, name, twin)
+                _beat(f"oracle {scheme} {name} {tuple(twin.qweight.shape)}")
+    return ref.eval()
+
+
+# ------------------------------------------------------------------ config 4
+CONFIG4 = dict(vocab_size=32000, context_length=768, d_model=2048, num_layers=12, num_heads=16, d_ff=5632)
+PROMPT, NEW = 512, 256
+
+
+@pytest.fixture(scope="module")
+def config4(cuda):
+    torch.manual_seed(40)
+    _beat("config 4: building the dense model")
+    model = modeling.TransformerLM(**CONFIG4).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w4a16_g128")
+    ref = _oracle_model_(model, "w4a16_g128")
+    yield ref, fast
+    del ref, fast
+    torch.cuda.empty_cache()
+
+
+@torch.no_grad()
+def _oracle_greedy(ref, prompt, new_tokens):
+    """modeling.greedy_decode's loop with the logits of every step kept: tokens [B, T + new],
+    logits [B, new, V] (row t: the logits that chose new token t)."""
+    batch, prompt_len = prompt.shape
+    cache = ref.new_cache(batch, prompt_len + new_tokens)
+    tokens, logits_all = [prompt], []
+    step_input = prompt
+    for i in range(new_tokens):
+        logits = ref(step_input, cache, last_token_only=True)[:, -1, :].float()
+        logits_all.append(logits)
+        step_input = torch.argmax(logits, dim=-1, keepdim=True)
+        tokens.append(step_input)
+        if i % 32 == 0:
+            _beat(f"oracle decode step {i}")
+    return torch.cat(tokens, dim=1), torch.stack(logits_all, dim=1)
+
+
+@torch.no_grad()
+def _teacher_forced_logits(dec, prompt, ref_tokens, new_tokens):
+    """The fused decoder's logits along the oracle's token sequence: row t = logits after the
+    prompt and the oracle's first t new tokens, through the decode-step kernels (t >= 1) or the
+    prompt pass (t = 0)."""
+    dec.prefill(prompt)
+    out = []
+    prompt_len = prompt.shape[1]
+    # row 0 comes from the prompt pass; recompute it the way prefill chose its token
+    cache = dec.model.new_cache(prompt.shape[0], prompt_len + 1)
+    out.append(dec.model(prompt, cache, last_token_only=True)[:, -1, :].float().cpu())
+    del cache
+    for t in range(1, new_tokens):
+        forced = ref_tokens[:, prompt_len + t - 1].to(dec.device)
+        torch.index_select(dec.embedding, 0, forced, out=dec.embedded)
+        out.append(dec._logits().float().cpu())
+        dec.counters.add_(1)
+    return torch.stack(out, dim=1)
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_config4_greedy_tokens_against_the_oracle_model(config4, cuda, batch):
+    ref, fast = config4
+    prompt = torch.randint(0, CONFIG4["vocab_size"], (batch, PROMPT), generator=torch.Generator().manual_seed(400 + batch))
+    _beat(f"config 4 batch {batch}: oracle greedy decode")
+    ref_tokens, ref_logits = _oracle_greedy(ref, prompt, NEW)
+    top2 = torch.topk(ref_logits, 2, dim=-1).values
+    margins = top2[..., 0] - top2[..., 1]                       # [B, NEW]
+    _beat(f"config 4 batch {batch}: fused decoder")
+    dec = decoding.FusedDecoder(fast, batch, PROMPT + NEW)
+    dec.prefill(prompt.to(cuda))
+    got = torch.cat((prompt, dec.generate(NEW).cpu()), dim=1)
+    # replayed once more from the recorded graph: the same tokens, bit for bit
+    dec.prefill(prompt.to(cuda))
+    again = torch.cat((prompt, dec.generate(NEW).cpu()), dim=1)
+    assert torch.equal(got, again)
+
+    _beat(f"config 4 batch {batch}: teacher-forced pass")
+    forced = _teacher_forced_logits(dec, prompt.to(cuda), ref_tokens, NEW)  # [B, NEW, V]
+    diff = (forced.double() - ref_logits.double())
+    step_err = diff.abs().amax(dim=-1)                          # [B, NEW] max-abs logit error per step
+    rel = float(diff.norm() / ref_logits.double().norm())
+    noise = float(step_err.max())
+    pred = forced.argmax(dim=-1)
+    want = ref_tokens[:, PROMPT:]
+    disagree = pred != want
+    # a differing choice g != r needs ref[r] - ref[g] <= 2 * (that step's logit error): both runs
+    # rank their own logits correctly, so anything larger would be a wrong logit, not a near-tie
+    gap = torch.gather(ref_logits, 2, want.unsqueeze(-1)).squeeze(-1) - torch.gather(ref_logits, 2, pred.unsqueeze(-1)).squeeze(-1)
+    assert bool((gap[disagree] <= 2 * step_err[disagree] + 1e-6).all())
+    assert rel <= 2e-2, rel                                     # logits after 12 layers of bf16 activations
+    assert noise <= 0.05, noise
+
+    rows = []
+    unexplained = []
+    for b in range(batch):
+        d = (got[b, PROMPT:] != ref_tokens[b, PROMPT:]).nonzero()
+        first = int(d[0]) if len(d) else None
+        row = {"row": b, "identical_prefix": first if first is not None else NEW,
+               "teacher_forced_agreement": float((~disagree[b]).float().mean()),
+               "min_oracle_margin": float(margins[b].min())}
+        if first is not None:
+            row["oracle_margin_at_first_difference"] = float(margins[b, first])
+            row["logit_error_at_first_difference"] = float(step_err[b, first])
+            # the two runs saw the same context up to this step, so their logits differ by exactly
+            # the teacher-forced error of this step: a flip needs the oracle's margin within twice that
+            if float(margins[b, first]) > 2 * float(step_err[b, first]) + 1e-6:
+                unexplained.append(row)
+        rows.append(row)
+    report = {"config": CONFIG4, "scheme": "w4a16_g128", "batch": batch, "prompt": PROMPT, "new_tokens": NEW,
+              "logits_relative_frobenius_error": rel, "logits_max_abs_error": noise,
+              "teacher_forced_top1_agreement": float((~disagree).float().mean()),
+              "teacher_forced_disagreements": int(disagree.sum()),
+              "largest_oracle_gap_at_a_disagreement": float(gap[disagree].max()) if bool(disagree.any()) else 0.0,
+              "rows": rows}
+    OUT_DIR.mkdir(exist_ok=True)
+    (OUT_DIR / f"config4_tokens_b{batch}.json").write_text(json.dumps(report, indent=1))
+    print(json.dumps(report))
+    assert not unexplained, unexplained
+    # the choices agree on all but a few near-ties
+    assert report["teacher_forced_top1_agreement"] >= 0.97, report["teacher_forced_top1_agreement"]
+
+
+# ------------------------------------------------------------------ config 5
+CONFIG5 = dict(vocab_size=128256, context_length=2048 + 16, d_model=4096, num_layers=1, num_heads=32, num_kv_heads=8,
+               d_ff=14336)
+CONTEXT, BATCH5 = 2048, 32
+
+
+@pytest.fixture(scope="module")
+def config5(cuda):
+    torch.manual_seed(50)
+    _beat("config 5: building one dense layer + embedding + lm_head")
+    model = modeling.TransformerLM(**CONFIG5).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w8a16")
+    ref = _oracle_model_(model, "w8a16")
+    yield ref, fast
+    del ref, fast
+    torch.cuda.empty_cache()
+
+
+@torch.no_grad()
+def test_config5_decode_step_at_context_2048_against_the_oracle_layer(config5, cuda):
+    """Batch 32, one new token at position 2047 over a cache of 2047 seeded random rows (filling it
+    by a 32 x 2047-token CPU prefill would take minutes and test nothing more of the step)."""
+    ref, fast = config5
+    g = torch.Generator().manual_seed(51)
+    pos = CONTEXT - 1
+    keys = torch.randn((BATCH5, 8, pos, 128), generator=g)
+    values = torch.randn((BATCH5, 8, pos, 128), generator=g)
+    token = torch.randint(0, CONFIG5["vocab_size"], (BATCH5, 1), generator=g)
+    cache = ref.new_cache(BATCH5, CONTEXT)
+    cache.keys[0][:, :, :pos] = keys
+    cache.values[0][:, :, :pos] = values
+    cache.length = pos
+    _beat("config 5: oracle decode step")
+    want = ref(token, cache, last_token_only=True)[:, -1, :].float()
+    new_k, new_v = cache.keys[0][:, :, pos].clone(), cache.values[0][:, :, pos].clone()
+
+    dec = decoding.FusedDecoder(fast, BATCH5, CONTEXT)
+    dec.cache.keys[0][:, :, :pos] = keys.to(cuda)
+    dec.cache.values[0][:, :, :pos] = values.to(cuda)
+    dec.cache.length, dec.cache.static = pos, True
+    dec.cache.position.fill_(pos)
+    torch.index_select(dec.embedding, 0, token.view(-1).to(cuda), out=dec.embedded)
+    got = dec._logits().float().cpu()
+    assert got.shape == (BATCH5, CONFIG5["vocab_size"]) and bool(torch.isfinite(got).all())
+    max_abs, rel = errors(got, want)
+    print("config 5 decode step: max-abs", max_abs, "rel-fro", rel)
+    assert rel <= 5e-3 and max_abs <= 5e-2, (max_abs, rel)
+    # the step's key / value rows (RoPE + cache write of the fused attention kernel)
+    assert errors(dec.cache.keys[0][:, :, pos].cpu(), new_k)[1] <= 2e-3
+    assert errors(dec.cache.values[0][:, :, pos].cpu(), new_v)[1] <= 2e-3
+    # greedy choice over the 128256-entry vocabulary wherever the oracle's margin exceeds the error
+    top2 = torch.topk(want, 2, dim=-1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 2 * max_abs
+    assert int(clear.sum()) >= BATCH5 // 4
+    assert torch.equal(got.argmax(-1)[clear], want.argmax(-1)[clear])
+    # deterministic: the same step again gives the same bits
+    dec.cache.position.fill_(pos)
+    assert torch.equal(dec._logits().float().cpu(), got)
+
+
+@torch.no_grad()
+@pytest.mark.parametrize("fused", [False, True])
+def test_config5_prefill_2048_tokens_against_the_oracle_layer(config5, cuda, fused):
+    """One sequence of 2048 tokens (M = 2048 tile GEMMs on the real layer widths).  ``fused``: the
+    library-kernel prompt pass with flash-attention arithmetic (bf16 probabilities), otherwise the
+    model's own code around the library's GEMMs (fp32 masked softmax, as the oracle)."""
+    ref, fast = config5
+    prompt = torch.randint(0, CONFIG5["vocab_size"], (1, CONTEXT), generator=torch.Generator().manual_seed(52))
+    _beat(f"config 5: oracle prefill (fused={fused})")
+    cache = ref.new_cache(1, CONTEXT + 1)
+    want = ref(prompt, cache, last_token_only=True)[:, -1, :].float()
+    dec = decoding.FusedDecoder(fast, 1, CONTEXT + 8)
+    if fused:
+        got = dec._prefill_rows(prompt.to(cuda), 0).float().cpu()
+    else:
+        dec.cache.static = False
+        got = fast(prompt.to(cuda), dec.cache.rows(0, 1), last_token_only=True)[:, -1, :].float().cpu()
+    max_abs, rel = errors(got, want)
+    print("config 5 prefill fused" if fused else "config 5 prefill model code", "max-abs", max_abs, "rel-fro", rel)
+    assert rel <= (1e-2 if fused else 5e-3), (max_abs, rel)
+    # the cache rows the pass wrote, against the oracle's
+    k_err = errors(dec.cache.keys[0][0, :, :CONTEXT].cpu(), cache.keys[0][0, :, :CONTEXT])[1]
+    v_err = errors(dec.cache.values[0][0, :, :CONTEXT].cpu(), cache.values[0][0, :, :CONTEXT])[1]
+    assert k_err <= 2e-3 and v_err <= 2e-3, (k_err, v_err)
+
+
+@torch.no_grad()
+def test_config5_stack_properties(cuda):
+    """Four layers of the stack at full width (the 32-layer stack is the benchmark's): finite,
+    run-to-run identical, and the library-kernel prompt pass agrees with the model-code pass."""
+    from ajllm_amd.e2e_bench import build_quantized_model
+
+    config = dict(CONFIG5, num_layers=4, vocab_size=32000)
+    model = build_quantized_model(cuda, "w8a16", seed=53, config=config)
+    for layer in model.layers:
+        layer.attention.use_flash_attention = True
+    prompt = torch.randint(0, 32000, (2, 1024), generator=torch.Generator().manual_seed(54)).to(cuda)
+    dec = decoding.FusedDecoder(model, 2, 1024 + 40)
+    a = dec._prefill_rows(prompt, 0).float()
+    b = dec._prefill_rows(prompt, 0).float()
+    assert bool(torch.isfinite(a).all()) and torch.equal(a, b)
+    dec.cache.static = False
+    c = model(prompt, dec.cache.rows(0, 2), last_token_only=True)[:, -1, :].float()
+    assert errors(a, c)[1] <= 1e-2
+    dec.prefill(prompt, fused=True)
+    t1 = dec.generate(32).clone()
+    dec.prefill(prompt, fused=True)
+    t2 = dec.generate(32)
+    assert torch.equal(t1, t2) and int(t1.min()) >= 0 and int(t1.max()) < 32000
+    del dec, model
+    torch.cuda.empty_cache()

@@ -280,3 +280,55 @@ def test_gemm_with_gate_epilogue_equals_gemm_then_swiglu(cuda, scheme, m, f, k):
     gate = torch.nn.functional.silu(ref[:, :f]) * ref[:, f:]
     assert errors(got.double().cpu(), gate.cpu())[1] <= 4e-3  # bf16 output
     assert not fused.gate_fusable(64) and lib.ajq_gemm_gate_supported(m, 2 * f + 16, k, 1) == 0
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+@pytest.mark.parametrize("m,k", [(1, 1024), (3, 2048), (16, 2048), (1, 4096), (8, 4096), (2, 5632), (8, 5632)])
+def test_gemv_with_norm_or_gate_prologue_against_the_oracle(cuda, scheme, m, k):
+    """ajq_w*a16_gemv_norm / _gate against the oracle product: the activations are formed on the CPU
+    exactly as the model code forms them (RMSNorm in fp32 then a bf16 cast, layers.py:70-74 behind the
+    residual add of transformer.py:45-50; silu(a) * u, activations.py:24-25) and multiplied with the
+    oracle's dequantized weight in fp64.  Tolerances are the north-star ones (max-abs 1e-2, relative
+    Frobenius 2e-3); a differently ordered sum of squares on the GPU may round a few activations to
+    the neighbouring bf16 value, which is far inside them."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    n = 272
+    w_hat, wq, meta = _quantized(scheme, n, k, 300 + k, cuda)
+    assert lib.ajq_gemv_fused_supported(m, k) == 1
+    g = torch.Generator().manual_seed(9 * m + k)
+    h = torch.randn((m, k), generator=g)
+    d = torch.randn((m, k), generator=g) * 0.5
+    gain = torch.rand(k, generator=g) + 0.5
+    eps = 1e-5
+    norm_fn = lib.ajq_w4a16_gemv_norm if scheme == "w4" else lib.ajq_w8a16_gemv_norm
+    gate_fn = lib.ajq_w4a16_gemv_gate if scheme == "w4" else lib.ajq_w8a16_gemv_gate
+    for delta in (d, None):
+        hg, gg = h.to(cuda), gain.to(cuda)
+        dg = delta.to(cuda) if delta is not None else None
+        h_out = torch.zeros((m, k), dtype=torch.float32, device=cuda)
+        y = torch.empty((m, n), dtype=torch.float32, device=cuda)
+        _lib.check(norm_fn(hg.data_ptr(), dg.data_ptr() if dg is not None else None, gg.data_ptr(), eps,
+                           h_out.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32, st),
+                   "gemv_norm")
+        torch.cuda.synchronize()
+        s = h + delta if delta is not None else h.clone()
+        assert torch.equal(h_out.cpu(), s)                      # the updated residual stream, one fp32 add
+        rms = torch.sqrt(torch.mean(s.square(), dim=-1, keepdim=True) + eps)
+        x = ((s / rms) * gain).to(torch.bfloat16)
+        want = qspec.quant_linear(x, w_hat, accumulate=torch.float64, out_dtype=torch.float64)
+        max_abs, rel = errors(y.cpu(), want)
+        assert max_abs <= MAX_ABS_TOL and rel <= REL_FRO_TOL, (max_abs, rel)
+        assert max_abs <= 3e-3, max_abs
+    ab = torch.randn((m, 2 * k), generator=g) * 2
+    y = torch.empty((m, n), dtype=torch.float32, device=cuda)
+    abg = ab.to(cuda)
+    _lib.check(gate_fn(abg.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32, st),
+               "gemv_gate")
+    torch.cuda.synchronize()
+    a, u = ab[:, :k], ab[:, k:]
+    x = (a * torch.sigmoid(a) * u).to(torch.bfloat16)           # silu(a) * u as activations.py:11-25 writes it
+    want = qspec.quant_linear(x, w_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    max_abs, rel = errors(y.cpu(), want)
+    assert max_abs <= MAX_ABS_TOL and rel <= REL_FRO_TOL, (max_abs, rel)

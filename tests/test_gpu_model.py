@@ -471,6 +471,58 @@ def test_fused_decoder_tokens_match_the_oracle_model(cuda):
     assert report["identical_rows"] + len(report["attributable"]) == 4
 
 
+@pytest.mark.parametrize("scheme,batch", [("w4a16_g128", 1), ("w8a16", 4)])
+def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme, batch):
+    """Widths the prologue GEMVs are built for (d_model 1024, d_ff 2048, grouped-query heads), with the
+    norm and gate prologues forced on: the graph-replayed tokens against the CPU oracle model, and the
+    decode-step logits of every step along the oracle's tokens against the oracle's logits."""
+    torch.manual_seed(16)
+    model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=1024, num_layers=3, num_heads=8,
+                                   d_ff=2048, num_kv_heads=4).eval()
+    ref = _oracle_model(model, scheme)
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    prompt = torch.randint(0, 2048, (batch, 48), generator=torch.Generator().manual_seed(13))
+    new = 48
+    with torch.no_grad():
+        cache = ref.new_cache(batch, 48 + new)
+        step_input, ref_new, ref_logits = prompt, [], []
+        for _ in range(new):
+            logits = ref(step_input, cache, last_token_only=True)[:, -1, :].float()
+            step_input = logits.argmax(-1, keepdim=True)
+            ref_new.append(step_input)
+            ref_logits.append(logits)
+    ref_new, ref_logits = torch.cat(ref_new, 1), torch.stack(ref_logits, 1)
+    top2 = torch.topk(ref_logits, 2, dim=-1).values
+    margins = top2[..., 0] - top2[..., 1]
+    dec = decoding.FusedDecoder(fast, batch, 48 + new)
+    assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
+    dec.fuse_norm = dec.fuse_gate = True
+    dec.prefill(prompt.to(cuda))
+    got = dec.generate(new).cpu()
+    # teacher-forced: decode-step logits along the oracle's tokens
+    dec.prefill(prompt.to(cuda))
+    forced = []
+    with torch.no_grad():
+        for t in range(1, new):
+            torch.index_select(dec.embedding, 0, ref_new[:, t - 1].to(cuda), out=dec.embedded)
+            forced.append(dec._logits().float().cpu())
+            dec.counters.add_(1)
+    forced = torch.stack(forced, 1)                              # rows t = 1 .. new - 1
+    diff = forced.double() - ref_logits[:, 1:].double()
+    step_err = torch.cat((torch.zeros(batch, 1, dtype=torch.float64), diff.abs().amax(-1)), 1)
+    rel = float(diff.norm() / ref_logits[:, 1:].double().norm())
+    print(scheme, batch, "teacher-forced logits rel", rel, "max-abs", float(step_err.max()))
+    assert rel <= 1e-2, rel
+    pred = forced.argmax(-1)
+    disagree = pred != ref_new[:, 1:]
+    assert bool((margins[:, 1:][disagree] <= 2 * step_err[:, 1:][disagree] + 1e-6).all())
+    for b in range(batch):
+        d = (got[b] != ref_new[b]).nonzero()
+        if len(d) and int(d[0]) > 0:
+            first = int(d[0])
+            assert float(margins[b, first]) <= 2 * float(step_err[b, first]) + 1e-6, (b, first)
+
+
 def test_quantized_checkpoint_round_trip(cuda, tmp_path):
     """save_quantized -> load_quantized gives a model with the same canonical tensors and the same
     logits; a dense reference-style checkpoint converts to the same file contents; a flipped byte is
