@@ -46,6 +46,8 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "ajq_w8a16_gemm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ajq_noalloc_scratch_bytes": (c_size_t, []),
+    "ajq_w4a16_gemm_noalloc": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_add_rmsnorm": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p]),
     "ajq_rope_cache": (
         c_int,

@@ -1,5 +1,6 @@
 // C ABI of libajq.so: argument validation, launch geometry, error reporting.
 #include <stdarg.h>
+#include <atomic>
 #include <stdio.h>
 
 #include "ajq_common.h"
@@ -37,6 +38,33 @@ int check_launch(const char* what) {
 }
 
 constexpr int kMaxGemvM = 16;
+
+// ---- scratch of the entry point that allocates nothing (ajq_w4a16_gemm_noalloc): the per-row,
+// per-group activation sums of the W4 tile kernels.  Every GPU the library runs on holds its own
+// copy of the array at its own address until the process ends; host code never uses the array's
+// name as an address, only the device address that hipGetSymbolAddress returns for the current
+// device.
+constexpr size_t kScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, resolved once per device.
+int scratch_address(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(AJQ_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(AJQ_ERR_UNSUPPORTED, "device index %d is outside 0..%d", dev, kMaxDevices - 1);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(AJQ_ERR_HIP, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread resolves the same address
+  }
+  *out = ptr;
+  return AJQ_OK;
+}
 
 // Kernels that stage more than 64 KiB in LDS must be opted in once per process
 // (and per device); the largest size granted so far is remembered per kernel and device.
@@ -554,6 +582,21 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                                                        (hipStream_t)stream))
     return s;
   return check_launch("ajq_w4a16_gemm");
+}
+
+size_t ajq_noalloc_scratch_bytes(void) { return kScratchBytes; }
+
+int ajq_w4a16_gemm_noalloc(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                           int out_dtype, void* stream) {
+  if (M < 1 || K < 1) return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_noalloc: M and K must be positive (got %d, %d)", M, K);
+  const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
+  if (need > kScratchBytes)
+    return fail(AJQ_ERR_WORKSPACE,
+                "ajq_w4a16_gemm_noalloc: M=%d, K=%d needs %zu bytes of group sums, the built-in scratch holds %zu "
+                "(use ajq_w4a16_gemm with a caller workspace)", M, K, need, kScratchBytes);
+  void* ptr = nullptr;
+  if (int s = scratch_address(&ptr)) return s;
+  return ajq_w4a16_gemm(x, M, K, wq, meta, N, y, out_dtype, ptr, kScratchBytes, stream);
 }
 
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,

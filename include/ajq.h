@@ -153,6 +153,18 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
+/* ajq_w4a16_gemm for callers that cannot allocate device memory or pass a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the group sums live in
+ * a 16 MiB array inside the library's code object, one copy per GPU, held until the process ends
+ * (ajq_noalloc_scratch_bytes() returns its size).  No counterpart in the reference.  The call
+ * allocates and frees nothing; shapes whose ajq_w4a16_gemm_workspace_bytes(M, K) exceeds the
+ * array return AJQ_ERR_WORKSPACE.  All calls on one GPU share the array: two calls that overlap
+ * in time on one GPU (different streams, or threads) race on it; calls on one stream do not.
+ * The first call on a device resolves the array's address and should not run under capture. */
+size_t ajq_noalloc_scratch_bytes(void);
+int ajq_w4a16_gemm_noalloc(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                           void* y, int out_dtype, void* stream);
+
 /* ---- the small operators of one decode step around the linears -------------------
  * fp32 residual stream; fp32 or bf16 KV cache (cache_dtype); outputs that feed a linear are bf16.  `pos` is a
  * DEVICE pointer to the step's cache row, so a recorded HIP graph replays per token. */
