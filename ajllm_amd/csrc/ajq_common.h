@@ -37,15 +37,42 @@ __device__ __forceinline__ u32x4_t w4_to_bf16_biased(uint32_t w) {
   return r;
 }
 
-// Four int8 (one dword, k order) -> two dwords of bf16 pairs, exact: one SDWA
-// convert per byte (sign-extending byte select), one v_perm_b32 per pair.
-// |q| <= 127 has at most 7 significant bits, so the high half of the fp32 IS the bf16.
+// The constants of the W4 unpack as run-time values, the nibble mask in an SGPR and the bf16 bias
+// (128.0 twice) in a VGPR: a VOP3 instruction takes no literal on this target, so from
+// (w & mask) | bias the compiler forms one v_and_or_b32 only if both already sit in registers
+// (with literals it emits an AND and an OR).  The asm statements are empty: they hide the values
+// from constant folding and contain no instruction.
+struct W4Consts {
+  uint32_t mask, bias;
+};
+__device__ __forceinline__ W4Consts w4_consts() {
+  W4Consts c{0x000F000Fu, 0x43004300u};
+  asm volatile("" : "+s"(c.mask));
+  asm volatile("" : "+v"(c.bias));
+  return c;
+}
+
+// private W4 dword -> 8 bf16 holding 128+q (see w4_to_bf16_biased): 3 shifts + 4 v_and_or_b32.
+// Plain C on purpose: the compiler pads the wait states between an MFMA and a VALU instruction
+// that touches its registers only for instructions it can see, not for the text of an asm.
+__device__ __forceinline__ u32x4_t w4_unpack(uint32_t w, W4Consts c) {
+  u32x4_t r;
+  r.x = (w & c.mask) | c.bias;
+  r.y = ((w >> 4) & c.mask) | c.bias;
+  r.z = ((w >> 8) & c.mask) | c.bias;
+  r.w = ((w >> 12) & c.mask) | c.bias;
+  return r;
+}
+
+// Four int8 (one dword, k order) -> two dwords of bf16 pairs, exact: the compiler turns each
+// sign-extending byte extract + convert into one v_cvt_f32_i32 with an SDWA byte select, and one
+// v_perm_b32 per pair takes the high halves.  |q| <= 127 has at most 7 significant bits, so the
+// high half of the fp32 IS the bf16.
 __device__ __forceinline__ u32x2_t w8_to_bf16(uint32_t w) {
-  float f0, f1, f2, f3;
-  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(f0) : "v"(w));
-  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(f1) : "v"(w));
-  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(f2) : "v"(w));
-  asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(f3) : "v"(w));
+  const float f0 = (float)(int)(int8_t)(w);
+  const float f1 = (float)(int)(int8_t)(w >> 8);
+  const float f2 = (float)(int)(int8_t)(w >> 16);
+  const float f3 = (float)((int)w >> 24);
   u32x2_t r;
   r.x = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
   r.y = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);

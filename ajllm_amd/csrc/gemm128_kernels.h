@@ -137,9 +137,7 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
   __syncthreads();
 
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));
+  const W4Consts w4c = w4_consts();
 
   int ring = 0;  // slot of the current block
   for (int kb = 0; kb < G; ++kb) {
@@ -174,7 +172,7 @@ __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
       for (int t = 0; t < TB; ++t) {
         if (kW4) {
           if (s < 8) {
-            bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], mask, magic);
+            bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], w4c);
           } else {
             // ninth step: -(128 + z) against the three pieces of the group sum (lanes kh = 0 only)
             const uint32_t z = (mraw[t] >> 19) & 0xFu;  // fp16(128 + z): z sits in mantissa bits 3..6

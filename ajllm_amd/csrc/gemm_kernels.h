@@ -247,13 +247,12 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));
+  const W4Consts w4c = w4_consts();
 
   for (int kb = 0; kb < G; ++kb) {
     // Loads are issued unconditionally (the last block is simply fetched again): a branch
-    // between the MFMAs would cut the loop body into separately scheduled pieces.
+    // between the MFMAs would cut the loop body into separately scheduled pieces (results are
+    // the same either way; the parity tests pass with the branch too).
     const int kb_next = min(kb + 1, G - 1);
 
     // ---- this block's packed weights, LDS -> registers (W8: the second 64-k tile is
@@ -284,7 +283,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
       for (int t = 0; t < 2; ++t) {
         if (kW4) {
           if (s < 8) {
-            bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], mask, magic);
+            bf[t][s] = w4_unpack(raw[t][s & 1][s >> 1], w4c);
           } else {
             // ninth step: -(128 + z) against the three pieces of the group sum (lanes kh = 0 only)
             const uint32_t z = (mraw[t] >> 19) & 0xFu;  // fp16(128 + z): z sits in mantissa bits 3..6

@@ -171,9 +171,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   }
 
   // ---- the matmul, as in dequant_gemv_kernel
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));
+  const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -184,11 +182,9 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-        part = mfma16(a, w4_unpack(w[p][0][j], mask, magic), part);
+        part = mfma16(a, w4_unpack(w[p][0][j], w4c), part);
         asum = mfma16(a, ones, asum);
       }
-      // all four components stay live for the compiler (see dequant_gemv_kernel)
-      asm volatile("" : "+v"(part), "+v"(asum));
 #pragma unroll
       for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
     }

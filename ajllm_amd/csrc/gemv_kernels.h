@@ -28,23 +28,6 @@
 
 namespace ajq {
 
-__device__ __forceinline__ uint32_t and_or_b32(uint32_t a, uint32_t mask_sgpr, uint32_t magic_vgpr) {
-  uint32_t r;
-  // VOP3 on gfx9 takes no literal: the mask rides in an SGPR, the magic in a VGPR
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask_sgpr), "v"(magic_vgpr));
-  return r;
-}
-
-// private W4 dword -> 8 bf16 holding 128+q (see w4_to_bf16_biased), 7 VALU ops
-__device__ __forceinline__ u32x4_t w4_unpack(uint32_t w, uint32_t mask, uint32_t magic) {
-  u32x4_t r;
-  r.x = and_or_b32(w, mask, magic);
-  r.y = and_or_b32(w >> 4, mask, magic);
-  r.z = and_or_b32(w >> 8, mask, magic);
-  r.w = and_or_b32(w >> 12, mask, magic);
-  return r;
-}
-
 // One batch of a wave: TPW consecutive k groups, their weights, meta words and the
 // matching slice of the activations, all in registers.
 template <int TPW, int kXLoads, int kLoadsPerGroup>
@@ -123,9 +106,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));  // keep it in a VGPR for v_and_or_b32
+  const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const int row = min(nl, M - 1);
   const uint16_t* xrow = xs + row * kStride + 8 * kc;
@@ -163,13 +144,9 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
             const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-            part = mfma16(a, w4_unpack(b.w[p][0][j], mask, magic), part);
+            part = mfma16(a, w4_unpack(b.w[p][0][j], w4c), part);
             asum = mfma16(a, ones, asum);
           }
-          // All four components stay live for the compiler.  With the components of unused
-          // rows dead (MROWS < 4) it reuses their registers while the MFMAs that still write
-          // them are in flight: the 16-wave configuration returned garbage that way.
-          asm volatile("" : "+v"(part), "+v"(asum));
           // (128+q) and (128+z) cancel in fp32 before the scale is applied
 #pragma unroll
           for (int i = 0; i < (MROWS < 4 ? MROWS : 4); ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[i]);
@@ -328,9 +305,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_mt_kernel(
         *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = xv[i];
     }
   }
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));
+  const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
   // group sums of the activations (zero-point term), once for all row tiles
@@ -360,9 +335,8 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_mt_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-          part = mfma16(a, w4_unpack(b.w[p][0][j], mask, magic), part);
+          part = mfma16(a, w4_unpack(b.w[p][0][j], w4c), part);
         }
-        asm volatile("" : "+v"(part));  // all four components live: see dequant_gemv_kernel
 #pragma unroll
         for (int i = 0; i < kLive; ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[p][i]);
       }

@@ -108,9 +108,7 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  const uint32_t mask = 0x000F000Fu;
-  uint32_t magic = 0x43004300u;
-  asm volatile("" : "+v"(magic));  // keep it in a VGPR for v_and_or_b32
+  const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + nl * kStride + 8 * kc;  // A fragment of row block 0; block b is 16 rows further
   f32x4_t acc[NT][MB];
@@ -152,7 +150,7 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
           for (int j = 0; j < 4; ++j) {
             u32x4_t w[NT];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) w[t] = w4_unpack(b.w[t][p][0][j], mask, magic);
+            for (int t = 0; t < NT; ++t) w[t] = w4_unpack(b.w[t][p][0][j], w4c);
 #pragma unroll
             for (int r = 0; r < MB; ++r) {
               const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + r * 16 * kStride + p * kGroup + 32 * j);
