@@ -66,7 +66,16 @@ SIGNATURES: dict[str, tuple] = {
     ),
     "ajq_greedy_pick": (
         c_int,
-        [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p],
+        [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "ajq_gemv_merge_max_splits": (c_int, [c_int, c_int]),
+    "ajq_w4a16_gemv_merge": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ajq_w8a16_gemv_merge": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
+    "ajq_attn_step_partial": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+         c_int, c_void_p, c_void_p, c_size_t, c_void_p],
     ),
     "ajq_gemv_fused_supported": (c_int, [c_int, c_int]),
     "ajq_w4a16_gemv_norm": (

@@ -398,13 +398,13 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
 template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
 int launch_gemv_pro_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
                         int out_f32, const float* src0, const float* src1, const float* gain, float eps, float* h_out,
-                        hipStream_t stream) {
+                        hipStream_t stream, int S = 0) {
   constexpr size_t lds = gemv_pro_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
   auto kernel = dequant_gemv_pro_kernel<kWaves, TPW, MROWS, kW4, kPro>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
-                     meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out);
+                     meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out, S);
   return AJQ_OK;
 }
 
@@ -445,6 +445,33 @@ int launch_gemv_pro(int M, int K, const uint32_t* wq, const uint32_t* meta, cons
   if (M <= 4) AJQ_PRO(11, 4, 4);
   AJQ_PRO(11, 4, 8);
 #undef AJQ_PRO
+}
+
+// The output projection with the attention's row chunks merged on its way in: K = heads * 128 with
+// K = 2048 (eight waves of two heads) or 4096 (eight waves of four); a lane holds at most
+// merge_chunks_per_lane chunks of a (row, head), the four lane quarters every fourth chunk.
+int gemv_merge_max_splits(int M, int K) {
+  const int tpw = K == 2048 ? 2 : K == 4096 ? 4 : 0;
+  if (!tpw || M < 1) return 0;
+  const int mrows = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : 0;
+  if (!mrows || mrows * tpw > 8) return 0;
+  return 4 * merge_chunks_per_lane(mrows, tpw);
+}
+
+template <bool kW4>
+int launch_gemv_merge(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
+                      int out_f32, const float* partial, int S, hipStream_t stream) {
+#define AJQ_MRG(T, R) \
+  return launch_gemv_pro_cfg<8, T, R, kW4, kProMerge>(M, K, wq, meta, scales8, N, y, out_f32, partial, nullptr, nullptr, \
+                                                      0.f, nullptr, stream, S)
+  if (K == 2048) {
+    if (M <= 1) AJQ_MRG(2, 1);
+    if (M <= 2) AJQ_MRG(2, 2);
+    AJQ_MRG(2, 4);
+  }
+  if (M <= 1) AJQ_MRG(4, 1);
+  AJQ_MRG(4, 2);
+#undef AJQ_MRG
 }
 
 int check_pro(const char* name, int M, int K, const void* a, const void* b) {
@@ -549,6 +576,34 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
                                                nullptr, 0.f, nullptr, (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemv_gate");
+}
+
+int ajq_gemv_merge_max_splits(int M, int K) { return gemv_merge_max_splits(M, K); }
+
+int ajq_w4a16_gemv_merge(const float* partial, int S, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                         void* y, int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w4a16_gemv_merge", partial, M, K, wq, meta, N, y, out_dtype, kGroup)) return s;
+  const int cap = gemv_merge_max_splits(M, K);
+  if (cap == 0 || S < 1 || S > cap)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_w4a16_gemv_merge: M=%d, K=%d, S=%d is not built (ajq_gemv_merge_max_splits gives %d)",
+                M, K, S, cap);
+  if (int s = launch_gemv_merge<true>(M, K, wq, meta, nullptr, N, y, out_dtype == AJQ_OUT_F32, partial, S,
+                                      (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w4a16_gemv_merge");
+}
+
+int ajq_w8a16_gemv_merge(const float* partial, int S, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                         void* y, int out_dtype, void* stream) {
+  if (int s = check_matmul_args("ajq_w8a16_gemv_merge", partial, M, K, wq, scales, N, y, out_dtype, kGroup)) return s;
+  const int cap = gemv_merge_max_splits(M, K);
+  if (cap == 0 || S < 1 || S > cap)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_w8a16_gemv_merge: M=%d, K=%d, S=%d is not built (ajq_gemv_merge_max_splits gives %d)",
+                M, K, S, cap);
+  if (int s = launch_gemv_merge<false>(M, K, wq, nullptr, scales, N, y, out_dtype == AJQ_OUT_F32, partial, S,
+                                       (hipStream_t)stream))
+    return s;
+  return check_launch("ajq_w8a16_gemv_merge");
 }
 
 // --------------------------------------------------------------- GEMM -----
@@ -691,7 +746,7 @@ void launch_attn(const float* q, void* kcache, void* vcache, const long long* po
   hipLaunchKernelGGL((attn_decode_kernel<R, CacheT, kStep>), dim3(B * Hkv, S), dim3(256), 0, stream, q,
                      reinterpret_cast<CacheT*>(kcache), reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale,
                      partial, out, cosine, sine);
-  if (S > 1)
+  if (S > 1 && out != nullptr)  // out == nullptr: the caller merges the chunks itself (ajq_w*a16_gemv_merge)
     hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, stream, partial, S, out);
 }
 
@@ -768,7 +823,7 @@ int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, f
 size_t ajq_attn_decode_workspace_bytes(int B, int H) {
   if (B < 1 || H < 1) return 0;
   // sized for the largest split count: the number of cache heads is not known here
-  return (size_t)B * H * kAttnMaxSplits * 130 * sizeof(float);
+  return (size_t)B * H * kAttnMaxSplits * kAttnPartialStride * sizeof(float);
 }
 
 int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, const int64_t* pos, int B,
@@ -801,43 +856,68 @@ size_t ajq_attn_step_workspace_bytes(int B, int H) {
   return ajq_attn_decode_workspace_bytes(B, H);
 }
 
-int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, void* kcache,
-                  void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
-                  void* workspace, size_t workspace_bytes, void* stream) {
-  if (!qkv || !cosine || !sine || !pos || !kcache || !vcache || !out)
-    return fail(AJQ_ERR_NULL, "ajq_attn_step: null pointer argument");
-  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: head_dim %d (only 128 is built)", head_dim);
+namespace {
+// out != nullptr: bf16 attention output (merged by a second launch when there are several row
+// chunks); out == nullptr: the chunks' partial results stay in the workspace, at most max_splits of them
+int attn_step_impl(const char* name, const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
+                   void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len,
+                   uint16_t* out, int max_splits, int* splits, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!qkv || !cosine || !sine || !pos || !kcache || !vcache) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "%s: head_dim %d (only 128 is built)", name, head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
-    return fail(AJQ_ERR_SHAPE, "ajq_attn_step: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
+    return fail(AJQ_ERR_SHAPE, "%s: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", name, B, H, Hkv, max_len);
   const int R = H / Hkv;
   if (R != 1 && R != 2 && R != 4)
-    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: %d query heads per cache head (1, 2 and 4 are built)", R);
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: %d query heads per cache head (1, 2 and 4 are built)", name, R);
   if (cache_dtype != AJQ_KV_F32 && cache_dtype != AJQ_KV_BF16)
-    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_step: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", name, cache_dtype);
   if (!aligned16(qkv) || !aligned16(cosine) || !aligned16(sine) || !aligned16(kcache) || !aligned16(vcache))
-    return fail(AJQ_ERR_ALIGN, "ajq_attn_step: qkv, the tables and the caches must be 16-byte aligned");
-  const int S = attn_splits(B, Hkv, max_len);
-  if (S > 1 && (!workspace || workspace_bytes < ajq_attn_step_workspace_bytes(B, H) || !aligned16(workspace)))
-    return fail(AJQ_ERR_WORKSPACE, "ajq_attn_step: 16-byte aligned workspace of %zu bytes needed, %zu given",
+    return fail(AJQ_ERR_ALIGN, "%s: qkv, the tables and the caches must be 16-byte aligned", name);
+  int S = attn_splits(B, Hkv, max_len);
+  if (S > max_splits) S = max_splits;
+  if ((S > 1 || !out) && (!workspace || workspace_bytes < ajq_attn_step_workspace_bytes(B, H) || !aligned16(workspace)))
+    return fail(AJQ_ERR_WORKSPACE, "%s: 16-byte aligned workspace of %zu bytes needed, %zu given", name,
                 ajq_attn_step_workspace_bytes(B, H), workspace_bytes);
+  if (splits) *splits = S;
   const float scale = 1.0f / sqrtf((float)head_dim);
   pick_attn<true>(R, cache_dtype)(qkv, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len,
                                   scale, S, reinterpret_cast<float*>(workspace), out, cosine, sine,
                                   (hipStream_t)stream);
-  return check_launch("ajq_attn_step");
+  return check_launch(name);
+}
+}  // namespace
+
+int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, void* kcache,
+                  void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+  if (!out) return fail(AJQ_ERR_NULL, "ajq_attn_step: null pointer argument");
+  return attn_step_impl("ajq_attn_step", qkv, cosine, sine, pos, kcache, vcache, cache_dtype, B, H, Hkv, head_dim,
+                        max_len, out, kAttnMaxSplits, nullptr, workspace, workspace_bytes, stream);
+}
+
+int ajq_attn_step_partial(const float* qkv, const float* cosine, const float* sine, const int64_t* pos, void* kcache,
+                          void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len,
+                          int max_splits, int* splits, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!splits) return fail(AJQ_ERR_NULL, "ajq_attn_step_partial: splits must point to an int");
+  if (max_splits < 1) return fail(AJQ_ERR_SHAPE, "ajq_attn_step_partial: max_splits must be at least 1");
+  return attn_step_impl("ajq_attn_step_partial", qkv, cosine, sine, pos, kcache, vcache, cache_dtype, B, H, Hkv,
+                        head_dim, max_len, nullptr, max_splits, splits, workspace, workspace_bytes, stream);
 }
 
 int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embedding, int D, float* hidden,
-                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, void* stream) {
+                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, int64_t* advance, uint32_t* ticket,
+                    void* stream) {
   if (!logits || !embedding || !hidden || !token || !out || !step)
     return fail(AJQ_ERR_NULL, "ajq_greedy_pick: null pointer argument");
+  if ((advance != nullptr) != (ticket != nullptr))
+    return fail(AJQ_ERR_NULL, "ajq_greedy_pick: advance and ticket go together (both or neither)");
   if (B < 1 || V < 1 || ld < V || ld % 4 != 0 || D < 4 || D % 4 != 0 || out_ld < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_greedy_pick: unsupported shape (B=%d V=%d ld=%d D=%d out_ld=%d)", B, V, ld, D, out_ld);
   if (!aligned16(logits) || !aligned16(embedding) || !aligned16(hidden))
     return fail(AJQ_ERR_ALIGN, "ajq_greedy_pick: logits, embedding and hidden must be 16-byte aligned");
   hipLaunchKernelGGL(greedy_pick_kernel, dim3(B), dim3(1024), 0, (hipStream_t)stream, logits, V, ld, embedding, D, hidden,
                      reinterpret_cast<long long*>(token), reinterpret_cast<long long*>(out), out_ld,
-                     reinterpret_cast<const long long*>(step));
+                     reinterpret_cast<const long long*>(step), reinterpret_cast<long long*>(advance), ticket);
   return check_launch("ajq_greedy_pick");
 }
 

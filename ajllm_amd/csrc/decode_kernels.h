@@ -141,6 +141,9 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
 struct KvRow8 {
   float4 a, b;
 };
+// One partial result of a row chunk: (maximum, denominator, 0, 0, 128 weighted value sums); the
+// sums start on a 16-byte boundary so that a GEMV prologue can fetch them with 128-bit loads.
+constexpr int kAttnPartialStride = 132;
 __device__ __forceinline__ KvRow8 load_row8(const float* p) {
   const float4* p4 = reinterpret_cast<const float4*>(p);
   return KvRow8{p4[0], p4[1]};
@@ -316,13 +319,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
       A.x += sacc[r][w][2 * lane] * cw;
       A.y += sacc[r][w][2 * lane + 1] * cw;
     }
-    if (S == 1) {
+    if (S == 1 && out != nullptr) {
       const uint32_t o = pack2_bf16(A.x / L, A.y / L);
       reinterpret_cast<uint32_t*>(out + (size_t)(bh0 + r) * hd)[lane] = o;
-    } else {
-      float* dst = partial + ((size_t)(bh0 + r) * S + s) * (hd + 2);
-      if (lane == 0) { dst[0] = M16; dst[1] = L; }
-      *reinterpret_cast<float2*>(dst + 2 + 2 * lane) = A;
+    } else {  // several chunks, or a caller that merges them itself (out == nullptr)
+      float* dst = partial + ((size_t)(bh0 + r) * S + s) * kAttnPartialStride;
+      if (lane == 0) *reinterpret_cast<float4*>(dst) = float4{M16, L, 0.f, 0.f};
+      *reinterpret_cast<float2*>(dst + 4 + 2 * lane) = A;
     }
   }
 }
@@ -334,12 +337,13 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
                                                         uint16_t* __restrict__ out) {
   constexpr int hd = 128;
   const int bh = blockIdx.x, lane = threadIdx.x;
-  const float* src = partial + (size_t)bh * S * (hd + 2);
+  const float* src = partial + (size_t)bh * S * kAttnPartialStride;
   const int sl = min(lane & 15, S - 1);
-  const float2 ml = *reinterpret_cast<const float2*>(src + sl * (hd + 2));  // (max, denominator) of chunk lane % 16
+  const float2 ml = *reinterpret_cast<const float2*>(src + sl * kAttnPartialStride);  // (max, denominator) of chunk lane % 16
   float2 a[16];
 #pragma unroll
-  for (int s = 0; s < 16; ++s) a[s] = *reinterpret_cast<const float2*>(src + min(s, S - 1) * (hd + 2) + 2 + 2 * lane);
+  for (int s = 0; s < 16; ++s)
+    a[s] = *reinterpret_cast<const float2*>(src + min(s, S - 1) * kAttnPartialStride + 4 + 2 * lane);
   float M = ml.x;
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
@@ -362,12 +366,14 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
 // Greedy choice at the end of a decode step, one workgroup of 1024 threads per sequence:
 // token = argmax(logits[b, 0..V)) (the lowest index among equal maxima, as torch.argmax),
 // written to token[b] and to out[b, *step]; then hidden[b, :] = embedding[token, :], the next
-// step's input.  `step` is only read.
+// step's input.  With `advance` (two int64 counters, `step` may be one of them) the last workgroup
+// to finish adds one to both; `ticket` is a zeroed word the kernel leaves zeroed.
 __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restrict__ logits, int V, int ld,
                                                            const float* __restrict__ embedding, int D,
                                                            float* __restrict__ hidden, long long* __restrict__ token,
                                                            long long* __restrict__ out, int out_ld,
-                                                           const long long* __restrict__ step) {
+                                                           const long long* __restrict__ step,
+                                                           long long* advance, unsigned* ticket) {
   const int b = blockIdx.x, t = threadIdx.x;
   const float* row = logits + (size_t)b * ld;
   float best = -INFINITY;
@@ -417,6 +423,16 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
     chosen = bi;
     token[b] = bi;
     out[(size_t)b * out_ld + min(max(*step, 0LL), (long long)out_ld - 1)] = bi;  // device data: held inside the row
+    if (advance) {
+      // the step's two counters (cache row, output column) advance here, once every workgroup has
+      // read them: this thread's read of *step above has returned (its value addressed the store)
+      // before its ticket is drawn, so the workgroup that draws the last ticket writes after all reads
+      if (atomicAdd(ticket, 1u) == gridDim.x - 1) {
+        advance[0] += 1;
+        advance[1] += 1;
+        *ticket = 0u;
+      }
+    }
   }
   __syncthreads();
   const float4* e4 = reinterpret_cast<const float4*>(embedding + (size_t)chosen * D);

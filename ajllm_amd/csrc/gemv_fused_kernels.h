@@ -2,21 +2,33 @@
 // K == kWaves * TPW * 128):
 //   kPro == kProNorm:  x = bf16( RMSNorm(h + delta) * gain ),  h + delta also written out
 //                      (the residual update and the norm in front of q|k|v and w1|w3);
-//   kPro == kProGate:  x = bf16( silu(a) * u ) for ab = (a | u)  (the SwiGLU gate in front of w2).
+//   kPro == kProGate:  x = bf16( silu(a) * u ) for ab = (a | u)  (the SwiGLU gate in front of w2);
+//   kPro == kProMerge: x = the single-query attention output, merged from the partial results
+//                      of its S row chunks (what attn_merge_kernel computes, in front of the
+//                      output projection: K = heads * 128, one k group per head).
 // The matmul is dequant_gemv_kernel's straight-line variant: one workgroup per 16-row tile of
 // N, wave w owns k groups [w * TPW, (w + 1) * TPW), weight loads first.  What changes is where
 // a wave's k-slice of the activations comes from: it loads the fp32 sources of its slice (every
 // workgroup repeats that work; the sources are a few KB and sit in L2), forms the bf16 values
-// in registers and stages them in its private LDS rows as before.  The norm needs the whole
+// in registers and stages them in its private LDS rows as before.  The source loads are issued
+// in front of the weight loads: vector loads return in issue order, the sources come from L2 and
+// the weights from HBM, so this way the prologue arithmetic runs while the weights travel
+// (issued behind them, the sources could not be touched before the last weight tile arrived).  The norm needs the whole
 // row's sum of squares: every wave reduces its slice per row, the eight partial sums meet in
 // LDS behind one barrier (the weight loads are in flight meanwhile).  Workgroup 0 writes the
 // updated residual stream, to a buffer other than the one being read.
 #pragma once
 #include "gemv_kernels.h"
+#include "decode_kernels.h"
 
 namespace ajq {
 
-constexpr int kProNorm = 1, kProGate = 2;
+constexpr int kProNorm = 1, kProGate = 2, kProMerge = 3;
+
+// chunks of one (row, head) a lane of the merge prologue takes (the 4 lane quarters take every 4th chunk)
+constexpr int merge_chunks_per_lane(int mrows, int tpw) {
+  return 8 / (mrows * tpw) > 4 ? 4 : (8 / (mrows * tpw) < 1 ? 1 : 8 / (mrows * tpw));
+}
 
 template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
@@ -26,11 +38,12 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     int m_flags,  // M | out_f32 << 8
     int N, void* __restrict__ y,
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
-    const float* __restrict__ src0,        // norm: h_in [M, K];  gate: ab [M, 2K]
+    const float* __restrict__ src0,        // norm: h_in [M, K];  gate: ab [M, 2K];  merge: partial [M * K / 128][S][132]
     const float* __restrict__ src1,        // norm: delta [M, K] or nullptr
     const float* __restrict__ gain,        // norm: [K]
     float eps,                             // norm
-    float* __restrict__ h_out) {           // norm: h_in + delta [M, K]; must not alias h_in
+    float* __restrict__ h_out,             // norm: h_in + delta [M, K]; must not alias h_in
+    int S) {                               // merge: row chunks per (row, head), 1 <= S <= 4 * merge_chunks_per_lane
   const int M = m_flags & 0xFF;
   const bool out_f32 = (m_flags >> 8) != 0;
   constexpr int kSlice = TPW * kGroup;
@@ -53,18 +66,28 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   float* ssq = red + kWaves * 64 * 4;  // [MROWS][kWaves] partial sums of squares
   const int g0 = wave * TPW;
 
-  // ---- loads: weights first, then the fp32 sources of this wave's activation slice, then meta
+  // ---- loads: the fp32 sources of this wave's activation slice, then weights and meta
   u32x4_t w[TPW][kLoadsPerGroup];
   uint32_t mw[TPW];
   float4 a0[kXLoads][2], a1[kXLoads][2], a2[kXLoads][2];
+  constexpr int kCpl = merge_chunks_per_lane(MROWS, TPW);
+  constexpr int kPairs = kPro == kProMerge ? MROWS * TPW : 1;  // (row, head) pairs of this wave
+  float4 pm[kPairs][kCpl], pa[kPairs][kCpl][2];                // merge: (max, denominator, -, -) and 8 sums per chunk
   __builtin_amdgcn_sched_barrier(0);
-  {
-    const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
+  if (kPro == kProMerge) {
+    const int sgrp = lane >> 4, c = lane & 15;
 #pragma unroll
-    for (int p = 0; p < TPW; ++p)
+    for (int q = 0; q < kPairs; ++q) {
+      const int m = min(q / TPW, M - 1), head = g0 + q % TPW;
+      const float* base = src0 + (size_t)(m * G + head) * S * kAttnPartialStride;
 #pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h)
-        w[p][h] = __builtin_nontemporal_load(wtile + (p * kLoadsPerGroup + h) * 64);
+      for (int j = 0; j < kCpl; ++j) {
+        const float* rec = base + (size_t)min(sgrp + 4 * j, S - 1) * kAttnPartialStride;
+        pm[q][j] = *reinterpret_cast<const float4*>(rec);
+        pa[q][j][0] = *reinterpret_cast<const float4*>(rec + 4 + 8 * c);
+        pa[q][j][1] = *reinterpret_cast<const float4*>(rec + 8 + 8 * c);
+      }
+    }
   }
 #pragma unroll
   for (int i = 0; i < kXLoads; ++i) {
@@ -85,14 +108,22 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       const float4* pg = reinterpret_cast<const float4*>(gain + k);
       a2[i][0] = pg[0];
       a2[i][1] = pg[1];
-    } else {
-      const float4* pa = reinterpret_cast<const float4*>(src0 + (size_t)m * 2 * K + k);
+    } else if (kPro == kProGate) {
+      const float4* pa_ = reinterpret_cast<const float4*>(src0 + (size_t)m * 2 * K + k);
       const float4* pu = reinterpret_cast<const float4*>(src0 + (size_t)m * 2 * K + K + k);
-      a0[i][0] = pa[0];
-      a0[i][1] = pa[1];
+      a0[i][0] = pa_[0];
+      a0[i][1] = pa_[1];
       a1[i][0] = pu[0];
       a1[i][1] = pu[1];
     }
+  }
+  {
+    const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
+#pragma unroll
+    for (int p = 0; p < TPW; ++p)
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        w[p][h] = __builtin_nontemporal_load(wtile + (p * kLoadsPerGroup + h) * 64);
   }
   if (kW4) {
     const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
@@ -100,16 +131,6 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
   }
   __builtin_amdgcn_sched_barrier(0);
-
-  float sc[TPW], zc[TPW];
-  if (kW4) {
-#pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      sc[p] = f16_bits_to_f32(mw[p] & 0xFFFFu);
-      zc[p] = f16_bits_to_f32(mw[p] >> 16);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
 
   // ---- the activations of this slice, 8 per lane and load
   float xv[kXLoads][8];
@@ -148,7 +169,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       xv[i][4] = (xv[i][4] / rms) * g1v.x; xv[i][5] = (xv[i][5] / rms) * g1v.y;
       xv[i][6] = (xv[i][6] / rms) * g1v.z; xv[i][7] = (xv[i][7] / rms) * g1v.w;
     }
-  } else {
+  } else if (kPro == kProGate) {
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const float av[8] = {a0[i][0].x, a0[i][0].y, a0[i][0].z, a0[i][0].w, a0[i][1].x, a0[i][1].y, a0[i][1].z, a0[i][1].w};
@@ -157,9 +178,49 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       for (int e = 0; e < 8; ++e) xv[i][e] = av[e] * (1.0f / (1.0f + expf(-av[e]))) * uv[e];
     }
   }
+  if (kPro == kProMerge) {
+    // every (row, head) pair of the wave: lane quarter `sgrp` holds chunks sgrp, sgrp + 4, ... of the
+    // 8 dimensions 8c .. 8c + 7; maxima, denominators and sums meet across the quarters, quarter 0
+    // normalises and stages the 8 activations
+    const int sgrp = lane >> 4, c = lane & 15;
+#pragma unroll
+    for (int q = 0; q < kPairs; ++q) {
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < kCpl; ++j)
+        if (sgrp + 4 * j < S) mloc = fmaxf(mloc, pm[q][j].x);
+      float mall = fmaxf(mloc, __shfl_xor(mloc, 16));
+      mall = fmaxf(mall, __shfl_xor(mall, 32));
+      float L = 0.f, A[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < kCpl; ++j) {
+        if (sgrp + 4 * j < S) {
+          const float cw = pm[q][j].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(pm[q][j].x - mall);
+          L += pm[q][j].y * cw;
+          A[0] += pa[q][j][0].x * cw; A[1] += pa[q][j][0].y * cw; A[2] += pa[q][j][0].z * cw; A[3] += pa[q][j][0].w * cw;
+          A[4] += pa[q][j][1].x * cw; A[5] += pa[q][j][1].y * cw; A[6] += pa[q][j][1].z * cw; A[7] += pa[q][j][1].w * cw;
+        }
+      }
+      L += __shfl_xor(L, 16);
+      L += __shfl_xor(L, 32);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        A[e] += __shfl_xor(A[e], 16);
+        A[e] += __shfl_xor(A[e], 32);
+      }
+      if (sgrp == 0) {
+        u32x4_t pk;
+        pk.x = pack2_bf16(A[0] / L, A[1] / L);
+        pk.y = pack2_bf16(A[2] / L, A[3] / L);
+        pk.z = pack2_bf16(A[4] / L, A[5] / L);
+        pk.w = pack2_bf16(A[6] / L, A[7] / L);
+        *reinterpret_cast<u32x4_t*>(xs + (q / TPW) * kStride + (q % TPW) * kGroup + 8 * c) = pk;
+      }
+    }
+  }
   // bf16, into the wave's own LDS rows
 #pragma unroll
-  for (int i = 0; i < kXLoads; ++i) {
+  for (int i = 0; i < (kPro == kProMerge ? 0 : kXLoads); ++i) {
     const int v = lane + 64 * i;
     u32x4_t pk;
     pk.x = pack2_bf16(xv[i][0], xv[i][1]);
@@ -171,6 +232,14 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   }
 
   // ---- the matmul, as in dequant_gemv_kernel
+  float sc[TPW], zc[TPW];
+  if (kW4) {
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      sc[p] = f16_bits_to_f32(mw[p] & 0xFFFFu);
+      zc[p] = f16_bits_to_f32(mw[p] >> 16);
+    }
+  }
   const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;

@@ -10,6 +10,8 @@ the chosen token fed back on the device: no host round trip between steps.
 
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib, modeling
@@ -168,6 +170,21 @@ class _FusedLinear:
                       self.rows16, y.data_ptr(), _lib.AJQ_OUT_F32, _stream()), "gemv_norm")
         return y
 
+    def merge_splits(self, batch: int) -> int:
+        """Largest number of attention row chunks the GEMV that merges them on its way in takes
+        for ``batch`` rows of this layer's input width (0: not built)."""
+        return int(_lib.load().ajq_gemv_merge_max_splits(batch, self.in_features))
+
+    def after_merge(self, partial: torch.Tensor, splits: int, rows: int) -> torch.Tensor:
+        """``self(attention output)`` with the output merged from ``splits`` partial results per
+        (row, head) on the way in (``ajq_attn_step_partial`` left them in ``partial``), one launch."""
+        lib = _lib.load()
+        y = torch.empty((rows, self.rows16), dtype=torch.float32, device=partial.device)
+        fn = lib.ajq_w8a16_gemv_merge if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_merge
+        _lib.check(fn(partial.data_ptr(), splits, rows, self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, y.data_ptr(), _lib.AJQ_OUT_F32, _stream()), "gemv_merge")
+        return y
+
     def after_gate(self, ab: torch.Tensor) -> torch.Tensor:
         """``self(bf16(silu(a) * u))`` for ``ab = (a | u)``, one launch."""
         lib = _lib.load()
@@ -181,8 +198,10 @@ class _FusedLinear:
 class FusedDecoder(GraphDecoder):
     """GraphDecoder whose step runs on this library's kernels only: fused q|k|v and w1|w3
     matmuls, residual add + RMSNorm, RoPE + cache write + single-query attention in one launch
-    and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), plus the
-    embedding lookup and the argmax from PyTorch.  Nine launches per layer (eight where the attention needs no merge).
+    and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), the greedy pick
+    with the embedding lookup and the step counters (``ajq_greedy_pick``).  Five launches per layer
+    at batch 1 (q|k|v with the norm, attention, output projection with the merge of the attention's
+    row chunks, w1|w3 with the norm, w2 with the gate: ``launches_per_step``), up to nine at large batch.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
@@ -233,8 +252,10 @@ class FusedDecoder(GraphDecoder):
         self.embedded = torch.zeros((batch, d), dtype=torch.float32, device=dev)  # embedding row of self.token
         self.hidden = torch.zeros((batch, d), dtype=torch.float32, device=dev)
         self.hidden2 = torch.zeros((batch, d), dtype=torch.float32, device=dev)
-        # write position and output column advance together: one tensor, one increment per step
+        # write position and output column advance together: one tensor, incremented by the greedy
+        # pick at the end of a step (its last workgroup to finish; ``ticket`` is its scratch word)
         self.counters = torch.zeros(2, dtype=torch.long, device=dev)
+        self.ticket = torch.zeros(1, dtype=torch.int32, device=dev)
         self.cache.position = self.counters[0:1]
         self.step_index = self.counters[1:2]
         self.logits_full: torch.Tensor | None = None
@@ -246,6 +267,10 @@ class FusedDecoder(GraphDecoder):
         self.fuse_norm = batch <= 4 and self.head.fusable(batch)
         self.fuse_gate = (batch == 1 and self.layers[0]["w2"].fusable(batch)
                           and self.layers[0]["w13"].rows16 == 2 * self.d_ff)
+        # the output projection merges the attention's row chunks on its way in where that is built
+        # (small batches; one launch less per layer)
+        self.merge_splits = self.layers[0]["o"].merge_splits(batch) if self.layers[0]["o"].in_features == d else 0
+        self.fuse_merge = self.merge_splits > 0
         self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)
@@ -325,14 +350,27 @@ class FusedDecoder(GraphDecoder):
     @torch.no_grad()
     def _step(self) -> None:
         """One token: the layer stack, then the greedy choice, its embedding row (the next step's
-        input) and the two counters, in two launches."""
+        input) and the two counters in one launch."""
         self._logits()
         full = self.logits_full
         _lib.check(_lib.load().ajq_greedy_pick(full.data_ptr(), self.batch, self.vocab, full.shape[1],
                                                self.embedding.data_ptr(), self.model.d_model, self.embedded.data_ptr(),
                                                self.token.data_ptr(), self.out.data_ptr(), self.out.shape[1],
-                                               self.step_index.data_ptr(), _stream()), "greedy_pick")
-        self.counters.add_(1)
+                                               self.step_index.data_ptr(), self.counters.data_ptr(),
+                                               self.ticket.data_ptr(), _stream()), "greedy_pick")
+
+    def launches_per_step(self) -> int:
+        """Kernel launches of one decode step as this decoder is configured."""
+        lib = _lib.load()
+        per_layer = 2 if self.fuse_norm else 4           # q|k|v and w1|w3, each with or without its norm launch
+        per_layer += 1                                   # attention
+        if not self.fuse_merge:                          # merge of its row chunks (none if there is one chunk)
+            per_layer += 1
+        per_layer += 1                                   # output projection
+        per_layer += 1 if self.fuse_gate else 2          # w2 with or without the gate launch
+        head = 1 if self.fuse_norm else 2
+        first_copy = 0 if self.fuse_norm else 1          # embedding row copied into the residual stream
+        return per_layer * len(self.layers) + head + first_copy + 1  # + greedy pick (token, embedding row, counters)
 
     def _logits(self) -> torch.Tensor:
         """Logits ``[B, V]`` of the token whose embedding row is in ``self.embedded`` (``prefill`` and
@@ -361,12 +399,22 @@ class FusedDecoder(GraphDecoder):
 
         for index, w in enumerate(self.layers):
             qkv = normed_linear(w["qkv"], w["g1"], w["eps1"])
-            _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
-                                         self.cache.keys[index].data_ptr(), self.cache.values[index].data_ptr(),
-                                         self.kv_flag, b, self.heads, self.kv_heads, 128, self.max_len,
-                                         self.attended.data_ptr(), self.attn_ws.data_ptr(), self.attn_ws_bytes, st),
-                       "attn_step")
-            delta = w["o"](self.attended)
+            if self.fuse_merge:
+                splits = ctypes.c_int(0)
+                _lib.check(lib.ajq_attn_step_partial(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
+                                                     pos.data_ptr(), self.cache.keys[index].data_ptr(),
+                                                     self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
+                                                     self.kv_heads, 128, self.max_len, self.merge_splits,
+                                                     ctypes.addressof(splits), self.attn_ws.data_ptr(),
+                                                     self.attn_ws_bytes, st), "attn_step_partial")
+                delta = w["o"].after_merge(self.attn_ws, splits.value, b)
+            else:
+                _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
+                                             self.cache.keys[index].data_ptr(), self.cache.values[index].data_ptr(),
+                                             self.kv_flag, b, self.heads, self.kv_heads, 128, self.max_len,
+                                             self.attended.data_ptr(), self.attn_ws.data_ptr(), self.attn_ws_bytes, st),
+                           "attn_step")
+                delta = w["o"](self.attended)
             ab = normed_linear(w["w13"], w["g2"], w["eps2"])
             if self.fuse_gate:
                 delta = w["w2"].after_gate(ab)

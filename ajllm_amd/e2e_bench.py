@@ -60,6 +60,51 @@ def _linear_seconds_per_step(dec: "decoding.FusedDecoder", batch: int, device) -
     return start.elapsed_time(stop) / 1e3 / 20
 
 
+@torch.no_grad()
+def bench_decode_short(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") -> list[dict]:
+    """The graph-replayed greedy decode of :func:`bench_decode` alone (prompt 512, 256 new tokens, batch 1
+    and 8), without the eager-loop comparison: a few seconds, for the default benchmark line."""
+    t0 = time.perf_counter()
+    model = build_quantized_model(device, scheme)
+    torch.cuda.synchronize()
+    build_s = time.perf_counter() - t0
+    packed = sum(m.wq.numel() * 4 + m.meta.numel() * m.meta.element_size()
+                 for m in model.modules() if isinstance(m, QuantLinear))
+    results = []
+    for batch in batches:
+        g = torch.Generator().manual_seed(100 + batch)
+        prompt = torch.randint(0, CONFIG["vocab_size"], (batch, PROMPT_LEN), generator=g).to(device)
+        dec = decoding.FusedDecoder(model, batch, PROMPT_LEN + NEW_TOKENS)
+        dec.prefill(prompt, fused=True)
+        dec.generate(8)  # eager step + capture + first replays
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        tokens = dec.generate(NEW_TOKENS)
+        torch.cuda.synchronize()
+        t_graph = time.perf_counter() - t0
+        steps = NEW_TOKENS - 8
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.prefill(prompt, fused=True)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        t_linear = _linear_seconds_per_step(dec, batch, device)
+        step = t_graph / steps
+        r = {"scheme": scheme, "batch": batch, "prompt": PROMPT_LEN, "new_tokens": NEW_TOKENS,
+             "decode_tok/s": batch * steps / t_graph, "ms_per_step": step * 1e3,
+             "prefill_library_kernels_s": t_prefill, "prefill_library_kernels_tok/s": batch * PROMPT_LEN / t_prefill,
+             "quant_linear_ms_per_step": t_linear * 1e3, "quant_linear_share_of_step": t_linear / step,
+             "quant_linear_GB/s": packed / t_linear / 1e9, "packed_weight_bytes": packed,
+             "launches_per_step": dec.launches_per_step(), "model_build_s": build_s,
+             "tokens_in_vocab": bool(int(tokens.min()) >= 0 and int(tokens.max()) < CONFIG["vocab_size"])}
+        log("decode", r)
+        results.append(r)
+        del dec
+    del model
+    torch.cuda.empty_cache()
+    return results
+
+
 def cache2_for(model, prompt):
     """A dynamic KV cache holding the prompt (for a one-step logits comparison)."""
     cache = model.new_cache(prompt.shape[0], prompt.shape[1] + 8)

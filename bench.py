@@ -13,9 +13,12 @@ Default run (what the driver calls: ``python bench.py --gpus 1 --steps K --warmu
   TFLOP/s against the bf16 dense MFMA peak, and the CPU baseline: the oracle's quantized
   linear timed on this box's host cores for the same GEMV shape.
 
+* also after it: the end-to-end greedy decode of the 12-layer W4A16 model (prompt 512 + 256 tokens,
+  batch 1 and 8) in tokens/s, short form.
+
 ``--sweep`` adds the rest of the decode sweep (three shapes x M in {1, 4, 16}, W4 and W8)
-and all prefill shapes; ``--decode`` adds the end-to-end decode tokens/s of the 12-layer
-model.  One JSON line is printed on stdout; everything else goes to stderr.
+and all prefill shapes; ``--decode`` replaces the short decode leg by the long one (eager PyTorch loop
+beside it, token comparison between the two loops).  One JSON line is printed on stdout; everything else goes to stderr.
 """
 
 from __future__ import annotations
@@ -306,6 +309,12 @@ def main() -> int:
                     "expanded to bf16, and the MFMA rate sustained with no memory traffic (random operands "
                     "reach the power limit and the shader clock drops)",
         }
+    if not args.no_extras and not args.decode:
+        # config 4 end to end, short form: the 12-layer W4A16 model, prompt 512 + 256 greedy tokens,
+        # batch 1 and 8, decode step replayed from a HIP graph (tokens/s is the third headline metric)
+        from ajllm_amd.e2e_bench import bench_decode_short
+
+        extras["decode"] = bench_decode_short(device, log)
     if args.sweep:
         sweep = []
         for scheme in ("w4", "w8"):

@@ -139,6 +139,16 @@ int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
                         void* y, int out_dtype, void* stream);
 int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                         void* y, int out_dtype, void* stream);
+/*   _merge: x = bf16 of the single-query attention output [M, K] (K = heads * 128), merged from the S
+ *          partial results per (row, head) that ajq_attn_step_partial left in its workspace -- the
+ *          softmax-weighted value sum of scaled_dot_product_attention (src/ajllm/modeling/attention.py:20-33)
+ *          in front of output_proj (attention.py:120).  ajq_gemv_merge_max_splits(M, K) is the largest S
+ *          built for the shape (0: not built; K = 2048 with M <= 4, K = 4096 with M <= 2). */
+int ajq_gemv_merge_max_splits(int M, int K);
+int ajq_w4a16_gemv_merge(const float* partial, int S, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                         void* y, int out_dtype, void* stream);
+int ajq_w8a16_gemv_merge(const float* partial, int S, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                         void* y, int out_dtype, void* stream);
 
 /* any M >= 1; bf16 MFMA.  M <= 16 runs the GEMV above, 17 <= M < 128 (several sequences decoded
  * together) a weight-streaming kernel with 32-row activation blocks, and from M = 128 on the
@@ -207,6 +217,16 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
                   void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
                   int max_len, uint16_t* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ajq_attn_step without the merge of its row chunks: the S partial results per (sequence, query
+ * head) stay in the workspace as records of 132 floats (maximum as a base-2 exponent, denominator,
+ * two pad words, 128 weighted value sums) for ajq_w*a16_gemv_merge, the output projection that
+ * merges them on its way in (one launch less per layer).  At most max_splits chunks are used (what
+ * ajq_gemv_merge_max_splits allows for the batch); *splits (host memory) receives S. */
+int ajq_attn_step_partial(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
+                          void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
+                          int max_len, int max_splits, int* splits, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
 /* ab[B, 2F] = (w1 x | w3 x) -> out[B, F] = bf16(silu(w1 x) * w3 x)
  * (SwiGLU.forward, src/ajllm/modeling/activations.py:24-25, between its linears). */
 int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
@@ -227,7 +247,8 @@ int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int
  * stride out_ld), and hidden[b, :] = embedding[token[b], :] (Embedding.forward,
  * src/ajllm/modeling/layers.py:52-53), the next step's input.  token, out, step: int64. */
 int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embedding, int D, float* hidden,
-                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, void* stream);
+                    int64_t* token, int64_t* out, int out_ld, const int64_t* step, int64_t* advance, uint32_t* ticket,
+                    void* stream);
 
 #ifdef __cplusplus
 }

@@ -375,10 +375,89 @@ def test_greedy_pick(cuda):
         out = torch.full((b, 9), -1, dtype=torch.long, device=cuda)
         step = torch.tensor([4], device=cuda)
         _lib.check(lib.ajq_greedy_pick(logits.data_ptr(), b, v, ld, emb.data_ptr(), d, hidden.data_ptr(), token.data_ptr(),
-                                       out.data_ptr(), 9, step.data_ptr(), st), "greedy_pick")
+                                       out.data_ptr(), 9, step.data_ptr(), None, None, st), "greedy_pick")
         want = torch.argmax(logits[:, :v], dim=-1)
         assert want[0] == 7 and torch.equal(token.view(-1), want) and torch.equal(out[:, 4], want)
         assert (out[:, :4] == -1).all() and (out[:, 5:] == -1).all() and torch.equal(hidden, emb[want])
+        assert int(step) == 4
+        # with the step's counters advanced by the kernel itself: every workgroup still writes column 4,
+        # both counters end one higher, the ticket word is left at zero; twice in a row
+        counters = torch.tensor([100, 4], dtype=torch.long, device=cuda)
+        ticket = torch.zeros(1, dtype=torch.int32, device=cuda)
+        for rep in range(2):
+            out.fill_(-1)
+            _lib.check(lib.ajq_greedy_pick(logits.data_ptr(), b, v, ld, emb.data_ptr(), d, hidden.data_ptr(),
+                                           token.data_ptr(), out.data_ptr(), 9, counters[1:].data_ptr(),
+                                           counters.data_ptr(), ticket.data_ptr(), st), "greedy_pick")
+            assert torch.equal(out[:, 4 + rep], want) and int((out != -1).sum()) == b
+            assert counters.tolist() == [101 + rep, 5 + rep] and int(ticket) == 0
+        with pytest.raises(ValueError):
+            _lib.check(lib.ajq_greedy_pick(logits.data_ptr(), b, v, ld, emb.data_ptr(), d, hidden.data_ptr(),
+                                           token.data_ptr(), out.data_ptr(), 9, step.data_ptr(), counters.data_ptr(), None,
+                                           st), "greedy_pick")
+
+
+@pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
+@pytest.mark.parametrize("b,h,hkv,pos,max_len", [(1, 16, 16, 700, 768), (2, 16, 4, 300, 2048), (4, 16, 8, 90, 128),
+                                                 (1, 32, 8, 2000, 2100), (2, 32, 32, 40, 64), (1, 16, 16, 0, 768)])
+def test_output_projection_that_merges_the_attention_chunks(cuda, scheme, b, h, hkv, pos, max_len):
+    """ajq_attn_step_partial + ajq_w*a16_gemv_merge against ajq_attn_step (which merges the chunks in a
+    launch of its own and rounds to bf16) followed by the plain GEMV: the same activations up to a
+    differently ordered sum, so the outputs agree to a bf16 rounding of a few activations; also
+    against the masked-softmax statement of the model code times the oracle's dequantized weight."""
+    import ctypes
+
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(1000 * b + h + pos)
+    d = h * 128
+    cap = lib.ajq_gemv_merge_max_splits(b, d)
+    assert cap >= 4
+    layer = QuantLinear.from_weight((torch.randn((272, d), generator=g) * 0.02).to(cuda), scheme)
+    fused = decoding._FusedLinear([layer])
+    qkv = torch.randn((b, (h + 2 * hkv) * 128), generator=g).to(cuda)
+    keys = torch.randn((b, hkv, max_len, 128), generator=g).to(cuda)
+    values = torch.randn((b, hkv, max_len, 128), generator=g).to(cuda)
+    half = torch.arange(64, dtype=torch.float32)
+    angles = torch.arange(max_len, dtype=torch.float32)[:, None] / (10000.0 ** (2 * half / 128))[None, :]
+    cos, sin = torch.cos(angles).to(cuda).contiguous(), torch.sin(angles).to(cuda).contiguous()
+    position = torch.tensor([pos], device=cuda)
+    ws_bytes = lib.ajq_attn_step_workspace_bytes(b, h)
+    ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
+    k1, v1, k2, v2 = keys.clone(), values.clone(), keys.clone(), values.clone()
+    attended = torch.empty((b, d), dtype=torch.bfloat16, device=cuda)
+    _lib.check(lib.ajq_attn_step(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), position.data_ptr(), k1.data_ptr(),
+                                 v1.data_ptr(), _lib.AJQ_KV_F32, b, h, hkv, 128, max_len, attended.data_ptr(),
+                                 ws.data_ptr(), ws_bytes, st), "attn_step")
+    want = fused(attended)
+    ws2 = torch.zeros_like(ws).view(torch.float32)
+    splits = ctypes.c_int(0)
+    _lib.check(lib.ajq_attn_step_partial(qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), position.data_ptr(),
+                                         k2.data_ptr(), v2.data_ptr(), _lib.AJQ_KV_F32, b, h, hkv, 128, max_len, cap,
+                                         ctypes.addressof(splits), ws2.data_ptr(), ws_bytes, st), "attn_step_partial")
+    assert 1 <= splits.value <= cap
+    got = fused.after_merge(ws2, splits.value, b)
+    torch.cuda.synchronize()
+    assert torch.equal(k1, k2) and torch.equal(v1, v2)           # the step's cache row, written by both
+    max_abs, rel = errors(got, want)
+    assert rel <= 2e-3 and max_abs <= 2e-2, (max_abs, rel)
+    # against the statement: softmax(q k^T / sqrt(128)) v per head with the step's row included, in fp64
+    qk = qkv.double().cpu()
+    rot = lambda x, p: torch.stack((x[..., 0::2] * torch.cos(angles[p]).double() - x[..., 1::2] * torch.sin(angles[p]).double(),
+                                    x[..., 0::2] * torch.sin(angles[p]).double() + x[..., 1::2] * torch.cos(angles[p]).double()),
+                                   dim=-1).flatten(-2)
+    q = rot(qk[:, : h * 128].view(b, h, 128), pos)
+    kk, vv = k2[:, :, : pos + 1].double().cpu(), v2[:, :, : pos + 1].double().cpu()
+    rep = h // hkv
+    scores = torch.einsum("bhd,bhtd->bht", q, kk.repeat_interleave(rep, dim=1)) / 128 ** 0.5
+    att = torch.einsum("bht,bhtd->bhd", torch.softmax(scores, -1), vv.repeat_interleave(rep, dim=1)).reshape(b, d)
+    w_hat = (qspec.dequantize_w8(layer.qweight.cpu().numpy(), layer.scales.cpu().numpy()) if scheme == "w8a16" else
+             qspec.dequantize_w4(layer.qweight.cpu().numpy(), layer.scales.cpu().numpy(), layer.zeros.cpu().numpy()))
+    ref = qspec.quant_linear(att.to(torch.bfloat16), torch.from_numpy(w_hat), accumulate=torch.float64,
+                             out_dtype=torch.float64)
+    max_abs, rel = errors(got[:, :272], ref)
+    assert rel <= 2e-3 and max_abs <= MAX_ABS_TOL, (max_abs, rel)
 
 
 @pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
