@@ -31,7 +31,6 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_w4a16_gemm_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_size_t,
                                     c_void_p]),
     "ajq_w8a16_gemm_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
-    "ajq_probe_mfma_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w8": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ajq_quantize_w4_g128": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ajq_repack_w4": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
@@ -104,7 +103,39 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
 }
 
+# libajq_bench.so (include/ajq_bench.h): measurement probes for bench.py, not operators
+BENCH_LIBRARY_PATH = Path(__file__).resolve().parent / "libajq_bench.so"
+
+
+class BenchResult(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 112), ("us_per_stage", ctypes.c_double), ("frac_hbm_peak", ctypes.c_double),
+                ("matches_reference", c_int), ("error_word", c_int)]
+
+
+BENCH_SIGNATURES: dict[str, tuple] = {
+    "ajqb_last_error": (c_char_p, []),
+    "ajqb_mfma_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ajqb_launch_alternatives": (c_int, [c_int, c_int, ctypes.POINTER(BenchResult), c_int, ctypes.POINTER(c_int)]),
+}
+
 _lib: ctypes.CDLL | None = None
+_bench_lib: ctypes.CDLL | None = None
+
+
+def load_bench() -> ctypes.CDLL:
+    """The bench-only probe library, bound on first use (built by ``python -m ajllm_amd.build``)."""
+    global _bench_lib
+    if _bench_lib is not None:
+        return _bench_lib
+    if not BENCH_LIBRARY_PATH.exists():
+        raise RuntimeError(f"{BENCH_LIBRARY_PATH} is missing: build it with `python -m ajllm_amd.build`")
+    lib = ctypes.CDLL(str(BENCH_LIBRARY_PATH))
+    for name, (restype, argtypes) in BENCH_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _bench_lib = lib
+    return lib
 
 
 def load() -> ctypes.CDLL:

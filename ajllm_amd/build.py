@@ -15,6 +15,9 @@ from pathlib import Path
 PACKAGE_DIR = Path(__file__).resolve().parent
 SOURCE = PACKAGE_DIR / "csrc" / "ajq.hip"
 LIBRARY = PACKAGE_DIR / "libajq.so"
+# measurement probes for bench.py (include/ajq_bench.h); the operator library does not depend on it
+BENCH_SOURCE = PACKAGE_DIR / "csrc" / "ajq_bench.hip"
+BENCH_LIBRARY = PACKAGE_DIR / "libajq_bench.so"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -30,10 +33,10 @@ HIPCC_FLAGS = [
 ]
 
 
-def build_library(verbose: bool = False) -> Path:
+def build_library(verbose: bool = False, source: Path = SOURCE, library: Path = LIBRARY) -> Path:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    tmp = LIBRARY.with_suffix(".so.tmp%d" % os.getpid())
-    cmd = [hipcc, *HIPCC_FLAGS, str(SOURCE), "-o", str(tmp)]
+    tmp = library.with_suffix(".so.tmp%d" % os.getpid())
+    cmd = [hipcc, *HIPCC_FLAGS, str(source), "-o", str(tmp)]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -44,9 +47,14 @@ def build_library(verbose: bool = False) -> Path:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{stderr}")
     if stderr.strip() and verbose:
         print(stderr, file=sys.stderr)
-    os.replace(tmp, LIBRARY)
-    return LIBRARY
+    os.replace(tmp, library)
+    return library
+
+
+def build_bench_library(verbose: bool = False) -> Path:
+    return build_library(verbose, BENCH_SOURCE, BENCH_LIBRARY)
 
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_bench_library(verbose=True))

@@ -13,7 +13,6 @@
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
 #include "prefill_attention.h"
-#include "probe_kernels.h"
 
 using namespace ajq;
 
@@ -244,18 +243,6 @@ int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream) {
   hipLaunchKernelGGL(repack_w8_kernel<true>, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, wq, N, K, reinterpret_cast<uint32_t*>(q));
   return check_launch("ajq_unrepack_w8");
-}
-
-int ajq_probe_mfma_rate(int random_operands, int iters, int workgroups, float* sink, long long* clocks,
-                        double* flops_per_launch, void* stream) {
-  if (!sink || !clocks) return fail(AJQ_ERR_NULL, "ajq_probe_mfma_rate: sink and clocks must be device buffers");
-  if (iters < 1 || workgroups < 1 || workgroups > 65536)
-    return fail(AJQ_ERR_SHAPE, "ajq_probe_mfma_rate: iters=%d, workgroups=%d out of range", iters, workgroups);
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(kProbeThreads), 0, (hipStream_t)stream,
-                     random_operands, iters, sink, clocks);
-  if (flops_per_launch)
-    *flops_per_launch = (double)workgroups * (kProbeThreads / 64) * (double)iters * kProbeChains * 32768.0;
-  return check_launch("ajq_probe_mfma_rate");
 }
 
 }  // extern "C"

@@ -24,6 +24,7 @@ beside it, token comparison between the two loops).  One JSON line is printed on
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -184,11 +185,9 @@ def bench_dense_library_gemm(m: int, n: int, k: int, steps: int, warmup: int, de
 def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launches: int = 4) -> dict:
     """bf16 MFMA rate the GPU sustains from registers alone (no memory traffic): with constant
     operands and with random mantissas, where the power limit lowers the shader clock."""
-    import ctypes
-
     from ajllm_amd import _lib
 
-    lib = _lib.load()
+    lib = _lib.load_bench()
     sink = torch.empty(workgroups * 512, dtype=torch.float32, device=device)
     clocks = torch.zeros(2, dtype=torch.int64, device=device)
     flops = ctypes.c_double(0.0)
@@ -196,8 +195,10 @@ def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launche
     out = {}
     for name, rnd in (("constant_operands", 0), ("random_operands", 1)):
         def launch():
-            _lib.check(lib.ajq_probe_mfma_rate(rnd, iters, workgroups, sink.data_ptr(), clocks.data_ptr(),
-                                               ctypes.addressof(flops), stream.cuda_stream), "ajq_probe_mfma_rate")
+            status = lib.ajqb_mfma_rate(rnd, iters, workgroups, sink.data_ptr(), clocks.data_ptr(),
+                                        ctypes.addressof(flops), stream.cuda_stream)
+            if status:
+                raise RuntimeError(f"ajqb_mfma_rate: {lib.ajqb_last_error().decode()}")
         launch()
         torch.cuda.synchronize()
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -210,6 +211,31 @@ def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launche
         cycles, ticks = (int(v) for v in clocks.tolist())
         out[name] = {"TFLOP/s": flops.value / seconds / 1e12, "ms_per_launch": seconds * 1e3,
                      "shader_clock_GHz": cycles / max(ticks, 1) * 0.1}
+    return out
+
+
+def bench_launch_alternatives(stages: int = 64, reps: int = 20) -> list[dict]:
+    """What a chain of 8.7 MB GEMVs costs per matrix under the alternatives to one launch per matrix
+    (``ajqb_launch_alternatives``: launches in a HIP graph, prefetch on a second graph branch or inside
+    the kernel, one launch for all stages with the activations exchanged through device memory)."""
+    from ajllm_amd import _lib
+
+    lib = _lib.load_bench()
+    results = (_lib.BenchResult * 32)()
+    count = ctypes.c_int(0)
+    status = lib.ajqb_launch_alternatives(stages, reps, results, 32, ctypes.byref(count))
+    if status:
+        raise RuntimeError(f"ajqb_launch_alternatives: {lib.ajqb_last_error().decode()}")
+    out = []
+    for r in results[: count.value]:
+        row = {"what": r.name.decode(), "us_per_matrix": r.us_per_stage}
+        if r.frac_hbm_peak > 0:
+            row["frac_hbm_peak"] = r.frac_hbm_peak
+        if r.matches_reference >= 0:
+            row["output_equals_reference_chain"] = bool(r.matches_reference)
+        if r.error_word:
+            row["error_word"] = r.error_word
+        out.append(row)
     return out
 
 
@@ -267,6 +293,8 @@ def main() -> int:
     ap.add_argument("--decode", action="store_true", help="also time end-to-end greedy decode")
     ap.add_argument("--stack", action="store_true",
                     help="also time the Llama-3-8B-shaped W8A16 stack (4 x 2048 prefill, batch-32 decode at context 2048)")
+    ap.add_argument("--probes", action="store_true",
+                    help="also time the alternatives to one launch per matrix for a chain of GEMVs (bench-only probes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="timed region only")
     args = ap.parse_args()
@@ -344,6 +372,10 @@ def main() -> int:
         from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
 
         extras["decode"] = bench_decode(device, log)
+    if args.probes:
+        extras["gemv_chain_launch_alternatives"] = bench_launch_alternatives()
+        for row in extras["gemv_chain_launch_alternatives"]:
+            log("probe", json.dumps(row))
     if args.stack:
         from ajllm_amd.stack_bench import bench_stack
 

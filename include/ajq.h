@@ -75,15 +75,6 @@ int ajq_w4a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, con
 int ajq_w8a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N2,
                         uint16_t* y, void* stream);
 
-/* Device yardstick, no counterpart in the reference: every wave issues bf16 MFMAs back to
- * back from registers (no memory traffic), so launches timed by the caller give the MFMA
- * rate the GPU sustains -- with constant operands (random_operands = 0: nominal clock) or
- * with random mantissas (1: the power-limited rate real data can approach).
- * sink: device float[workgroups * 512]; clocks: device int64[2], receives shader cycles and
- * 100 MHz ticks over the loop; *flops_per_launch (host, may be NULL) = flops one launch does. */
-int ajq_probe_mfma_rate(int random_operands, int iters, int workgroups, float* sink, long long* clocks,
-                        double* flops_per_launch, void* stream);
-
 int ajq_version(void);
 const char* ajq_last_error(void);
 const char* ajq_status_string(int status);

@@ -198,27 +198,27 @@ def test_linearity_at_full_size(cuda):
 
 
 def test_mfma_rate_probe_runs_and_reports_clocks(cuda):
-    """The device yardstick entry point: a short launch finishes, counts its flops and reports a
+    """The device yardstick of the bench-only library: a short launch finishes, counts its flops and reports a
     plausible shader clock (the rate itself is a measurement, not a pass criterion); bad arguments
     are refused."""
     import ctypes
 
     from ajllm_amd import _lib
-    lib = _lib.load()
+    lib = _lib.load_bench()
     sink = torch.zeros(8 * 512, dtype=torch.float32, device=cuda)
     clocks = torch.zeros(2, dtype=torch.int64, device=cuda)
     flops = ctypes.c_double(0.0)
     for random_operands in (0, 1):
-        status = lib.ajq_probe_mfma_rate(random_operands, 2000, 8, sink.data_ptr(), clocks.data_ptr(),
-                                         ctypes.addressof(flops), torch.cuda.current_stream().cuda_stream)
+        status = lib.ajqb_mfma_rate(random_operands, 2000, 8, sink.data_ptr(), clocks.data_ptr(),
+                                    ctypes.addressof(flops), torch.cuda.current_stream().cuda_stream)
         assert status == 0
         torch.cuda.synchronize()
         assert flops.value == 8 * 8 * 2000 * 4 * 32768.0
         cycles, ticks = (int(v) for v in clocks.tolist())
         assert ticks > 0 and 0.3 < cycles / ticks * 0.1 < 3.5  # GHz
         assert cycles >= 2000 * 4 * 32 * 0.9  # four 32-cycle MFMAs per iteration, issued in order
-    assert lib.ajq_probe_mfma_rate(0, 0, 8, sink.data_ptr(), clocks.data_ptr(), None, None) == -2
-    assert lib.ajq_probe_mfma_rate(0, 10, 8, None, clocks.data_ptr(), None, None) == -1
+    assert lib.ajqb_mfma_rate(0, 0, 8, sink.data_ptr(), clocks.data_ptr(), None, None) == -2
+    assert lib.ajqb_mfma_rate(0, 10, 8, None, clocks.data_ptr(), None, None) == -1
 
 
 def _random_shapes(count: int, seed: int):
@@ -332,3 +332,25 @@ def test_gemv_with_norm_or_gate_prologue_against_the_oracle(cuda, scheme, m, k):
     want = qspec.quant_linear(x, w_hat, accumulate=torch.float64, out_dtype=torch.float64)
     max_abs, rel = errors(y.cpu(), want)
     assert max_abs <= MAX_ABS_TOL and rel <= REL_FRO_TOL, (max_abs, rel)
+
+
+def test_launch_alternative_probes_reproduce_the_reference_chain(cuda):
+    """The bench-only probes of the alternatives to one launch per matrix (a chain of dependent GEMV
+    stages in ONE launch, activations exchanged through device memory behind flags or as stamped
+    records): a short run must finish without touching a spin limit and every dependent variant must
+    reproduce the per-stage-launch chain's last output bit for bit.  Timings are measurements, not
+    pass criteria."""
+    import ctypes
+
+    from ajllm_amd import _lib
+    lib = _lib.load_bench()
+    results = (_lib.BenchResult * 32)()
+    count = ctypes.c_int(0)
+    status = lib.ajqb_launch_alternatives(8, 2, results, 32, ctypes.byref(count))
+    assert status == 0, lib.ajqb_last_error().decode()
+    rows = results[: count.value]
+    assert len(rows) >= 12
+    compared = [r for r in rows if r.matches_reference >= 0]
+    assert len(compared) == 3 and all(r.matches_reference == 1 for r in compared)
+    assert all(r.error_word == 0 and r.us_per_stage > 0 for r in rows)
+    assert lib.ajqb_launch_alternatives(2, 2, results, 32, ctypes.byref(count)) == -2
