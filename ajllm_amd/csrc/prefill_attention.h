@@ -6,35 +6,40 @@
 //
 // q is fp32 [B, H, T, 128] (already rotated); keys and values are read where the model keeps
 // them, in the caches [B, Hkv, max_len, 128] (fp32 or bf16), rows 0 .. start + T - 1; out is
-// fp32 [B, T, H * 128], the layout the output projection takes.
+// fp32 or bf16 [B, T, H * 128], the layout the output projection takes.
 //
 // A workgroup of 4 waves owns 128 query rows of one (b, h), a wave two groups of 16 of them
-// (every key and value fragment read from LDS meets both), and walks the keys in blocks of 32.  Both products run transposed so that no operand changes layout
-// between them:
-//   S^T = K Q^T :  A = 16 keys x 32 dims from LDS (rows padded by 16 B), B = the wave's Q
-//                  fragments (registers, bf16, pre-scaled by log2(e) / sqrt(128));
-//                  lane (g = l / 16, r = l % 16) receives keys 4g..4g+3 of query row r;
-//   O^T += V^T P^T: the lane's 8 probabilities of a 32-key block ARE its B fragment
-//                  (contraction slot 8g + e <-> key 4g + e, or 16 + 4g + e - 4 for e >= 4), and
-//                  the A fragment takes the same keys of V^T, which is how V is laid down in
-//                  LDS (transposed on the way in, 2-byte stores).
-// Row maxima and sums need only the 4 lanes that share a query row (two shuffles).  The next
-// block of keys and values is fetched into registers while the current one is computed.  bf16
-// inputs, fp32 scores, probabilities rounded to bf16 for the second product, fp32 output
-// accumulators: the usual flash-attention arithmetic, not the eager fp32 one.
+// (every key and value fragment read from LDS meets both), and walks the keys in blocks of 64.
+// Both products run transposed so that no operand changes layout between them:
+//   S^T = K Q^T :  A = 16 keys x 32 dims from the row-major key tile in LDS, B = the wave's Q
+//                  fragments (registers, bf16, pre-scaled by log2(e) / sqrt(128)); lane
+//                  (g = l / 16, r = l % 16) receives keys 4g..4g+3 of query row r.  The
+//                  accumulator starts at minus the row's reference point, so the MFMA result is
+//                  the exponent itself.
+//   O^T += V^T P^T: the lane's 8 probabilities of a 32-key half ARE its B fragment (contraction
+//                  slot 8g + e <-> key 4g + e of the first 16-key tile for e < 4, of the second
+//                  for e >= 4), and the A fragment takes the same keys of V^T with two
+//                  transposing LDS reads (ds_read_b64_tr_b16) from the ROW-MAJOR value tile:
+//                  nothing is transposed on the way into LDS.
+// Both tiles are unpadded (a row is 256 B); the 16-byte chunks of a row sit in slots permuted by
+// the row index so that the fragment reads spread over all banks.
+//
+// Softmax bookkeeping is kept off the common path.  A row's reference point only moves when an
+// exponent would exceed 2^kPfSlack (always on the first block): the test is one compare of the
+// lane's sum of new probabilities (a sum of positives bounds each of them; inf passes it too),
+// and only then are the maxima taken (across the four lanes of a row with two lane swaps), the
+// probabilities recomputed and the accumulators rescaled.  Row sums stay per lane and meet once,
+// at the end.  bf16 inputs, fp32 scores, probabilities rounded to bf16 for the second product,
+// fp32 accumulators: the usual flash-attention arithmetic, not the eager fp32 one.
 #pragma once
 #include "ajq_common.h"
 
 namespace ajq {
 
-#ifndef AJQ_PF_QG
-#define AJQ_PF_QG 2
-#endif
-constexpr int kPfQG = AJQ_PF_QG;          // groups of 16 query rows per wave
-constexpr float kPfSlack = 8.0f;          // log2 of how far a row's scores may exceed its reference point
-constexpr int kPfBQ = 64 * kPfQG, kPfBK = 32, kPfHD = 128;
-constexpr int kPfKStride = kPfHD + 8;   // bf16 elements per K row in LDS
-constexpr int kPfVStride = kPfBK + 8;   // bf16 elements per V^T row in LDS (80 B: conflict-free 8-byte reads)
+constexpr float kPfSlack = 8.0f;          // log2 of how far a row's exponents may exceed its reference point
+constexpr float kPfTrigger = 4096.0f;     // lane sum of 16 probabilities above which the reference point is revisited
+constexpr int kPfBQ = 128, kPfBK = 64, kPfHD = 128;
+constexpr int kPfTileBytes = kPfBK * kPfHD * 2;  // 16 KiB: one block of keys (or values) as bf16
 
 __device__ __forceinline__ u32x4_t pack8_bf16(const float* v) {
   return u32x4_t{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
@@ -54,13 +59,52 @@ __device__ __forceinline__ u32x4_t to_bf16x8(const Raw8F32& r) {
 }
 __device__ __forceinline__ u32x4_t to_bf16x8(const u32x4_t& r) { return r; }
 
+// max / sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the lanes that share a query row):
+// v_permlane16_swap and v_permlane32_swap hand every lane its partner's value in one VALU
+// instruction each, without a trip through the LDS crossbar.
+__device__ __forceinline__ float quad_max(float x) {
+  typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+  uint32_t b = __float_as_uint(x);
+  u32x2v s = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  x = fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+  b = __float_as_uint(x);
+  s = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return fmaxf(__uint_as_float(s.x), __uint_as_float(s.y));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+  typedef uint32_t u32x2v __attribute__((ext_vector_type(2)));
+  uint32_t b = __float_as_uint(x);
+  u32x2v s = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  x = __uint_as_float(s.x) + __uint_as_float(s.y);
+  b = __float_as_uint(x);
+  s = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  return __uint_as_float(s.x) + __uint_as_float(s.y);
+}
+
+typedef short pf_i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) pf_i16x4_t pf_lds_i16x4_t;
+typedef __attribute__((address_space(3))) const u32x4_t pf_lds_u32x4_t;
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wint-to-pointer-cast"  // the host pass sees 64-bit pointers
+// Transposing LDS read: within each block of 16 lanes, lane 4 a + j receives element j of the
+// 8-byte rows addressed by lanes a, 4 + a, 8 + a and 12 + a of the block.
+__device__ __forceinline__ u32x2_t pf_read_tr(uint32_t address) {
+  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_lds_i16x4_t*)address));
+}
+__device__ __forceinline__ u32x4_t pf_read128(uint32_t address) { return *(pf_lds_u32x4_t*)address; }
+#pragma clang diagnostic pop
+
 template <typename CacheT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
                                                            const CacheT* __restrict__ vcache, int H, int Hkv, int T,
                                                            int start, int max_len, void* __restrict__ out, int out_bf16) {
-  // two buffers of each: a block is laid down while the previous one is still being read
-  __shared__ __attribute__((aligned(16))) uint16_t Ks2[2][kPfBK * kPfKStride];
-  __shared__ __attribute__((aligned(16))) uint16_t Vt2[2][kPfHD * kPfVStride];
+  // LDS map (the kernel declares no other LDS, so the array starts at address 0 and the reads
+  // below use absolute addresses): two stages of a key tile and a value tile, 16 KiB each.
+  //   stage s: keys at s * 32 Ki, values at s * 32 Ki + 16 Ki
+  // Key tile: 16-byte chunk c of key row k sits at k * 256 + 16 * (c ^ (k & 15)).
+  // Value tile: chunk c of row k sits at k * 256 + 16 * ((((c >> 1) ^ (k & 7)) << 1) | (c & 1))
+  // (32-byte segments permuted: a transposing read takes 8 bytes of each of 16 keys).
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPfTileBytes];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int qblocks = (T + kPfBQ - 1) / kPfBQ;
@@ -69,13 +113,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   const int q0 = qb * kPfBQ;
   const float qscale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
 
-  // ---- Q fragments of the wave's kPfQG groups of 16 rows: Q[qrow][32 s + 8 g .. + 8), scaled, bf16.
-  // Group u of wave w holds rows q0 + 16 (kPfQG w + u) .. + 15; this lane's row of it is qrow[u].
-  int qrow[kPfQG], q_pos[kPfQG];
-  u32x4_t qf[kPfQG][4];
+  // ---- Q fragments of the wave's two groups of 16 rows: Q[qrow][32 s + 8 g .. + 8), scaled, bf16.
+  // Group u of wave w holds rows q0 + 32 w + 16 u .. + 15; this lane's row of it is qrow[u].
+  int qrow[2], q_pos[2];
+  u32x4_t qf[2][4];
 #pragma unroll
-  for (int u = 0; u < kPfQG; ++u) {
-    qrow[u] = q0 + 16 * (kPfQG * wave + u) + r;
+  for (int u = 0; u < 2; ++u) {
+    qrow[u] = q0 + 32 * wave + 16 * u + r;
     q_pos[u] = start + qrow[u];
     const float* qp = q + ((size_t)bh * T + min(qrow[u], T - 1)) * kPfHD + 8 * g;
 #pragma unroll
@@ -90,134 +134,156 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   const CacheT* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
   const int kv_len = start + T;                               // rows the caches hold for this call
   const int kv_end = min(kv_len, start + q0 + kPfBQ);         // keys any row of this workgroup may see
+  const int nblk = (kv_end + kPfBK - 1) / kPfBK;
+  const int wave_last_pos = start + q0 + 32 * wave + 31;      // last query position of this wave
 
-  float m_run[kPfQG], l_run[kPfQG];
-  f32x4_t o[kPfQG][8];
+  float m_run[2], l_run[2];
+  f32x4_t negm[2];
+  f32x4_t o[2][8];
 #pragma unroll
-  for (int u = 0; u < kPfQG; ++u) {
-    m_run[u] = -INFINITY;
+  for (int u = 0; u < 2; ++u) {
+    m_run[u] = 0.f;
     l_run[u] = 0.f;
+    negm[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < 8; ++t) o[u][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // One block of keys and values in registers, as loaded (8 elements per chunk, two chunks per
-  // thread and operand): chunk c of K is (key c / 16, dims 8 (c % 16) ..), of V (key c % 32,
-  // dims 8 (c / 32) ..): keys vary fastest across the lanes that store V transposed.
+  // One block of keys and values in registers, as loaded: chunk ci = tid + 256 i (i < 4) is
+  // (key ci / 16, dims 8 (ci % 16) ..) of either tile; rows past the filled part of the cache
+  // repeat its last row (finite values; those keys are masked).
   typedef decltype(load8_raw(kbase)) raw8_t;
-  raw8_t kraw[2], vraw[2];
+  raw8_t kraw[4], vraw[4];
   auto fetch = [&](int kb0) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c = threadIdx.x + 256 * u;
-      kraw[u] = load8_raw(kbase + (size_t)min(kb0 + (c >> 4), kv_len - 1) * kPfHD + 8 * (c & 15));
-      vraw[u] = load8_raw(vbase + (size_t)min(kb0 + (c & 31), kv_len - 1) * kPfHD + 8 * (c >> 5));
+    for (int i = 0; i < 4; ++i) {
+      const int ci = threadIdx.x + 256 * i;
+      const size_t at = (size_t)min(kb0 + (ci >> 4), kv_len - 1) * kPfHD + 8 * (ci & 15);
+      kraw[i] = load8_raw(kbase + at);
+      vraw[i] = load8_raw(vbase + at);
     }
   };
-  // registers -> LDS: K block row-major (16-byte stores), V block transposed (2-byte stores)
-  auto lay_down = [&](int buf) {
+  // registers -> LDS, both tiles row-major, 16-byte stores into the permuted slots
+  uint32_t k_st[4], v_st[4];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c = threadIdx.x + 256 * u;
-      *reinterpret_cast<u32x4_t*>(Ks2[buf] + (c >> 4) * kPfKStride + 8 * (c & 15)) = to_bf16x8(kraw[u]);
-      const u32x4_t vv8 = to_bf16x8(vraw[u]);
-      uint16_t* dst = Vt2[buf] + (8 * (c >> 5)) * kPfVStride + (c & 31);
-      dst[0 * kPfVStride] = (uint16_t)(vv8.x & 0xFFFFu); dst[1 * kPfVStride] = (uint16_t)(vv8.x >> 16);
-      dst[2 * kPfVStride] = (uint16_t)(vv8.y & 0xFFFFu); dst[3 * kPfVStride] = (uint16_t)(vv8.y >> 16);
-      dst[4 * kPfVStride] = (uint16_t)(vv8.z & 0xFFFFu); dst[5 * kPfVStride] = (uint16_t)(vv8.z >> 16);
-      dst[6 * kPfVStride] = (uint16_t)(vv8.w & 0xFFFFu); dst[7 * kPfVStride] = (uint16_t)(vv8.w >> 16);
+  for (int i = 0; i < 4; ++i) {
+    const int ci = threadIdx.x + 256 * i, k = ci >> 4, c = ci & 15;
+    k_st[i] = (uint32_t)(k * 256 + 16 * (c ^ (k & 15)));
+    v_st[i] = (uint32_t)(kPfTileBytes + k * 256 + 16 * ((((c >> 1) ^ (k & 7)) << 1) | (c & 1)));
+  }
+  auto lay_down = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + k_st[i]) = to_bf16x8(kraw[i]);
+      *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + v_st[i]) = to_bf16x8(vraw[i]);
     }
   };
+  // ---- LDS read offsets within a stage.
+  // key fragment (tile jb, k-step s): row 16 jb + r, chunk 4 s + g  ->  (16 jb + r) * 256 + 16 * ((4 s + g) ^ r)
+  uint32_t k_rd[4];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) k_rd[s] = (uint32_t)(r * 256 + 16 * ((4 * s + g) ^ r));
+  // value fragment (half hf, slots 4 w2 .. 4 w2 + 3, dims 16 t ..): this lane addresses 8 bytes of key
+  // 32 hf + 16 w2 + 4 g + (r >> 2): piece (r & 3) of the 32-byte segment t, which sits in slot t ^ (key & 7)
+  const int vkey = 4 * g + (r >> 2);  // (16 w2 and 32 hf do not change key & 7)
+  uint32_t v_rd[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) v_rd[t] = (uint32_t)(kPfTileBytes + vkey * 256 + 32 * (t ^ (vkey & 7)) + 8 * (r & 3));
+
   fetch(0);
   lay_down(0);
-  if (kPfBK < kv_end) fetch(kPfBK);
+  if (nblk > 1) fetch(kPfBK);
   __syncthreads();
-  for (int kb0 = 0; kb0 < kv_end; kb0 += kPfBK) {
-    // One barrier per block: block kb0 is complete in buffer `cur` (laid down before the
-    // previous barrier); block kb0 + 32 goes from registers into the other buffer, which was
-    // last read before that barrier too; block kb0 + 64 starts its flight from memory.
-    const int cur = (kb0 / kPfBK) & 1;
-    const uint16_t* Ks = Ks2[cur];
-    const uint16_t* Vt = Vt2[cur];
-    if (kb0 + kPfBK < kv_end) {
-      lay_down(cur ^ 1);
-      if (kb0 + 2 * kPfBK < kv_end) fetch(kb0 + 2 * kPfBK);
+  for (int j = 0; j < nblk; ++j) {
+    // One barrier per block: block j is complete in stage j & 1 (laid down before the previous
+    // barrier); block j + 1 goes from registers into the other stage, which was last read before
+    // that barrier too; block j + 2 starts its flight from memory.
+    const int kb0 = j * kPfBK;
+    const uint32_t stage = (uint32_t)((j & 1) * 2 * kPfTileBytes);
+    if (j + 1 < nblk) {
+      lay_down((j + 1) & 1);
+      if (j + 2 < nblk) fetch(kb0 + 2 * kPfBK);
     }
-    // ---- scores of the two 16-key halves: sc[u][jb][i] = S[qrow[u]][key kb0 + 16 jb + 4 g + i]
-    // (log2 units); a key fragment is read once for all the wave's query groups
-    f32x4_t sc[kPfQG][2];
+    // a wave whose last query lies before the block has nothing to add (uniform per wave)
+    if (kb0 <= wave_last_pos) {
+      // ---- exponents of the four 16-key tiles: sc[u][jb][i] = S[qrow[u]][key kb0 + 16 jb + 4 g + i] - m_run[u]
+      // (log2 units); a key fragment is read once for both query groups
+      f32x4_t sc[2][4];
 #pragma unroll
-    for (int jb = 0; jb < 2; ++jb) {
+      for (int jb = 0; jb < 4; ++jb) {
 #pragma unroll
-      for (int u = 0; u < kPfQG; ++u) sc[u][jb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < 4; ++s) {
+          const u32x4_t a = pf_read128(stage + (uint32_t)(jb * 16 * 256) + k_rd[s]);
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(Ks + (16 * jb + r) * kPfKStride + 32 * s + 8 * g);
-#pragma unroll
-        for (int u = 0; u < kPfQG; ++u) sc[u][jb] = mfma16(a, qf[u][s], sc[u][jb]);
-      }
-    }
-    u32x4_t pf[kPfQG];
-    float corr[kPfQG];
-    // only blocks that reach past the wave's first query position need the causal mask
-    const bool diagonal = kb0 + kPfBK - 1 > start + q0 + 16 * kPfQG * wave;
-#pragma unroll
-    for (int u = 0; u < kPfQG; ++u) {
-      float p[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) p[e] = sc[u][e >> 2][e & 3];
-      if (diagonal) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int key_pos = kb0 + 16 * (e >> 2) + 4 * g + (e & 3);
-          if (key_pos > q_pos[u]) p[e] = -INFINITY;  // (also hides rows past kv_len)
+          for (int u = 0; u < 2; ++u) sc[u][jb] = mfma16(a, qf[u][s], s == 0 ? negm[u] : sc[u][jb]);
         }
       }
-      float mx = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      // The reference point of the row's exponentials moves only when the maximum has grown
-      // by more than 2^kPfSlack since it was set: probabilities stay below 2^kPfSlack (fp32
-      // sums and bf16 operands take that easily) and the accumulators are rescaled rarely.
-      const float m_new = mx > m_run[u] + kPfSlack ? mx : m_run[u];
-      corr[u] = __builtin_amdgcn_exp2f(m_run[u] - m_new);  // 1 when unchanged, 0 on the first block
-      float rowsum = 0.f;
+      // only blocks that reach past the wave's first query position need the causal mask
+      if (kb0 + kPfBK - 1 > wave_last_pos - 31) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        p[e] = __builtin_amdgcn_exp2f(p[e] - m_new);  // v_exp_f32: underflow to 0 is what is wanted
-        rowsum += p[e];
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (kb0 + 16 * jb + 4 * g + i > q_pos[u]) sc[u][jb][i] = -INFINITY;  // (also hides rows past kv_len)
       }
-      rowsum += __shfl_xor(rowsum, 16);
-      rowsum += __shfl_xor(rowsum, 32);
-      l_run[u] = l_run[u] * corr[u] + rowsum;
-      m_run[u] = m_new;
-      pf[u] = pack8_bf16(p);
-    }
-    bool rescale = false;
+      // The reference point of a row moves only when an exponent has outgrown it by more than
+      // kPfSlack (and on the first block, where it is still arbitrary).  One query group at a
+      // time, so that only one group's exponents and probabilities are live together.
+      u32x4_t pf[2][2];
 #pragma unroll
-    for (int u = 0; u < kPfQG; ++u) rescale |= corr[u] != 1.0f;
-    if (__builtin_amdgcn_ballot_w64(rescale) != 0) {
+      for (int u = 0; u < 2; ++u) {
+        float p[16], psum = 0.f;
 #pragma unroll
-      for (int u = 0; u < kPfQG; ++u)
+        for (int e = 0; e < 16; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(sc[u][e >> 2][e & 3]);  // v_exp_f32: underflow to 0 is what is wanted
+          psum += p[e];
+        }
+        const bool revisit = j == 0 || psum > kPfTrigger;
+        if (__builtin_amdgcn_ballot_w64(revisit) != 0) {
+          float mx = -INFINITY;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) o[u][t] *= corr[u];
-    }
-    // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the 32 keys; a value fragment is read once
+          for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[u][e >> 2][e & 3]);
+          mx = quad_max(mx);
+          const bool move = j == 0 || mx > kPfSlack;
+          const float shift = move ? mx : 0.f;
+          const float corr = (move && j != 0) ? __builtin_amdgcn_exp2f(-shift) : 1.0f;
+          psum = 0.f;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const uint16_t* vrow = Vt + (16 * t + r) * kPfVStride + 4 * g;
-      const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(vrow);        // keys 4g .. 4g+3
-      const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(vrow + 16);   // keys 16+4g .. 16+4g+3
-      const u32x4_t vf = {lo.x, lo.y, hi.x, hi.y};
+          for (int e = 0; e < 16; ++e) {
+            p[e] = __builtin_amdgcn_exp2f(sc[u][e >> 2][e & 3] - shift);
+            psum += p[e];
+          }
+          m_run[u] += shift;
+          negm[u] = f32x4_t{-m_run[u], -m_run[u], -m_run[u], -m_run[u]};
+          l_run[u] *= corr;
 #pragma unroll
-      for (int u = 0; u < kPfQG; ++u) o[u][t] = mfma16(vf, pf[u], o[u][t]);
+          for (int t = 0; t < 8; ++t) o[u][t] *= corr;
+        }
+        l_run[u] += psum;
+        pf[u][0] = pack8_bf16(&p[0]);
+        pf[u][1] = pack8_bf16(&p[8]);
+      }
+      // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the keys of each 32-key half; a value fragment is read once
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          const u32x2_t lo = pf_read_tr(stage + (uint32_t)(hf * 32 * 256) + v_rd[t]);             // tile 2 hf
+          const u32x2_t hi = pf_read_tr(stage + (uint32_t)(hf * 32 * 256 + 16 * 256) + v_rd[t]);  // tile 2 hf + 1
+          const u32x4_t vf = {lo.x, lo.y, hi.x, hi.y};
+#pragma unroll
+          for (int u = 0; u < 2; ++u) o[u][t] = mfma16(vf, pf[u][hf], o[u][t]);
+        }
+      }
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int u = 0; u < kPfQG; ++u) {
+  for (int u = 0; u < 2; ++u) {
+    const float inv = 1.0f / quad_sum(l_run[u]);
     if (qrow[u] >= T) continue;
-    const float inv = 1.0f / l_run[u];
     const size_t at = ((size_t)b * T + qrow[u]) * ((size_t)H * kPfHD) + (size_t)h * kPfHD + 4 * g;
     if (out_bf16) {
       uint16_t* dst = reinterpret_cast<uint16_t*>(out) + at;
