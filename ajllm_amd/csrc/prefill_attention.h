@@ -33,6 +33,7 @@
 // fp32 accumulators: the usual flash-attention arithmetic, not the eager fp32 one.
 #pragma once
 #include "ajq_common.h"
+#include "gemm_kernels.h"  // dma16: global -> LDS without registers
 
 namespace ajq {
 
@@ -84,6 +85,7 @@ __device__ __forceinline__ float quad_sum(float x) {
 typedef short pf_i16x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) pf_i16x4_t pf_lds_i16x4_t;
 typedef __attribute__((address_space(3))) const u32x4_t pf_lds_u32x4_t;
+typedef __attribute__((address_space(3))) unsigned char pf_lds_char_t;
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Wint-to-pointer-cast"  // the host pass sees 64-bit pointers
 // Transposing LDS read: within each block of 16 lanes, lane 4 a + j receives element j of the
@@ -98,14 +100,16 @@ template <typename CacheT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
                                                            const CacheT* __restrict__ vcache, int H, int Hkv, int T,
                                                            int start, int max_len, void* __restrict__ out, int out_bf16) {
-  // LDS map (the kernel declares no other LDS, so the array starts at address 0 and the reads
-  // below use absolute addresses): two stages of a key tile and a value tile, 16 KiB each.
+  // LDS map (byte addresses relative to lds0, the array's LDS address, which is 0 because the kernel
+  // declares no other LDS; naming it also keeps the array allocated when nothing else refers to
+  // it): two stages of a key tile and a value tile, 16 KiB each.
   //   stage s: keys at s * 32 Ki, values at s * 32 Ki + 16 Ki
   // Key tile: 16-byte chunk c of key row k sits at k * 256 + 16 * (c ^ (k & 15)).
   // Value tile: chunk c of row k sits at k * 256 + 16 * ((((c >> 1) ^ (k & 7)) << 1) | (c & 1))
   // (32-byte segments permuted: a transposing read takes 8 bytes of each of 16 keys).
   __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * kPfTileBytes];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(pf_lds_char_t*)lds;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int qblocks = (T + kPfBQ - 1) / kPfBQ;
   const int qb = qblocks - 1 - blockIdx.x;  // the long rows first
@@ -149,73 +153,126 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
     for (int t = 0; t < 8; ++t) o[u][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // One block of keys and values in registers, as loaded: chunk ci = tid + 256 i (i < 4) is
-  // (key ci / 16, dims 8 (ci % 16) ..) of either tile; rows past the filled part of the cache
-  // repeat its last row (finite values; those keys are masked).
+  // ---- Keys and values on their way into LDS.
+  // bf16 caches: global -> LDS directly, one block ahead.  A wave-wide request fills 1 KiB = 4 key
+  // rows; wave w takes rows 4 w .. 4 w + 3 of every group of 16, so (row & 15) = 4 w + lane / 16 is
+  // fixed per lane and the chunk it must fetch for its slot is too.
+  // fp32 caches: through registers (converted on the way), one block in registers while the
+  // previous one is being read: chunk ci = tid + 256 i (i < 4) is (key ci / 16, dims 8 (ci % 16) ..).
+  // Rows past the filled part of the cache repeat its last row (finite values; those keys are masked).
+#ifndef AJQ_PF_DMA
+#define AJQ_PF_DMA 1
+#endif
+#ifndef AJQ_PF_PRE
+#define AJQ_PF_PRE 1
+#endif
+  constexpr bool kDma = sizeof(CacheT) == 2 && AJQ_PF_DMA;
+  constexpr bool kPre = kDma && AJQ_PF_PRE;
+  const int krow = 4 * wave + (lane >> 4), slot = lane & 15;
+  const uint32_t k_chunk = (uint32_t)(slot ^ krow);
+  const uint32_t v_chunk = (uint32_t)((((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1));
+  auto issue_dma = [&](int jblk) {
+    const int kb0 = jblk * kPfBK;
+    const uint32_t stage = lds0 + (uint32_t)((jblk & 1) * 2 * kPfTileBytes);
+    if (kb0 + kPfBK <= kv_len) {
+      const uint32_t kv = (uint32_t)(krow * 256) + k_chunk * 16u, vv = (uint32_t)(krow * 256) + v_chunk * 16u;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const size_t row0 = (size_t)(kb0 + 16 * i) * 256;
+        dma16(reinterpret_cast<const char*>(kbase) + row0, kv, stage + (uint32_t)((wave + 4 * i) * 1024));
+        dma16(reinterpret_cast<const char*>(vbase) + row0, vv, stage + (uint32_t)(kPfTileBytes + (wave + 4 * i) * 1024));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t row = (uint32_t)min(kb0 + 16 * i + krow, kv_len - 1) * 256u;
+        dma16(kbase, row + k_chunk * 16u, stage + (uint32_t)((wave + 4 * i) * 1024));
+        dma16(vbase, row + v_chunk * 16u, stage + (uint32_t)(kPfTileBytes + (wave + 4 * i) * 1024));
+      }
+    }
+  };
   typedef decltype(load8_raw(kbase)) raw8_t;
-  raw8_t kraw[4], vraw[4];
+  raw8_t kraw[kDma ? 1 : 4], vraw[kDma ? 1 : 4];
+  uint32_t k_st[kDma ? 1 : 4], v_st[kDma ? 1 : 4];
   auto fetch = [&](int kb0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < (kDma ? 0 : 4); ++i) {
       const int ci = threadIdx.x + 256 * i;
       const size_t at = (size_t)min(kb0 + (ci >> 4), kv_len - 1) * kPfHD + 8 * (ci & 15);
       kraw[i] = load8_raw(kbase + at);
       vraw[i] = load8_raw(vbase + at);
     }
   };
-  // registers -> LDS, both tiles row-major, 16-byte stores into the permuted slots
-  uint32_t k_st[4], v_st[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < (kDma ? 0 : 4); ++i) {
     const int ci = threadIdx.x + 256 * i, k = ci >> 4, c = ci & 15;
     k_st[i] = (uint32_t)(k * 256 + 16 * (c ^ (k & 15)));
     v_st[i] = (uint32_t)(kPfTileBytes + k * 256 + 16 * ((((c >> 1) ^ (k & 7)) << 1) | (c & 1)));
   }
   auto lay_down = [&](int stage) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < (kDma ? 0 : 4); ++i) {
       *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + k_st[i]) = to_bf16x8(kraw[i]);
       *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + v_st[i]) = to_bf16x8(vraw[i]);
     }
   };
-  // ---- LDS read offsets within a stage.
+  // ---- LDS read addresses (of the stage being read; flipped to the other stage after every block).
   // key fragment (tile jb, k-step s): row 16 jb + r, chunk 4 s + g  ->  (16 jb + r) * 256 + 16 * ((4 s + g) ^ r)
   uint32_t k_rd[4];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) k_rd[s] = (uint32_t)(r * 256 + 16 * ((4 * s + g) ^ r));
+  for (int s = 0; s < 4; ++s) k_rd[s] = lds0 + (uint32_t)(r * 256 + 16 * ((4 * s + g) ^ r));
   // value fragment (half hf, slots 4 w2 .. 4 w2 + 3, dims 16 t ..): this lane addresses 8 bytes of key
   // 32 hf + 16 w2 + 4 g + (r >> 2): piece (r & 3) of the 32-byte segment t, which sits in slot t ^ (key & 7)
   const int vkey = 4 * g + (r >> 2);  // (16 w2 and 32 hf do not change key & 7)
   uint32_t v_rd[8];
 #pragma unroll
-  for (int t = 0; t < 8; ++t) v_rd[t] = (uint32_t)(kPfTileBytes + vkey * 256 + 32 * (t ^ (vkey & 7)) + 8 * (r & 3));
+  for (int t = 0; t < 8; ++t) v_rd[t] = lds0 + (uint32_t)(kPfTileBytes + vkey * 256 + 32 * (t ^ (vkey & 7)) + 8 * (r & 3));
 
-  fetch(0);
-  lay_down(0);
-  if (nblk > 1) fetch(kPfBK);
+  if (kDma) {
+    issue_dma(0);
+  } else {
+    fetch(0);
+    lay_down(0);
+    if (nblk > 1) fetch(kPfBK);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   for (int j = 0; j < nblk; ++j) {
-    // One barrier per block: block j is complete in stage j & 1 (laid down before the previous
-    // barrier); block j + 1 goes from registers into the other stage, which was last read before
-    // that barrier too; block j + 2 starts its flight from memory.
+    // One barrier per block: block j is complete in stage j & 1 (it landed before the previous
+    // barrier); block j + 1 goes into the other stage, which was last read before that barrier
+    // too (fp32 caches: from registers, while block j + 2 starts its flight from memory).
     const int kb0 = j * kPfBK;
-    const uint32_t stage = (uint32_t)((j & 1) * 2 * kPfTileBytes);
     if (j + 1 < nblk) {
-      lay_down((j + 1) & 1);
-      if (j + 2 < nblk) fetch(kb0 + 2 * kPfBK);
+      if (kDma) {
+        issue_dma(j + 1);
+      } else {
+        lay_down((j + 1) & 1);
+        if (j + 2 < nblk) fetch(kb0 + 2 * kPfBK);
+      }
     }
-    // a wave whose last query lies before the block has nothing to add (uniform per wave)
+    // a wave whose last query lies before the block has nothing to add
     if (kb0 <= wave_last_pos) {
       // ---- exponents of the four 16-key tiles: sc[u][jb][i] = S[qrow[u]][key kb0 + 16 jb + 4 g + i] - m_run[u]
-      // (log2 units); a key fragment is read once for both query groups
+      // (log2 units).  k-step outermost: the eight products of a step are independent, and a key
+      // fragment is read once for both query groups.
       f32x4_t sc[2][4];
+      u32x4_t ka[4];
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) {
+      for (int jb = 0; jb < 4; ++jb) ka[jb] = pf_read128(k_rd[0] + (uint32_t)(jb * 16 * 256));
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const u32x4_t a = pf_read128(stage + (uint32_t)(jb * 16 * 256) + k_rd[s]);
+      for (int s = 0; s < 4; ++s) {
+        u32x4_t kn[4];
+        if (kPre && s < 3) {  // (the fp32 path has no registers to spare for a second set)
 #pragma unroll
-          for (int u = 0; u < 2; ++u) sc[u][jb] = mfma16(a, qf[u][s], s == 0 ? negm[u] : sc[u][jb]);
+          for (int jb = 0; jb < 4; ++jb) kn[jb] = pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
+        }
+#pragma unroll
+        for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+          for (int u = 0; u < 2; ++u) sc[u][jb] = mfma16(ka[jb], qf[u][s], s == 0 ? negm[u] : sc[u][jb]);
+        if (s < 3) {
+#pragma unroll
+          for (int jb = 0; jb < 4; ++jb) ka[jb] = kPre ? kn[jb] : pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
         }
       }
       // only blocks that reach past the wave's first query position need the causal mask
@@ -265,19 +322,36 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
         pf[u][0] = pack8_bf16(&p[0]);
         pf[u][1] = pack8_bf16(&p[8]);
       }
-      // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the keys of each 32-key half; a value fragment is read once
+      // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the keys of each 32-key half; a value fragment
+      // (two transposing reads: the half's first and second 16-key tile) meets both query groups.
+      // The second half's fragments are requested as the first half's are consumed.
+      constexpr int kRing = kPre ? 8 : 4;  // fragments in flight (the fp32 path has fewer registers to spare)
+      auto v_lo = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256)); };
+      auto v_hi = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256 + 16 * 256)); };
+      u32x2_t vlo[kRing], vhi[kRing];
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
+      for (int i = 0; i < kRing; ++i) {
+        vlo[i] = v_lo(i);
+        vhi[i] = v_hi(i);
+      }
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          const u32x2_t lo = pf_read_tr(stage + (uint32_t)(hf * 32 * 256) + v_rd[t]);             // tile 2 hf
-          const u32x2_t hi = pf_read_tr(stage + (uint32_t)(hf * 32 * 256 + 16 * 256) + v_rd[t]);  // tile 2 hf + 1
-          const u32x4_t vf = {lo.x, lo.y, hi.x, hi.y};
+      for (int i = 0; i < 16; ++i) {  // i = 8 hf + t
+        const u32x4_t vf = {vlo[i % kRing].x, vlo[i % kRing].y, vhi[i % kRing].x, vhi[i % kRing].y};
 #pragma unroll
-          for (int u = 0; u < 2; ++u) o[u][t] = mfma16(vf, pf[u][hf], o[u][t]);
+        for (int u = 0; u < 2; ++u) o[u][i & 7] = mfma16(vf, pf[u][i >> 3], o[u][i & 7]);
+        if (i + kRing < 16) {
+          vlo[i % kRing] = v_lo(i + kRing);
+          vhi[i % kRing] = v_hi(i + kRing);
         }
       }
     }
+    // flip every read address to the other stage
+#pragma unroll
+    for (int s = 0; s < 4; ++s) k_rd[s] ^= (uint32_t)(2 * kPfTileBytes);
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v_rd[t] ^= (uint32_t)(2 * kPfTileBytes);
+    // the next block must have landed and every wave must be done with this one
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 #pragma unroll
