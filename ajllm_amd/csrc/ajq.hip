@@ -923,7 +923,7 @@ int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int
   const int out_bf16 = out_dtype == AJQ_OUT_BF16;
   if (!aligned16(q) || !aligned16(kcache) || !aligned16(vcache) || !aligned16(out))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_prefill: q, the caches and out must be 16-byte aligned");
-  const dim3 grid((T + kPfBQ - 1) / kPfBQ, B * H);
+  const dim3 grid((unsigned)(((T + kPfBQ - 1) / kPfBQ) * B * H));  // (the kernel orders the work by cost)
   if (cache_dtype == AJQ_KV_F32)
     hipLaunchKernelGGL(attn_prefill_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, q,
                        reinterpret_cast<const float*>(kcache), reinterpret_cast<const float*>(vcache), H, Hkv, T, start,

@@ -111,29 +111,26 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   const uint32_t lds0 = (uint32_t)(uintptr_t)(pf_lds_char_t*)lds;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
+  // Work order.  The hardware deals workgroups to the 8 XCDs round-robin by linear index and,
+  // inside an XCD, hands the next one to whichever CU has room.  A query block's cost grows with
+  // its position (causal), so the linear order is: XCD k takes a contiguous eighth of the (b, h)
+  // pairs (the heads that share a cache head stay on one XCD and its L2) and walks its query
+  // blocks from the longest to the shortest.  (With B * H not a multiple of 8: plain longest first.)
   const int qblocks = (T + kPfBQ - 1) / kPfBQ;
-  const int qb = qblocks - 1 - blockIdx.x;  // the long rows first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H, hk = h / (H / Hkv);
+  const int BH = (int)(gridDim.x / (unsigned)qblocks);
+  int qb, bh;
+  if ((BH & 7) == 0) {
+    const int per_xcd = BH >> 3, m = (int)(blockIdx.x >> 3);
+    qb = qblocks - 1 - m / per_xcd;
+    bh = (int)(blockIdx.x & 7) * per_xcd + m % per_xcd;
+  } else {
+    qb = qblocks - 1 - (int)blockIdx.x / BH;
+    bh = (int)blockIdx.x % BH;
+  }
+  const int b = bh / H, h = bh % H, hk = h / (H / Hkv);
   const int q0 = qb * kPfBQ;
   const float qscale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
 
-  // ---- Q fragments of the wave's two groups of 16 rows: Q[qrow][32 s + 8 g .. + 8), scaled, bf16.
-  // Group u of wave w holds rows q0 + 32 w + 16 u .. + 15; this lane's row of it is qrow[u].
-  int qrow[2], q_pos[2];
-  u32x4_t qf[2][4];
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    qrow[u] = q0 + 32 * wave + 16 * u + r;
-    q_pos[u] = start + qrow[u];
-    const float* qp = q + ((size_t)bh * T + min(qrow[u], T - 1)) * kPfHD + 8 * g;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const float4 a = reinterpret_cast<const float4*>(qp + 32 * s)[0], c = reinterpret_cast<const float4*>(qp + 32 * s)[1];
-      const float v[8] = {a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale,
-                          c.x * qscale, c.y * qscale, c.z * qscale, c.w * qscale};
-      qf[u][s] = pack8_bf16(v);
-    }
-  }
   const CacheT* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
   const CacheT* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
   const int kv_len = start + T;                               // rows the caches hold for this call
@@ -160,35 +157,23 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   // fp32 caches: through registers (converted on the way), one block in registers while the
   // previous one is being read: chunk ci = tid + 256 i (i < 4) is (key ci / 16, dims 8 (ci % 16) ..).
   // Rows past the filled part of the cache repeat its last row (finite values; those keys are masked).
-#ifndef AJQ_PF_DMA
-#define AJQ_PF_DMA 1
-#endif
-#ifndef AJQ_PF_PRE
-#define AJQ_PF_PRE 1
-#endif
-  constexpr bool kDma = sizeof(CacheT) == 2 && AJQ_PF_DMA;
-  constexpr bool kPre = kDma && AJQ_PF_PRE;
+  constexpr bool kDma = sizeof(CacheT) == 2;
   const int krow = 4 * wave + (lane >> 4), slot = lane & 15;
   const uint32_t k_chunk = (uint32_t)(slot ^ krow);
   const uint32_t v_chunk = (uint32_t)((((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1));
-  auto issue_dma = [&](int jblk) {
+  // part i (0 .. 3) of block jblk: this wave's 4 key rows and 4 value rows of the i-th group of 16
+  auto issue_dma = [&](int jblk, int i) {
     const int kb0 = jblk * kPfBK;
     const uint32_t stage = lds0 + (uint32_t)((jblk & 1) * 2 * kPfTileBytes);
+    const uint32_t k_to = stage + (uint32_t)((wave + 4 * i) * 1024), v_to = k_to + (uint32_t)kPfTileBytes;
     if (kb0 + kPfBK <= kv_len) {
-      const uint32_t kv = (uint32_t)(krow * 256) + k_chunk * 16u, vv = (uint32_t)(krow * 256) + v_chunk * 16u;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const size_t row0 = (size_t)(kb0 + 16 * i) * 256;
-        dma16(reinterpret_cast<const char*>(kbase) + row0, kv, stage + (uint32_t)((wave + 4 * i) * 1024));
-        dma16(reinterpret_cast<const char*>(vbase) + row0, vv, stage + (uint32_t)(kPfTileBytes + (wave + 4 * i) * 1024));
-      }
+      const size_t row0 = (size_t)(kb0 + 16 * i) * 256;
+      dma16(reinterpret_cast<const char*>(kbase) + row0, (uint32_t)(krow * 256) + k_chunk * 16u, k_to);
+      dma16(reinterpret_cast<const char*>(vbase) + row0, (uint32_t)(krow * 256) + v_chunk * 16u, v_to);
     } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t row = (uint32_t)min(kb0 + 16 * i + krow, kv_len - 1) * 256u;
-        dma16(kbase, row + k_chunk * 16u, stage + (uint32_t)((wave + 4 * i) * 1024));
-        dma16(vbase, row + v_chunk * 16u, stage + (uint32_t)(kPfTileBytes + (wave + 4 * i) * 1024));
-      }
+      const uint32_t row = (uint32_t)min(kb0 + 16 * i + krow, kv_len - 1) * 256u;
+      dma16(kbase, row + k_chunk * 16u, k_to);
+      dma16(vbase, row + v_chunk * 16u, v_to);
     }
   };
   typedef decltype(load8_raw(kbase)) raw8_t;
@@ -229,11 +214,30 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   for (int t = 0; t < 8; ++t) v_rd[t] = lds0 + (uint32_t)(kPfTileBytes + vkey * 256 + 32 * (t ^ (vkey & 7)) + 8 * (r & 3));
 
   if (kDma) {
-    issue_dma(0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_dma(0, i);
   } else {
     fetch(0);
     lay_down(0);
     if (nblk > 1) fetch(kPfBK);
+  }
+  // ---- (after the first block's requests, so that both round trips to memory overlap)
+  // Q fragments of the wave's two groups of 16 rows: Q[qrow][32 s + 8 g .. + 8), scaled, bf16.
+  // Group u of wave w holds rows q0 + 32 w + 16 u .. + 15; this lane's row of it is qrow[u].
+  int qrow[2], q_pos[2];
+  u32x4_t qf[2][4];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    qrow[u] = q0 + 32 * wave + 16 * u + r;
+    q_pos[u] = start + qrow[u];
+    const float* qp = q + ((size_t)bh * T + min(qrow[u], T - 1)) * kPfHD + 8 * g;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const float4 a = reinterpret_cast<const float4*>(qp + 32 * s)[0], c = reinterpret_cast<const float4*>(qp + 32 * s)[1];
+      const float v[8] = {a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale,
+                          c.x * qscale, c.y * qscale, c.z * qscale, c.w * qscale};
+      qf[u][s] = pack8_bf16(v);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -242,9 +246,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
     // barrier); block j + 1 goes into the other stage, which was last read before that barrier
     // too (fp32 caches: from registers, while block j + 2 starts its flight from memory).
     const int kb0 = j * kPfBK;
-    if (j + 1 < nblk) {
+    // bf16 caches: the requests for block j + 1 are issued between the products below (one part
+    // per k-step), or here by a wave that has no products to form
+    const bool more = j + 1 < nblk;
+    if (more) {
       if (kDma) {
-        issue_dma(j + 1);
+        if (kb0 > wave_last_pos) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) issue_dma(j + 1, i);
+        }
       } else {
         lay_down((j + 1) & 1);
         if (j + 2 < nblk) fetch(kb0 + 2 * kPfBK);
@@ -262,7 +272,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         u32x4_t kn[4];
-        if (kPre && s < 3) {  // (the fp32 path has no registers to spare for a second set)
+        if (kDma && s < 3) {  // (the fp32 path has no registers to spare for a second set)
 #pragma unroll
           for (int jb = 0; jb < 4; ++jb) kn[jb] = pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
         }
@@ -270,9 +280,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
         for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
           for (int u = 0; u < 2; ++u) sc[u][jb] = mfma16(ka[jb], qf[u][s], s == 0 ? negm[u] : sc[u][jb]);
+        if (kDma && more) issue_dma(j + 1, s);
         if (s < 3) {
 #pragma unroll
-          for (int jb = 0; jb < 4; ++jb) ka[jb] = kPre ? kn[jb] : pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
+          for (int jb = 0; jb < 4; ++jb) ka[jb] = kDma ? kn[jb] : pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
         }
       }
       // only blocks that reach past the wave's first query position need the causal mask
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
       // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the keys of each 32-key half; a value fragment
       // (two transposing reads: the half's first and second 16-key tile) meets both query groups.
       // The second half's fragments are requested as the first half's are consumed.
-      constexpr int kRing = kPre ? 8 : 4;  // fragments in flight (the fp32 path has fewer registers to spare)
+      constexpr int kRing = kDma ? 8 : 4;  // fragments in flight (the fp32 path has fewer registers to spare)
       auto v_lo = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256)); };
       auto v_hi = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256 + 16 * 256)); };
       u32x2_t vlo[kRing], vhi[kRing];

@@ -274,7 +274,8 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
 
 @pytest.mark.parametrize("b,heads,kv_heads,t,start,cache_dtype", [
     (2, 4, 2, 100, 0, torch.float32), (1, 2, 2, 64, 0, torch.float32), (1, 4, 1, 130, 37, torch.float32),
-    (3, 2, 1, 257, 5, torch.bfloat16), (1, 1, 1, 1, 9, torch.float32), (1, 8, 2, 512, 0, torch.bfloat16)])
+    (3, 2, 1, 257, 5, torch.bfloat16), (1, 1, 1, 1, 9, torch.float32), (1, 8, 2, 512, 0, torch.bfloat16),
+    (1, 32, 8, 2048, 0, torch.bfloat16), (2, 8, 8, 300, 131, torch.bfloat16), (1, 3, 1, 200, 70, torch.float32)])
 def test_flash_prefill_attention(cuda, b, heads, kv_heads, t, start, cache_dtype):
     """ajq_attn_prefill against the model code's masked softmax attention.  The kernel rounds q, k, v
     and the probabilities to bf16 (flash-attention arithmetic): compared with the fp32 statement on the
