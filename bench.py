@@ -182,6 +182,30 @@ def bench_dense_library_gemm(m: int, n: int, k: int, steps: int, warmup: int, de
             "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS}
 
 
+def bench_flash_prefill(batch: int, heads: int, kv_heads: int, seq: int, cache_dtype, device, reps: int = 10) -> dict:
+    """Causal prefill attention (``ajq_attn_prefill``) on config 5's prefill shape: head_dim 128,
+    fp32 queries, bf16 output; flops counted for the causal half only."""
+    from ajllm_amd.attention import flash_prefill
+
+    g = torch.Generator(device="cpu").manual_seed(11)
+    q = torch.randn((batch, heads, seq, 128), generator=g).to(device)
+    keys = torch.randn((batch, kv_heads, seq, 128), generator=g).to(device).to(cache_dtype)
+    values = torch.randn((batch, kv_heads, seq, 128), generator=g).to(device).to(cache_dtype)
+    for _ in range(3):
+        flash_prefill(q, keys, values, 0, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        flash_prefill(q, keys, values, 0, out_dtype=torch.bfloat16)
+    end.record()
+    end.synchronize()
+    us = start.elapsed_time(end) * 1e3 / reps
+    flops = 4.0 * batch * heads * seq * seq * 0.5 * 128
+    return {"B": batch, "H": heads, "Hkv": kv_heads, "T": seq, "kv_cache": str(cache_dtype).replace("torch.", ""),
+            "us_per_call": us, "causal_TFLOP/s": flops / us * 1e-6, "frac_mfma_peak": flops / us * 1e-6 / MFMA_BF16_PEAK_TFLOPS}
+
+
 def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launches: int = 4) -> dict:
     """bf16 MFMA rate the GPU sustains from registers alone (no memory traffic): with constant
     operands and with random mantissas, where the power limit lowers the shader clock."""
@@ -337,6 +361,11 @@ def main() -> int:
                     "expanded to bf16, and the MFMA rate sustained with no memory traffic (random operands "
                     "reach the power limit and the shader clock drops)",
         }
+    if not args.no_extras:
+        flash = [bench_flash_prefill(4, 32, 8, 2048, dt, device) for dt in (torch.bfloat16, torch.float32)]
+        for r in flash:
+            log("prefill attention", json.dumps(r))
+        extras["prefill_attention"] = flash
     if not args.no_extras and not args.decode:
         # config 4 end to end, short form: the 12-layer W4A16 model, prompt 512 + 256 greedy tokens,
         # batch 1 and 8, decode step replayed from a HIP graph (tokens/s is the third headline metric)
