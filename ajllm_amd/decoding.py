@@ -75,11 +75,36 @@ class GraphDecoder:
         self.produced = 1
         self.prompt_len = prompt.shape[1]
 
+    def _all_rows_done(self, eos_token_id: int) -> int | None:
+        """Number of tokens after which every row has produced ``eos_token_id`` (None: not yet)."""
+        seen = (self.out[:, : self.produced] == eos_token_id)
+        if not bool(seen.any(dim=1).all()):
+            return None
+        first = seen.int().argmax(dim=1)  # index of each row's first eos
+        return int(first.max()) + 1
+
     @torch.no_grad()
-    def generate(self, new_tokens: int) -> torch.Tensor:
-        """Decode until ``new_tokens`` tokens exist since ``prefill`` and return them ``[B, new_tokens]``."""
+    def generate(self, new_tokens: int, eos_token_id: int | None = None, eos_check_every: int = 16) -> torch.Tensor:
+        """Decode until ``new_tokens`` tokens exist since ``prefill`` and return them ``[B, new_tokens]``.
+
+        With ``eos_token_id`` decoding stops once every row has produced it, as the reference's
+        ``generate`` does for its one row (src/ajllm/generation/generator.py:26-27) and
+        ``modeling.greedy_decode`` for a batch: the returned tensor ends with the step at which the
+        last row produced it.  The host looks at the tokens every ``eos_check_every`` steps only (a
+        look is a synchronisation); steps replayed past the stopping point are cut off the result."""
         if self.prompt_len + new_tokens > self.max_len:
             raise ValueError("the KV cache is too short for this many tokens")
+        if eos_token_id is not None:
+            if eos_check_every < 1:
+                raise ValueError("eos_check_every must be positive")
+            target = self.produced
+            while True:
+                done_at = self._all_rows_done(eos_token_id)
+                if done_at is not None or target >= new_tokens:
+                    break
+                target = min(new_tokens, target + eos_check_every)
+                self.generate(target)
+            return self.out[:, : (done_at if done_at is not None else new_tokens)].clone()
         current = torch.cuda.current_stream(self.device)
         self.stream.wait_stream(current)
         with torch.cuda.stream(self.stream):

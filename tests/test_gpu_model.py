@@ -272,6 +272,36 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
     assert rel <= 1e-3, (max_abs, rel)
 
 
+@pytest.mark.parametrize("batch", [1, 3])
+def test_graph_decoders_stop_at_eos(cuda, batch):
+    """generate(eos_token_id=...): the result is the plain run cut after the step at which the last
+    row has produced the token (generator.py:26-27 for one row; every row, as modeling.greedy_decode),
+    whatever the spacing of the host's looks."""
+    torch.manual_seed(4)
+    model = modeling.TransformerLM(vocab_size=512, context_length=96, d_model=256, num_layers=2, num_heads=2,
+                                   d_ff=640, num_kv_heads=2).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w8a16")
+    prompt = torch.randint(0, 512, (batch, 12), generator=torch.Generator().manual_seed(3)).to(cuda)
+    for cls in (decoding.GraphDecoder, decoding.FusedDecoder):
+        dec = cls(fast, batch, 60)
+        dec.prefill(prompt)
+        full = dec.generate(40).cpu()
+        # a token every row produces if there is one (else row 0's sixth: the run then goes to the end)
+        common = set(full[0].tolist())
+        for row in full[1:]:
+            common &= set(row.tolist())
+        eos = min(common) if common else int(full[0, 5])
+        seen = full == eos
+        stop = int(seen.int().argmax(dim=1).max()) + 1 if bool(seen.any(dim=1).all()) else 40
+        for every in (1, 7, 16):
+            dec = cls(fast, batch, 60)
+            dec.prefill(prompt)
+            got = dec.generate(40, eos_token_id=eos, eos_check_every=every).cpu()
+            assert got.shape[1] == stop and torch.equal(got, full[:, :stop]), (cls.__name__, every, stop, got.shape)
+    if batch == 1:
+        assert stop < 40  # (one row always has a common token: the stop is exercised)
+
+
 @pytest.mark.parametrize("b,heads,kv_heads,t,start,cache_dtype", [
     (2, 4, 2, 100, 0, torch.float32), (1, 2, 2, 64, 0, torch.float32), (1, 4, 1, 130, 37, torch.float32),
     (3, 2, 1, 257, 5, torch.bfloat16), (1, 1, 1, 1, 9, torch.float32), (1, 8, 2, 512, 0, torch.bfloat16),
