@@ -73,9 +73,11 @@ def quantization_report(model: torch.nn.Module, dataset, scheme: str, batches: i
                         context_length: int, device, seed: int, skip: tuple[str, ...] = ()) -> dict[str, object]:
     """Score ``model`` and a quantized copy of it on the same windows.
 
-    The copy is made on the host, moved to ``device`` and quantized there, so the caller's model is
-    left as it was.  ``loss_delta`` is quantized minus dense."""
-    dense = evaluate_model(model.to(device), dataset, batches, batch_size, context_length, device, seed)
+    Both scores come from copies moved to ``device`` (the quantized one is quantized there): the
+    caller's model stays where and as it was.  ``loss_delta`` is quantized minus dense."""
+    dense_copy = copy.deepcopy(model).to(device)
+    dense = evaluate_model(dense_copy, dataset, batches, batch_size, context_length, device, seed)
+    del dense_copy
     twin = copy.deepcopy(model).to(device)
     quantize_model_(twin, scheme=scheme, skip=skip)
     quant = evaluate_model(twin, dataset, batches, batch_size, context_length, device, seed)
