@@ -321,6 +321,9 @@ def main() -> int:
                     help="also time the alternatives to one launch per matrix for a chain of GEMVs (bench-only probes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="timed region only")
+    ap.add_argument("--no-decode", action="store_true",
+                    help="skip the short end-to-end decode leg of the default line (counter-collection runs: "
+                         "the profiler does not survive the leg's graph replays)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on exactly one GPU (the quantized linear is a single-GPU "
@@ -366,7 +369,7 @@ def main() -> int:
         for r in flash:
             log("prefill attention", json.dumps(r))
         extras["prefill_attention"] = flash
-    if not args.no_extras and not args.decode:
+    if not args.no_extras and not args.decode and not args.no_decode:
         # config 4 end to end, short form: the 12-layer W4A16 model, prompt 512 + 256 greedy tokens,
         # batch 1 and 8, decode step replayed from a HIP graph (tokens/s is the third headline metric)
         from ajllm_amd.e2e_bench import bench_decode_short
