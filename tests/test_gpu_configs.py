@@ -12,10 +12,10 @@ oracle's own top-1 minus top-2 logit is below the measured logit error of the tw
 Teacher-forced: the decode kernels fed the oracle's tokens, so that every one of the 256 steps is
 compared on the same context; a differing choice is again accepted only below the measured error.
 The numbers (identical-prefix lengths, agreement rate, margins, logit error) go to
-``gpurun_out/config4_tokens_b<batch>.json``.
+``config4_tokens_b<batch>.json`` in the output directory ``OUT_DIR``.
 
 The oracle side takes a minute or two of CPU work per case; a heartbeat line is appended to
-``gpurun_out/config_tests_progress.log`` while it runs.
+``config_tests_progress.log`` in the same directory while it runs.
 """
 
 import copy
