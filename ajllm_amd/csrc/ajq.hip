@@ -9,6 +9,7 @@
 #include "gemv_kernels.h"
 #include "gemv_fused_kernels.h"
 #include "gemm_kernels.h"
+#include "gemm_ring_kernels.h"
 #include "gemm128_kernels.h"
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
@@ -112,9 +113,20 @@ int check_matmul_args(const char* name, const void* x, int M, int K, const void*
 template <int MT, bool kW4, bool kGate = false>
 int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                    const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
+  const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
+#ifndef AJQ_G2_RING
+#define AJQ_G2_RING 1
+#endif
+  if (AJQ_G2_RING && !kW4 && K % 256 == 0) {
+    // W8: the same tiles with the operands in a ring of four 64-k stages, loaded by a wave of its own
+    auto ring = dequant_gemm256r_w8_kernel<kGate>;
+    if (int s = allow_big_lds(ring, kGRLdsBytes)) return s;
+    hipLaunchKernelGGL(ring, dim3(tiles), dim3(kGRThreads), kGRLdsBytes, stream, x, M, K,
+                       reinterpret_cast<const u32x4_t*>(wq), scales8, N, y, out_f32);
+    return AJQ_OK;
+  }
   auto kernel = dequant_gemm256_kernel<MT, kW4, kGate>;
   if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
-  const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
   hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,
                      reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
                      reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);

@@ -129,6 +129,94 @@ constexpr int kG2W8Base = 2 * kG2TileBytes;
 constexpr int kG2WStride = 16384, kG2MetaStride = 512;
 constexpr size_t kG2LdsBytes = 160 * 1024;
 
+// Epilogue of the 256 x 128 tile kernels.  Accumulator register r of lane (col, kh) is row
+// (r & 3) + 8 * (r >> 2) + 4 * kh of its 32 x 32 block.  bf16 output: the tile is laid out row-major
+// in LDS (from address 0: the caller guarantees that every wave is done with the tile buffers and that
+// no request into them is in flight) and leaves in whole 256-byte rows, four rows per wave-wide
+// 128-bit store; 2-byte stores straight from the accumulators took 2-3 times as long.
+template <int MT, bool kW4, bool kGate>
+__device__ __forceinline__ void gemm256_store(f32x16_t (&acc)[MT][2], char* lds, void* __restrict__ y, int out_f32, int N,
+                                              int m0, int n0, const uint16_t* __restrict__ scales8, int lane, int wave,
+                                              int wm, int wn, int col, int kh) {
+  constexpr int kWaves = 16 / MT;
+  constexpr int kWaveRows = 32 * MT;
+  constexpr int kLoadRows = kG2BM / kWaves;
+  // Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart) use different banks.
+  constexpr int kOutStride = 272;
+  // column of the weight tensor behind the wave's 32-column block t
+  auto column = [&](int t) -> int {
+    if (kGate) return t * (N >> 1) + n0 + wn * 32 + col;
+    return n0 + wn * 64 + t * 32 + col;
+  };
+  float cs[2] = {1.0f, 1.0f};
+  if (!kW4) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(column(t), N - 1)]);
+  }
+  if (kGate) {
+    // block 0 holds the gate projection a, block 1 the up projection u of the same columns:
+    // out = bf16( a * sigmoid(a) * u ), [M, N / 2], staged like the plain bf16 tile (64 columns:
+    // 128-byte rows 144 bytes apart) and stored eight rows per wave-wide 128-bit store
+    constexpr int kGateStride = 144;
+    const int F = N >> 1;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        const float a = acc[i][0][r] * cs[0], u = acc[i][1][r] * cs[1];
+        *reinterpret_cast<uint16_t*>(lds + row * kGateStride + (wn * 32 + col) * 2) =
+            f32_to_bf16_rne(a * (1.0f / (1.0f + expf(-a))) * u);
+      }
+    __syncthreads();
+    const int piece = lane & 7, rsub = lane >> 3;
+#pragma unroll
+    for (int j = 0; j < kLoadRows / 8; ++j) {
+      const int row = wave * kLoadRows + j * 8 + rsub;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kGateStride + piece * 16);
+      *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * F + n0 + piece * 8) = v;
+    }
+    return;
+  }
+  if (!out_f32) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+          *reinterpret_cast<uint16_t*>(lds + row * kOutStride + (wn * 64 + t * 32 + col) * 2) =
+              f32_to_bf16_rne(acc[i][t][r] * cs[t]);
+        }
+    __syncthreads();
+    // lane -> (row within a group of 4, 16-byte piece of the 256-byte row); columns past N are dropped
+    const int piece = lane & 15, rsub = lane >> 4;
+    const bool live = n0 + piece * 8 < N;
+#pragma unroll
+    for (int j = 0; j < kLoadRows / 4; ++j) {
+      const int row = wave * kLoadRows + j * 4 + rsub;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kOutStride + piece * 16);
+      if (live)
+        *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * N + n0 + piece * 8) = v;
+    }
+    return;
+  }
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int n = column(t);
+    if (n >= N) continue;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
+        reinterpret_cast<float*>(y)[(size_t)m * N + n] = acc[i][t][r] * cs[t];
+      }
+    }
+  }
+}
+
 // MT = 32-row blocks per wave: 4 -> 4 waves (2 x 2, wave tile 128 x 64), 2 -> 8 waves
 // (4 x 2, wave tile 64 x 64, two waves per SIMD).
 // kGate: the weights are the w1 | w3 rows of a SwiGLU feed-forward (N = 2 F, F % 64 == 0).  A
@@ -357,84 +445,7 @@ __global__ __launch_bounds__(1024 / MT) void dequant_gemm256_kernel(
     __syncthreads();
   }
 
-  // ---- epilogue: accumulator register r of lane (col, kh) is row (r & 3) + 8 * (r >> 2) + 4 * kh.
-  // bf16 output: the tile is laid out row-major in LDS (the activation buffers are free: every
-  // wave has passed the loop's last barrier) and leaves in whole 256-byte rows, four rows per
-  // wave-wide 128-bit store; 2-byte stores straight from the accumulators took 2-3 times as long.
-  // Rows are 272 bytes apart so the two half-waves of a write (rows 4 apart) use different banks.
-  constexpr int kOutStride = 272;
-  // column of the weight tensor behind the wave's 32-column block t
-  auto column = [&](int t) -> int {
-    if (kGate) return t * (N >> 1) + n0 + wn * 32 + col;
-    return n0 + wn * 64 + t * 32 + col;
-  };
-  float cs[2] = {1.0f, 1.0f};
-  if (!kW4) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(column(t), N - 1)]);
-  }
-  if (kGate) {
-    // block 0 holds the gate projection a, block 1 the up projection u of the same columns:
-    // out = bf16( a * sigmoid(a) * u ), [M, N / 2], staged like the plain bf16 tile (64 columns:
-    // 128-byte rows 144 bytes apart) and stored eight rows per wave-wide 128-bit store
-    constexpr int kGateStride = 144;
-    const int F = N >> 1;
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-        const float a = acc[i][0][r] * cs[0], u = acc[i][1][r] * cs[1];
-        *reinterpret_cast<uint16_t*>(lds + row * kGateStride + (wn * 32 + col) * 2) =
-            f32_to_bf16_rne(a * (1.0f / (1.0f + expf(-a))) * u);
-      }
-    __syncthreads();
-    const int piece = lane & 7, rsub = lane >> 3;
-#pragma unroll
-    for (int j = 0; j < kLoadRows / 8; ++j) {
-      const int row = wave * kLoadRows + j * 8 + rsub;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kGateStride + piece * 16);
-      *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * F + n0 + piece * 8) = v;
-    }
-    return;
-  }
-  if (!out_f32) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-          *reinterpret_cast<uint16_t*>(lds + row * kOutStride + (wn * 64 + t * 32 + col) * 2) =
-              f32_to_bf16_rne(acc[i][t][r] * cs[t]);
-        }
-    __syncthreads();
-    // lane -> (row within a group of 4, 16-byte piece of the 256-byte row); columns past N are dropped
-    const int piece = lane & 15, rsub = lane >> 4;
-    const bool live = n0 + piece * 8 < N;
-#pragma unroll
-    for (int j = 0; j < kLoadRows / 4; ++j) {
-      const int row = wave * kLoadRows + j * 4 + rsub;
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kOutStride + piece * 16);
-      if (live)
-        *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * N + n0 + piece * 8) = v;
-    }
-    return;
-  }
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int n = column(t);
-    if (n >= N) continue;
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * kWaveRows + i * 32 + (r & 3) + 8 * (r >> 2) + 4 * kh;
-        reinterpret_cast<float*>(y)[(size_t)m * N + n] = acc[i][t][r] * cs[t];
-      }
-    }
-  }
+  gemm256_store<MT, kW4, kGate>(acc, lds, y, out_f32, N, m0, n0, scales8, lane, wave, wm, wn, col, kh);
 }
 
 }  // namespace ajq
