@@ -125,6 +125,16 @@ int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                        reinterpret_cast<const u32x4_t*>(wq), scales8, N, y, out_f32);
     return AJQ_OK;
   }
+#ifndef AJQ_G2_RING4
+#define AJQ_G2_RING4 1
+#endif
+  if (AJQ_G2_RING4 && kW4 && K % 256 == 0) {
+    auto ring = dequant_gemm256r_w4_kernel<kGate>;
+    if (int s = allow_big_lds(ring, kGR4LdsBytes)) return s;
+    hipLaunchKernelGGL(ring, dim3(tiles), dim3(kGRThreads), kGR4LdsBytes, stream, x, M, K,
+                       reinterpret_cast<const u32x4_t*>(wq), meta, reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
+    return AJQ_OK;
+  }
   auto kernel = dequant_gemm256_kernel<MT, kW4, kGate>;
   if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
   hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,

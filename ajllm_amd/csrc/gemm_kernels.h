@@ -137,7 +137,8 @@ constexpr size_t kG2LdsBytes = 160 * 1024;
 template <int MT, bool kW4, bool kGate>
 __device__ __forceinline__ void gemm256_store(f32x16_t (&acc)[MT][2], char* lds, void* __restrict__ y, int out_f32, int N,
                                               int m0, int n0, const uint16_t* __restrict__ scales8, int lane, int wave,
-                                              int wm, int wn, int col, int kh) {
+                                              int wm, int wn, int col, int kh, float unit0 = 1.0f,
+                                              float unit1 = 1.0f) {
   constexpr int kWaves = 16 / MT;
   constexpr int kWaveRows = 32 * MT;
   constexpr int kLoadRows = kG2BM / kWaves;
@@ -148,7 +149,7 @@ __device__ __forceinline__ void gemm256_store(f32x16_t (&acc)[MT][2], char* lds,
     if (kGate) return t * (N >> 1) + n0 + wn * 32 + col;
     return n0 + wn * 64 + t * 32 + col;
   };
-  float cs[2] = {1.0f, 1.0f};
+  float cs[2] = {unit0, unit1};  // W4: what the caller's accumulators are in units of (1 if already scaled)
   if (!kW4) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) cs[t] = f16_bits_to_f32(scales8[min(column(t), N - 1)]);
