@@ -155,6 +155,46 @@ def test_prefill_gemm_m8192(cuda, scheme, n):
     _check(scheme, "gemm", 8192, n, 4096, seed=32, cuda=cuda, outliers=True, max_rows=128)
 
 
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 512), (2048, 4096, 1280), (300, 512, 1024), (40, 512, 1024), (4, 512, 1024)])
+def test_w4_group_scales_far_apart_and_zero(cuda, m, n, k):
+    """W4 columns whose group scales differ by six orders of magnitude from one group to the next, with
+    constant-zero groups (scale 0) and constant non-zero groups (scale 0 too: they dequantize to 0) in
+    between, first and last.  The tile kernels carry their accumulators in units of the current group's
+    scale, so a wrong rescale at a group boundary, or a zero scale, shows as an O(1) error here.  Shapes:
+    256 x 128 tiles on the four-stage ring (K % 256 == 0), the same tiles double-buffered (K = 1280),
+    128 x 128 tiles, the weight-streaming kernel and the GEMV."""
+    from ajllm_amd import repack_w4, w4a16_matmul
+
+    gen = torch.Generator().manual_seed(m + n + k)
+    groups = k // 128
+    magnitude = torch.tensor([1e-3, 1.0, 0.0, 30.0, 1e-4, 3.0, 0.0, 0.0, 1e2, 1e-2])[
+        torch.randint(0, 10, (n, groups), generator=gen)
+    ]
+    magnitude[:, 0] = torch.where(torch.arange(n) % 3 == 0, 0.0, magnitude[:, 0])     # zero scale first
+    magnitude[:, -1] = torch.where(torch.arange(n) % 5 == 0, 0.0, magnitude[:, -1])   # and last
+    w = (torch.randn(n, groups, 128, generator=gen) * magnitude[:, :, None]).reshape(n, k)
+    w[7::11, 128:256] = 0.5  # constant non-zero groups
+    q, s, z = qspec.quantize_w4_g128(w.numpy())
+    assert (s == 0).any() and (s > 1).any()
+    qw = qspec.pack_int4(q)
+    w_hat = torch.from_numpy(qspec.dequantize_w4(qw, s, z))
+    wq, meta = repack_w4(torch.from_numpy(qw).to(cuda), torch.from_numpy(s).to(cuda), torch.from_numpy(z).to(cuda))
+    x = make_activations(m, k, 77, True)
+    y = w4a16_matmul(x.to(cuda), wq, meta, torch.float32).cpu()
+    rows = torch.arange(0, m, max(1, m // 128))
+    want = qspec.quant_linear(x[rows], w_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    assert torch.isfinite(y).all()
+    rel = float((y[rows].double() - want).norm() / want.norm())
+    assert rel <= 1e-5, rel
+    # columns are independent: a column's error is judged against that column's own magnitude
+    col_err = (y[rows].double() - want).norm(dim=0)
+    col_ref = want.norm(dim=0)
+    live = col_ref > 0
+    assert float((col_err[live] / col_ref[live]).max()) <= 1e-4
+    if (~live).any():
+        assert float(col_err[~live].max()) <= 1e-10
+
+
 @pytest.mark.parametrize("m", [1, 17, 63, 65, 100, 129, 300])
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemm_ragged_m(cuda, scheme, m):
