@@ -87,6 +87,15 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
          c_void_p],
     ),
+    "ajq_gemv_epilogue_supported": (c_int, [c_int, c_int]),
+    "ajq_w4a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p]),
+    "ajq_w8a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_void_p]),
+    "ajq_w4a16_gemv_rowscale": (c_int, [c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_int, c_int, c_void_p]),
+    "ajq_w8a16_gemv_rowscale": (c_int, [c_void_p, c_void_p, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_int,
+                                        c_void_p, c_int, c_int, c_void_p]),
     "ajq_w4a16_gemv_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_w8a16_gemv_gate": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_attn_step_workspace_bytes": (c_size_t, [c_int, c_int]),

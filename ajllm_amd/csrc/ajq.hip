@@ -403,6 +403,92 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
   return launch_skinny_cfg<8, 1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
+// ---- GEMV with work around the matmul for batched decode steps (row scale of a norm on the way out,
+// residual add with the next norm's preparation, SwiGLU gate): straight-line configurations only,
+// row bound 8 or 16
+template <int kWaves, int TPW, int MROWS, bool kW4, int kEpi>
+int launch_gemv_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                        int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  constexpr size_t lds = gemv_epi_lds_bytes(kWaves, TPW, MROWS);
+  static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
+  auto kernel = dequant_gemv_epi_kernel<kWaves, TPW, MROWS, kW4, true, kEpi>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
+                     meta, x, K, M | (out_f32 << 8), N, y, scales8, ep);
+  return AJQ_OK;
+}
+
+bool gemv_epi_supported(int M, int K) {
+  if (M < 1 || M > kMaxGemvM) return false;
+  if (K == 2048 || K == 4096) return true;
+  return K == 5632 && M <= 8;
+}
+
+template <bool kW4, int kEpi>
+int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                    int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+#define AJQ_EPI(W, T, R) return launch_gemv_epi_cfg<W, T, R, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
+  if (K == 2048) {
+    if (M <= 8) AJQ_EPI(8, 2, 8);
+    AJQ_EPI(8, 2, 16);
+  }
+  if (K == 4096) {
+    if (M <= 8) AJQ_EPI(8, 4, 8);
+    AJQ_EPI(8, 4, 16);
+  }
+  AJQ_EPI(11, 4, 8);
+#undef AJQ_EPI
+}
+
+int check_epi(const char* name, int M, int K) {
+  if (!gemv_epi_supported(M, K))
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d is not built (ajq_gemv_epilogue_supported)", name, M, K);
+  return AJQ_OK;
+}
+
+template <bool kW4>
+int gemv_rowscale(const char* name, const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
+                         const uint32_t* wq, const void* aux, int N, void* y, int out_dtype, int gate, void* stream) {
+  if (int s = check_matmul_args(name, xt, M, K, wq, aux, N, y, out_dtype, kGroup)) return s;
+  if (int s = check_epi(name, M, K)) return s;
+  if (!ssq || !aligned16(ssq)) return fail(ssq ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq must be non-null and 16-byte aligned", name);
+  const int waves = K == 5632 ? 11 : 8;
+  if (parts < 4 || parts % 4 != 0 || parts > waves * 32)
+    return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, %d]", name, parts, waves * 32);
+  if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);
+  GemvEpilogue ep{};
+  ep.ssq_in = ssq;
+  ep.parts = parts;
+  ep.inv_k = 1.0f / (float)K;
+  ep.eps = eps;
+  const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
+  const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
+  const int s = gate ? launch_gemv_epi<kW4, kEpiRowScale | kEpiGate>(xt, M, K, wq, meta, scales, N, y, 0, ep, (hipStream_t)stream)
+                     : launch_gemv_epi<kW4, kEpiRowScale>(xt, M, K, wq, meta, scales, N, y, out_dtype == AJQ_OUT_F32, ep,
+                                                          (hipStream_t)stream);
+  if (s) return s;
+  return check_launch(name);
+}
+
+template <bool kW4>
+int gemv_residual(const char* name, const uint16_t* x, int M, int K, const uint32_t* wq, const void* aux, int N,
+                         const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out, void* stream) {
+  if (int s = check_matmul_args(name, x, M, K, wq, aux, N, h_out, AJQ_OUT_F32, kGroup)) return s;
+  if (int s = check_epi(name, M, K)) return s;
+  if (!h_in || !gain || !xt_out || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (h_in == h_out) return fail(AJQ_ERR_NULL, "%s: h_out must be a buffer other than h_in", name);
+  GemvEpilogue ep{};
+  ep.h_in = h_in;
+  ep.gain = gain;
+  ep.h_out = h_out;
+  ep.xt = xt_out;
+  ep.ssq_out = ssq_out;
+  const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
+  const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
+  if (int s = launch_gemv_epi<kW4, kEpiResidual>(x, M, K, wq, meta, scales, N, nullptr, 1, ep, (hipStream_t)stream)) return s;
+  return check_launch(name);
+}
+
 // ---- GEMV with the activations produced on the way in (norm / gate prologue)
 template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
 int launch_gemv_pro_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
@@ -542,6 +628,30 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 }
 
 int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1 : 0; }
+
+int ajq_gemv_epilogue_supported(int M, int K) { return gemv_epi_supported(M, K) ? 1 : 0; }
+
+int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K, const uint32_t* wq,
+                            const uint32_t* meta, int N, void* y, int out_dtype, int gate, void* stream) {
+  return gemv_rowscale<true>("ajq_w4a16_gemv_rowscale", xt, ssq, parts, eps, M, K, wq, meta, N, y, out_dtype, gate, stream);
+}
+
+int ajq_w8a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K, const uint32_t* wq,
+                            const uint16_t* scales, int N, void* y, int out_dtype, int gate, void* stream) {
+  return gemv_rowscale<false>("ajq_w8a16_gemv_rowscale", xt, ssq, parts, eps, M, K, wq, scales, N, y, out_dtype, gate, stream);
+}
+
+int ajq_w4a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                            const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                            void* stream) {
+  return gemv_residual<true>("ajq_w4a16_gemv_residual", x, M, K, wq, meta, N, h_in, gain, h_out, xt_out, ssq_out, stream);
+}
+
+int ajq_w8a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                            const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                            void* stream) {
+  return gemv_residual<false>("ajq_w8a16_gemv_residual", x, M, K, wq, scales, N, h_in, gain, h_out, xt_out, ssq_out, stream);
+}
 
 int ajq_w4a16_gemv_norm(const float* h_in, const float* delta, const float* gain, float eps, float* h_out, int M, int K,
                         const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, void* stream) {

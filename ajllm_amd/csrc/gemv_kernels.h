@@ -41,14 +41,39 @@ struct GemvBatch {
 // MROWS >= M is the compile-time row bound that sizes the activation slice.
 // kSingle: K == kWaves * TPW * 128, every wave has exactly one full batch (no
 // loop, no clamped addresses, no tail tests).
-template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
-__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
+//
+// kEpi adds work around the matmul for batched decode steps, where a launch of its own for the
+// residual add, the RMSNorm or the SwiGLU gate costs more than the operation (bits may be combined):
+//  * kEpiRowScale: the activations are x~ = bf16((h) * gain), NOT yet normalised, and every output row is
+//    multiplied by rstd[m] = rsqrt(sum_k h[m][k]^2 / K + eps): the row scale of an RMSNorm commutes with
+//    the matmul.  The sum of squares arrives as `parts` partial sums per row (ssq_in[16][parts], written
+//    by the producing kernel's workgroups); every wave adds a fixed share of them while its weights
+//    travel and wave 0 adds the waves' shares in wave order: no atomics, run-to-run identical.
+//  * kEpiResidual: h_out = h_in + (x W^T) instead of y, together with x~ = bf16(h_out * gain) for the
+//    norm that follows and the workgroup's partial sum of squares of its 16 columns, ssq_out[m][tile].
+//  * kEpiGate: the 16 rows of a weight tile are 8 rows of the gate projection followed by the 8
+//    matching rows of the up projection; y[m][8 tile + j] = bf16(silu(a_j) * u_j), [M, N / 2].
+constexpr int kEpiRowScale = 1, kEpiResidual = 2, kEpiGate = 4;
+struct GemvEpilogue {
+  const float* ssq_in;  // row scale: [16][parts]
+  int parts;            //   partial sums per row, a multiple of 4, at most kWaves * 32
+  float inv_k, eps;     //   1 / K of the norm, its epsilon
+  const float* h_in;    // residual: [M, N]
+  const float* gain;    // residual: [N], gain of the norm that follows
+  float* h_out;         // residual: [M, N], must not alias h_in
+  uint16_t* xt;         // residual: bf16 [M, N]
+  float* ssq_out;       // residual: [16][N / 16]
+};
+
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi>
+__device__ __forceinline__ void dequant_gemv_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K,
     int m_flags,  // M | out_f32 << 8 (one word: the leading arguments arrive preloaded in SGPRs)
     int N, void* __restrict__ y,
-    const uint16_t* __restrict__ scales8) {  // W8: fp16 [N]; W4: unused
+    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
+    const GemvEpilogue& ep) {
   const int M = m_flags & 0xFF;
   const bool out_f32 = (m_flags >> 8) != 0;
   constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
@@ -169,13 +194,41 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   };
 
   // two register sets, ping-pong: the next batch is in flight while one is computed
+  // ---- what the epilogue variants need from memory is requested behind the first batch of weights
+  // (vector loads return in issue order: in front of them it would delay the HBM requests) and used at
+  // the end
+  constexpr int kLiveRows = MROWS < 4 ? MROWS : 4;
+  float* red2 = red + kWaves * 64 * 4;  // [16][kWaves] shares of the rows' sums of squares
+  float4 ssq_share[2];
+  float h_old[kLiveRows], gain_n = 0.f;
+  auto epilogue_loads = [&]() {
+    if (kEpi & kEpiRowScale) {
+      const int m = lane & 15, c = lane >> 4;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int j = wave * 4 + c + u * kWaves * 4;  // float4 index inside the row
+        const bool live = 4 * j < ep.parts;
+        const float4 t = *reinterpret_cast<const float4*>(ep.ssq_in + (size_t)m * ep.parts + (live ? 4 * j : 0));
+        ssq_share[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    if (kEpi & kEpiResidual) {
+      const int n = nt * kTileN + nl;
+      gain_n = ep.gain[n];
+#pragma unroll
+      for (int i = 0; i < kLiveRows; ++i) h_old[i] = ep.h_in[(size_t)min(4 * kc + i, M - 1) * N + n];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
   if (kSingle) {
     Batch b0;
     load(b0, g_begin);
+    epilogue_loads();
     compute(b0, g_begin);
   } else if (g_begin < g_end) {
     Batch b0, b1;
     load(b0, g_begin);
+    epilogue_loads();
     for (int g0 = g_begin; g0 < g_end; g0 += 2 * TPW) {
       const bool has1 = g0 + TPW < g_end;
       if (has1) load(b1, g0 + TPW);
@@ -197,6 +250,14 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
 #pragma unroll
   for (int i = 0; i < kLive; ++i) mine[i] = acc[i];
   if (kc < kRowQuads) redv[wave * (16 * kRowQuads) + lane] = mine;
+  if (kEpi & kEpiRowScale) {
+    // this wave's share of the rows' sums of squares: lane (row m = lane & 15, quarter c) holds 8 parts
+    float sh = ((ssq_share[0].x + ssq_share[0].y) + (ssq_share[0].z + ssq_share[0].w)) +
+               ((ssq_share[1].x + ssq_share[1].y) + (ssq_share[1].z + ssq_share[1].w));
+    sh += __shfl_xor(sh, 16);
+    sh += __shfl_xor(sh, 32);
+    if (kc == 0) red2[nl * kWaves + wave] = sh;
+  }
   __syncthreads();
   if (wave != 0 || kc >= kRowQuads) return;
   live_t part[kWaves];
@@ -208,17 +269,76 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
   const int n = nt * kTileN + nl;
   float cs = 1.0f;
   if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
+  float rstd[kLive];
+#pragma unroll
+  for (int i = 0; i < kLive; ++i) {
+    rstd[i] = 1.0f;
+    if (kEpi & kEpiRowScale) {
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) total += red2[min(4 * kc + i, 15) * kWaves + w];
+      rstd[i] = rsqrtf(total * ep.inv_k + ep.eps);
+    }
+  }
+  if (kEpi & kEpiResidual) {
+    // the updated residual stream, its bf16 image for the next matmul, and this tile's sums of squares
+    const int ntiles = N / kTileN;
+#pragma unroll
+    for (int i = 0; i < kLive; ++i) {
+      const int m = 4 * kc + i;
+      const float h = h_old[i] + sum[i] * cs * rstd[i];
+      if (m < M) {
+        ep.h_out[(size_t)m * N + n] = h;
+        ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+      }
+      float sq = m < M ? h * h : 0.f;
+      sq += __shfl_xor(sq, 1);
+      sq += __shfl_xor(sq, 2);
+      sq += __shfl_xor(sq, 4);
+      sq += __shfl_xor(sq, 8);
+      if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt] = sq;
+    }
+    return;
+  }
+  if (kEpi & kEpiGate) {
+    // columns 0..7 of the tile are gate projections, 8..15 the matching up projections
+#pragma unroll
+    for (int i = 0; i < kLive; ++i) {
+      const int m = 4 * kc + i;
+      const float v = sum[i] * cs * rstd[i];
+      const float other = __shfl_xor(v, 8);
+      if (nl < 8 && m < M)
+        reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + nt * 8 + nl] =
+            f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < kLive; ++i) {
     const int m = 4 * kc + i;
     if (m < M) {
-      const float v = sum[i] * cs;
+      const float v = sum[i] * cs * rstd[i];
       if (out_f32)
         reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
       else
         reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
     }
   }
+}
+
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
+__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K,
+    int m_flags, int N, void* __restrict__ y, const uint16_t* __restrict__ scales8) {
+  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, 0>(wq, meta, x, K, m_flags, N, y, scales8, GemvEpilogue{});
+}
+
+// the same kernel with work around the matmul (see kEpi above)
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi>
+__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_epi_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K,
+    int m_flags, int N, void* __restrict__ y, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
+  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, kEpi>(wq, meta, x, K, m_flags, N, y, scales8, ep);
 }
 
 // ---------------------------------------------------------------------------
@@ -400,6 +520,10 @@ constexpr size_t gemv_mt_lds_bytes(int waves, int tpw, int mrows) {
 // LDS bytes of one workgroup of dequant_gemv_kernel<kWaves, TPW, MROWS, *>
 constexpr size_t gemv_lds_bytes(int waves, int tpw, int mrows) {
   return (size_t)waves * mrows * (tpw * kGroup + 8) * 2 + (size_t)waves * 64 * 16;
+}
+// ... of dequant_gemv_epi_kernel: the rows' sums of squares, one share per wave, behind the rest
+constexpr size_t gemv_epi_lds_bytes(int waves, int tpw, int mrows) {
+  return gemv_lds_bytes(waves, tpw, mrows) + (size_t)16 * waves * 4;
 }
 
 }  // namespace ajq

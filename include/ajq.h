@@ -130,6 +130,37 @@ int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
                         void* y, int out_dtype, void* stream);
 int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                         void* y, int out_dtype, void* stream);
+/* The same GEMV with work around the matmul, for decode steps of several rows, where a launch of its own
+ * for the residual add, the RMSNorm or the SwiGLU gate costs more than the operation itself
+ * (TransformerBlock.forward, src/ajllm/modeling/transformer.py:45-50; RMSNorm, layers.py:70-74; SwiGLU,
+ * activations.py:24-25).  The row scale of an RMSNorm commutes with the matmul, so the pair below computes
+ *     h_out = h_in + x W1^T ;   y = (RMSNorm(h_out) * gain) W2^T
+ * in two launches, without a norm kernel between them:
+ *   _residual: h_out[M, N] = h_in + x W^T (fp32; h_out must not be h_in), xt_out = bf16(h_out * gain)
+ *              (gain[N]: of the norm that follows) and ssq_out[16][N / 16]: per row, the sum of squares of
+ *              h_out over each 16-column tile (rows >= M are not written);
+ *   _rowscale: y = rstd[m] * (xt W^T) with rstd[m] = rsqrt(sum(ssq[m][0 .. parts)) / K + eps), ssq laid out
+ *              [16][parts] as _residual leaves it (parts = K / 16; a multiple of 4, at most 256, 352 for
+ *              K = 5632).  gate != 0: the rows of W are tiles of 8 gate-projection rows followed by the 8
+ *              matching up-projection rows (w1 and w3 interleaved in blocks of 8) and
+ *              y[M, N / 2] = bf16(silu(a) * u), out_dtype AJQ_OUT_BF16.
+ * xt is rounded to bf16 BEFORE the row scale is applied (the reference order rounds the normalised value);
+ * both are one bf16 rounding of the same quantity up to the fp32 factor rstd.  Sums run in a fixed order:
+ * results are run-to-run identical.  Built for the (M, K) that ajq_gemv_epilogue_supported reports: M <= 16
+ * with K = 2048 or 4096, M <= 8 with K = 5632; AJQ_ERR_UNSUPPORTED otherwise. */
+int ajq_gemv_epilogue_supported(int M, int K);
+int ajq_w4a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                            const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                            void* stream);
+int ajq_w8a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
+                            const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                            void* stream);
+int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
+                            const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, int gate,
+                            void* stream);
+int ajq_w8a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
+                            const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
+                            void* stream);
 /*   _merge: x = bf16 of the single-query attention output [M, K] (K = heads * 128), merged from the S
  *          partial results per (row, head) that ajq_attn_step_partial left in its workspace -- the
  *          softmax-weighted value sum of scaled_dot_product_attention (src/ajllm/modeling/attention.py:20-33)

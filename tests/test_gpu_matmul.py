@@ -374,6 +374,81 @@ def test_gemv_with_norm_or_gate_prologue_against_the_oracle(cuda, scheme, m, k):
     assert max_abs <= MAX_ABS_TOL and rel <= REL_FRO_TOL, (max_abs, rel)
 
 
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+@pytest.mark.parametrize("m,k1,d,n2", [(8, 2048, 2048, 6144), (5, 5632, 2048, 11264), (16, 2048, 2048, 512),
+                                      (8, 4096, 4096, 1024), (13, 4096, 4096, 2048), (1, 2048, 2048, 256)])
+def test_gemv_residual_then_rowscale_against_the_oracle(cuda, scheme, m, k1, d, n2):
+    """h_out = h_in + x W1^T (ajq_w*a16_gemv_residual) followed by y = (RMSNorm(h_out) * gain) W2^T
+    (ajq_w*a16_gemv_rowscale) without a norm kernel between them: the residual add and the RMSNorm of
+    transformer.py:45-50 / layers.py:70-74 around two Linears.  Each output is checked against the
+    oracle's dequantized weights in fp64: the new residual stream, its bf16 image (bit for bit the
+    rounding of the kernel's own fp32 values), the per-tile sums of squares, the row-scaled product, and
+    the product against the REFERENCE order (normalise, round to bf16, multiply) within bf16 rounding.
+    With gate = 1 the rows of W2 count as tiles of 8 gate rows and 8 up rows: silu(a) * u in bf16."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.ajq_gemv_epilogue_supported(m, k1) == 1 and lib.ajq_gemv_epilogue_supported(m, d) == 1
+    w1_hat, wq1, meta1 = _quantized(scheme, d, k1, 500 + k1, cuda)
+    w2_hat, wq2, meta2 = _quantized(scheme, n2, d, 600 + n2, cuda)
+    g = torch.Generator().manual_seed(31 * m + d)
+    x = make_activations(m, k1, 11, True)
+    h_in = torch.randn((m, d), generator=g) * 3.0
+    gain = torch.rand(d, generator=g) + 0.5
+    eps = 1e-5
+    res_fn = lib.ajq_w4a16_gemv_residual if scheme == "w4" else lib.ajq_w8a16_gemv_residual
+    row_fn = lib.ajq_w4a16_gemv_rowscale if scheme == "w4" else lib.ajq_w8a16_gemv_rowscale
+    xg, hg, gg = x.to(cuda), h_in.to(cuda), gain.to(cuda)
+    h_out = torch.zeros((m, d), dtype=torch.float32, device=cuda)
+    xt = torch.zeros((m, d), dtype=torch.bfloat16, device=cuda)
+    ssq = torch.zeros((16, d // 16), dtype=torch.float32, device=cuda)
+    _lib.check(res_fn(xg.data_ptr(), m, k1, wq1.data_ptr(), meta1.data_ptr(), d, hg.data_ptr(), gg.data_ptr(),
+                      h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(), st), "gemv_residual")
+    y = torch.empty((m, n2), dtype=torch.float32, device=cuda)
+    _lib.check(row_fn(xt.data_ptr(), ssq.data_ptr(), d // 16, eps, m, d, wq2.data_ptr(), meta2.data_ptr(), n2,
+                      y.data_ptr(), _lib.AJQ_OUT_F32, 0, st), "gemv_rowscale")
+    y16 = torch.empty((m, n2), dtype=torch.bfloat16, device=cuda)
+    _lib.check(row_fn(xt.data_ptr(), ssq.data_ptr(), d // 16, eps, m, d, wq2.data_ptr(), meta2.data_ptr(), n2,
+                      y16.data_ptr(), _lib.AJQ_OUT_BF16, 0, st), "gemv_rowscale")
+    yg = torch.empty((m, n2 // 2), dtype=torch.bfloat16, device=cuda)
+    _lib.check(row_fn(xt.data_ptr(), ssq.data_ptr(), d // 16, eps, m, d, wq2.data_ptr(), meta2.data_ptr(), n2,
+                      yg.data_ptr(), _lib.AJQ_OUT_BF16, 1, st), "gemv_rowscale gate")
+    torch.cuda.synchronize()
+    h_out, xt, ssq, y, y16, yg = h_out.cpu(), xt.cpu(), ssq.cpu(), y.cpu(), y16.cpu(), yg.cpu()
+
+    # the residual stream
+    h_ref = h_in.double() + qspec.quant_linear(x, w1_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    max_abs, rel = errors(h_out, h_ref)
+    assert max_abs <= 2e-3 and rel <= 1e-5, (max_abs, rel)
+    # its bf16 image and the sums of squares, from the kernel's own fp32 values
+    assert torch.equal(xt, (h_out * gain).to(torch.bfloat16))
+    assert torch.equal(ssq[m:], torch.zeros_like(ssq[m:]))
+    tiles = h_out.double().square().reshape(m, d // 16, 16).sum(-1)
+    assert float((ssq[:m].double() - tiles).abs().max() / tiles.max()) <= 1e-6
+    # the row-scaled product
+    rstd = torch.rsqrt(h_out.double().square().mean(-1, keepdim=True) + eps)
+    want = rstd * qspec.quant_linear(xt, w2_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    max_abs, rel = errors(y, want)
+    assert max_abs <= MAX_ABS_TOL and rel <= 1e-5, (max_abs, rel)
+    assert torch.equal(y16, y.to(torch.bfloat16))
+    # the reference order: normalise in fp32, round to bf16, multiply
+    x_ref = ((h_ref.float() * torch.rsqrt(h_ref.float().square().mean(-1, keepdim=True) + eps)) * gain).to(torch.bfloat16)
+    ordered = qspec.quant_linear(x_ref, w2_hat, accumulate=torch.float64, out_dtype=torch.float64)
+    # (two independent bf16 roundings of every activation: 2^-9 / sqrt(3) each, relative, which does not
+    # average out over K; the bound is twice the expected 1.6e-3)
+    assert errors(y, ordered)[1] <= 3.2e-3
+    # the gate: tiles of 8 gate rows and 8 up rows
+    pairs = y.reshape(m, n2 // 16, 2, 8)
+    gate = (torch.nn.functional.silu(pairs[:, :, 0].double()) * pairs[:, :, 1].double()).reshape(m, n2 // 2)
+    assert bf16_rounding_excess(yg, gate, 4e-6 * float(gate.abs().max())) <= 0
+    # unsupported shapes and bad arguments are refused
+    assert lib.ajq_gemv_epilogue_supported(17, 2048) == 0 and lib.ajq_gemv_epilogue_supported(9, 5632) == 0
+    assert lib.ajq_gemv_epilogue_supported(4, 1024) == 0
+    assert row_fn(xt.data_ptr(), ssq.data_ptr(), 6, eps, m, d, wq2.data_ptr(), meta2.data_ptr(), n2, y.data_ptr(),
+                  _lib.AJQ_OUT_F32, 0, st) != 0
+
+
+
 def test_launch_alternative_probes_reproduce_the_reference_chain(cuda):
     """The bench-only probes of the alternatives to one launch per matrix (a chain of dependent GEMV
     stages in ONE launch, activations exchanged through device memory behind flags or as stamped
