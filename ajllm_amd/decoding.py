@@ -15,7 +15,7 @@ import ctypes
 import torch
 
 from . import _lib, modeling
-from .quant import QuantLinear, w4a16_matmul, w8a16_matmul
+from .quant import QuantLinear, repack_w4, repack_w8, w4a16_matmul, w8a16_matmul
 
 
 class GraphDecoder:
@@ -180,6 +180,64 @@ class _FusedLinear:
         _lib.check(status, "gemm_gate")
         return y
 
+    @classmethod
+    def interleaved_gate(cls, w1: QuantLinear, w3: QuantLinear) -> "_FusedLinear":
+        """(w1 | w3) with the rows interleaved in blocks of 8, so that every 16-row tile of the private
+        layout holds 8 gate-projection rows and the 8 matching up-projection rows: a GEMV workgroup
+        then has both factors of ``silu(a) * u`` for its 8 outputs (``rowscaled(..., gated=True)``).
+        Quantization is per row, so the canonical tensors are permuted, not requantized."""
+        if w1.scheme != w3.scheme or w1.in_features != w3.in_features or w1.out_features != w3.out_features:
+            raise ValueError("w1 and w3 must share scheme and shape")
+        if w1.out_features % 8 != 0:
+            raise ValueError("d_ff must be a multiple of 8")
+
+        def mix(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+            blocks = torch.stack((a.reshape(a.shape[0] // 8, 8, *a.shape[1:]), b.reshape(b.shape[0] // 8, 8, *b.shape[1:])), dim=1)
+            return blocks.reshape(2 * a.shape[0], *a.shape[1:]).contiguous()
+
+        self = cls.__new__(cls)
+        self.scheme = w1.scheme
+        self.in_features = w1.in_features
+        self.out_features = 2 * w1.out_features
+        if self.scheme == "w8a16":
+            self.wq = repack_w8(mix(w1.qweight, w3.qweight))
+            self.meta = mix(w1.scales, w3.scales)
+        else:
+            self.wq, self.meta = repack_w4(mix(w1.qweight, w3.qweight), mix(w1.scales, w3.scales), mix(w1.zeros, w3.zeros))
+        self.rows16 = self.wq.shape[0] * 16
+        return self
+
+    def epilogue_fusable(self, batch: int) -> bool:
+        """Whether the GEMVs with a residual / row-scale / gate epilogue are built for this batch and
+        input width."""
+        return bool(_lib.load().ajq_gemv_epilogue_supported(batch, self.in_features))
+
+    def residual(self, x_bf16: torch.Tensor, h_in: torch.Tensor, gain: torch.Tensor, h_out: torch.Tensor,
+                 xt: torch.Tensor, ssq: torch.Tensor) -> None:
+        """``h_out = h_in + self(x)``, ``xt = bf16(h_out * gain)`` and the per-tile sums of squares of
+        ``h_out`` in ``ssq`` (what the next ``rowscaled`` needs in place of a norm), one launch."""
+        lib = _lib.load()
+        fn = lib.ajq_w8a16_gemv_residual if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_residual
+        _lib.check(fn(x_bf16.data_ptr(), x_bf16.shape[0], self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(),
+                      _stream()), "gemv_residual")
+
+    def rowscaled(self, xt: torch.Tensor, ssq: torch.Tensor, eps: float, gated: torch.Tensor | None = None) -> torch.Tensor:
+        """``self(RMSNorm(h) * gain)`` from ``xt = bf16(h * gain)`` and the sums of squares ``residual`` left,
+        one launch; with ``gated`` (bf16 ``[rows, out / 2]``, for an ``interleaved_gate`` pair) the SwiGLU
+        product of the outputs is written there instead."""
+        lib = _lib.load()
+        rows = xt.shape[0]
+        fn = lib.ajq_w8a16_gemv_rowscale if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_rowscale
+        if gated is None:
+            y = torch.empty((rows, self.rows16), dtype=torch.float32, device=xt.device)
+            dtype, gate = _lib.AJQ_OUT_F32, 0
+        else:
+            y, dtype, gate = gated, _lib.AJQ_OUT_BF16, 1
+        _lib.check(fn(xt.data_ptr(), ssq.data_ptr(), ssq.shape[1], eps, rows, self.in_features, self.wq.data_ptr(),
+                      self.meta.data_ptr(), self.rows16, y.data_ptr(), dtype, gate, _stream()), "gemv_rowscale")
+        return y
+
     def fusable(self, batch: int) -> bool:
         """Whether the GEMV with a norm / gate prologue is built for this batch and input width."""
         return bool(_lib.load().ajq_gemv_fused_supported(batch, self.in_features))
@@ -296,6 +354,21 @@ class FusedDecoder(GraphDecoder):
         # (small batches; one launch less per layer)
         self.merge_splits = self.layers[0]["o"].merge_splits(batch) if self.layers[0]["o"].in_features == d else 0
         self.fuse_merge = self.merge_splits > 0
+        # Larger batches (every workgroup would re-read the fp32 sources of all rows): the norm's row scale
+        # is applied to the OUTPUTS of q|k|v, w1|w3 and the head instead, the output projection and w2 add
+        # the residual and prepare the next norm on their way out, and w1|w3 (rows interleaved in blocks
+        # of 8) applies the gate: six launches per layer instead of nine.
+        self.fuse_epilogue = (
+            not self.fuse_norm and self.d_ff % 8 == 0 and d // 16 <= 256
+            and self.layers[0]["o"].in_features == d
+            and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
+            and self.head.epilogue_fusable(batch)
+        )
+        if self.fuse_epilogue:
+            for w, layer in zip(self.layers, model.layers):
+                w["w13i"] = _FusedLinear.interleaved_gate(layer.feed_forward.w1, layer.feed_forward.w3)
+            self.xt = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
+            self.ssq = torch.zeros((16, d // 16), dtype=torch.float32, device=dev)
         self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)
@@ -387,6 +460,9 @@ class FusedDecoder(GraphDecoder):
     def launches_per_step(self) -> int:
         """Kernel launches of one decode step as this decoder is configured."""
         lib = _lib.load()
+        if self.fuse_epilogue:
+            # q|k|v, attention (+ merge), output projection, w1|w3 with the gate, w2; the first norm, head, pick
+            return (5 if self.fuse_merge else 6) * len(self.layers) + 3
         per_layer = 2 if self.fuse_norm else 4           # q|k|v and w1|w3, each with or without its norm launch
         per_layer += 1                                   # attention
         if not self.fuse_merge:                          # merge of its row chunks (none if there is one chunk)
@@ -400,6 +476,8 @@ class FusedDecoder(GraphDecoder):
     def _logits(self) -> torch.Tensor:
         """Logits ``[B, V]`` of the token whose embedding row is in ``self.embedded`` (``prefill`` and
         every step leave it there), at cache row ``cache.position``; the decoding state is untouched."""
+        if self.fuse_epilogue:
+            return self._logits_epilogue()
         lib, st = _lib.load(), _stream()
         b, d = self.batch, self.model.d_model
         pos = self.cache.position
@@ -447,6 +525,42 @@ class FusedDecoder(GraphDecoder):
                 _lib.check(lib.ajq_swiglu(ab.data_ptr(), self.gated.data_ptr(), b, self.d_ff, st), "swiglu")
                 delta = w["w2"](self.gated)
         self.logits_full = normed_linear(self.head, self.final_gain, self.final_eps)
+        return self.logits_full[:, : self.vocab]
+
+
+    def _attention(self, index: int, w: dict, qkv: torch.Tensor) -> None:
+        """RoPE, cache write and single-query attention of layer ``index`` into ``self.attended``."""
+        _lib.check(_lib.load().ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
+                                             self.cache.position.data_ptr(), self.cache.keys[index].data_ptr(),
+                                             self.cache.values[index].data_ptr(), self.kv_flag, self.batch, self.heads,
+                                             self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
+                                             self.attn_ws.data_ptr(), self.attn_ws_bytes, _stream()), "attn_step")
+
+    def _logits_epilogue(self) -> torch.Tensor:
+        """``_logits`` for batches too large for the norm / gate prologues: no norm, gate or residual launch
+        between the matmuls of a layer (only the very first norm of a step is a launch of its own)."""
+        lib, st = _lib.load(), _stream()
+        b, d = self.batch, self.model.d_model
+        first = self.layers[0]
+        _lib.check(lib.ajq_add_rmsnorm(self.embedded.data_ptr(), None, first["g1"].data_ptr(), first["eps1"],
+                                       self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+        cur = self.embedded
+
+        def other() -> torch.Tensor:
+            return self.hidden2 if cur is self.hidden else self.hidden
+
+        for index, w in enumerate(self.layers):
+            qkv = w["qkv"](self.normed) if index == 0 else w["qkv"].rowscaled(self.xt, self.ssq, w["eps1"])
+            self._attention(index, w, qkv)
+            nxt = other()
+            w["o"].residual(self.attended, cur, w["g2"], nxt, self.xt, self.ssq)
+            cur = nxt
+            w["w13i"].rowscaled(self.xt, self.ssq, w["eps2"], gated=self.gated)
+            nxt = other()
+            gain = self.layers[index + 1]["g1"] if index + 1 < len(self.layers) else self.final_gain
+            w["w2"].residual(self.gated, cur, gain, nxt, self.xt, self.ssq)
+            cur = nxt
+        self.logits_full = self.head.rowscaled(self.xt, self.ssq, self.final_eps)
         return self.logits_full[:, : self.vocab]
 
 

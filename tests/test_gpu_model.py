@@ -581,14 +581,9 @@ def test_fused_decoder_tokens_match_the_oracle_model(cuda):
     assert report["identical_rows"] + len(report["attributable"]) == 4
 
 
-@pytest.mark.parametrize("scheme,batch", [("w4a16_g128", 1), ("w8a16", 4)])
-def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme, batch):
-    """Widths the prologue GEMVs are built for (d_model 1024, d_ff 2048, grouped-query heads), with the
-    norm and gate prologues forced on: the graph-replayed tokens against the CPU oracle model, and the
-    decode-step logits of every step along the oracle's tokens against the oracle's logits."""
-    torch.manual_seed(16)
-    model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=1024, num_layers=3, num_heads=8,
-                                   d_ff=2048, num_kv_heads=4).eval()
+def _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure):
+    """The graph-replayed tokens of a FusedDecoder (set up by ``configure``) against the CPU oracle model,
+    and the decode-step logits of every step along the oracle's tokens against the oracle's logits."""
     ref = _oracle_model(model, scheme)
     fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
     prompt = torch.randint(0, 2048, (batch, 48), generator=torch.Generator().manual_seed(13))
@@ -605,8 +600,7 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
     top2 = torch.topk(ref_logits, 2, dim=-1).values
     margins = top2[..., 0] - top2[..., 1]
     dec = decoding.FusedDecoder(fast, batch, 48 + new)
-    assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
-    dec.fuse_norm = dec.fuse_gate = True
+    configure(dec)
     dec.prefill(prompt.to(cuda))
     got = dec.generate(new).cpu()
     # teacher-forced: decode-step logits along the oracle's tokens
@@ -631,6 +625,38 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
         if len(d) and int(d[0]) > 0:
             first = int(d[0])
             assert float(margins[b, first]) <= 2 * float(step_err[b, first]) + 1e-6, (b, first)
+
+
+@pytest.mark.parametrize("scheme,batch", [("w4a16_g128", 1), ("w8a16", 4)])
+def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme, batch):
+    """Widths the prologue GEMVs are built for (d_model 1024, d_ff 2048, grouped-query heads), with the
+    norm and gate prologues forced on."""
+    torch.manual_seed(16)
+    model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=1024, num_layers=3, num_heads=8,
+                                   d_ff=2048, num_kv_heads=4).eval()
+
+    def configure(dec):
+        assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
+        dec.fuse_norm = dec.fuse_gate = True
+
+    _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
+
+
+@pytest.mark.parametrize("scheme,batch,d_ff", [("w4a16_g128", 8, 5632), ("w8a16", 13, 2048), ("w4a16_g128", 5, 4096)])
+def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff):
+    """Batches above the prologue range on widths the epilogue GEMVs are built for (d_model 2048): no norm,
+    gate or residual launch inside a layer (the norm's row scale is applied to the matmul outputs, the
+    residual add and the next norm's preparation ride in the output projection and w2, w1|w3 applies the
+    gate on interleaved rows): six launches per layer."""
+    torch.manual_seed(18)
+    model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=2048, num_layers=2, num_heads=16,
+                                   d_ff=d_ff, num_kv_heads=4).eval()
+
+    def configure(dec):
+        assert dec.fuse_epilogue and not dec.fuse_norm and not dec.fuse_gate
+        assert dec.launches_per_step() == 6 * 2 + 3
+
+    _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
 
 
 def test_quantized_checkpoint_round_trip(cuda, tmp_path):
