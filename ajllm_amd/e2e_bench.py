@@ -97,6 +97,18 @@ def bench_decode_short(device, log=print, batches=(1, 8), scheme: str = "w4a16_g
              "quant_linear_GB/s": packed / t_linear / 1e9, "packed_weight_bytes": packed,
              "launches_per_step": dec.launches_per_step(), "model_build_s": build_s,
              "tokens_in_vocab": bool(int(tokens.min()) >= 0 and int(tokens.max()) < CONFIG["vocab_size"])}
+        # the same decode with keys and values stored as bf16 (the decoder's kv_dtype option; not the
+        # reference's arithmetic: its cache has the model's dtype)
+        del dec
+        dec = decoding.FusedDecoder(model, batch, PROMPT_LEN + NEW_TOKENS, torch.bfloat16)
+        dec.prefill(prompt, fused=True)
+        dec.generate(8)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.generate(NEW_TOKENS)
+        torch.cuda.synchronize()
+        t_bf16 = time.perf_counter() - t0
+        r["bf16_kv_cache"] = {"decode_tok/s": batch * steps / t_bf16, "ms_per_step": t_bf16 / steps * 1e3}
         log("decode", r)
         results.append(r)
         del dec
