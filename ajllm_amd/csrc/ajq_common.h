@@ -96,4 +96,18 @@ __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
 
+// Sum over the 16 lanes of a team, result in every lane: four adds whose second operand comes
+// through the DPP row rotate (a "row" is 16 lanes), no LDS crossbar round trips.
+template <int kRor>
+__device__ __forceinline__ float row_ror(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + kRor, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float team_sum16(float v) {
+  v += row_ror<8>(v);
+  v += row_ror<4>(v);
+  v += row_ror<2>(v);
+  v += row_ror<1>(v);
+  return v;
+}
+
 }  // namespace ajq

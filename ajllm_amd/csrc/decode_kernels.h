@@ -187,19 +187,6 @@ __device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
              __uint_as_float(v.w & 0xFFFF0000u)};
 }
 
-// Sum over the 16 lanes of a team, result in every lane: four adds whose second operand comes
-// through the DPP row rotate (a "row" is 16 lanes), no LDS crossbar round trips.
-template <int kRor>
-__device__ __forceinline__ float row_ror(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + kRor, 0xF, 0xF, false));
-}
-__device__ __forceinline__ float team_sum16(float v) {
-  v += row_ror<8>(v);
-  v += row_ror<4>(v);
-  v += row_ror<2>(v);
-  v += row_ror<1>(v);
-  return v;
-}
 // 2^x by the hardware instruction (1 ulp); the softmax below keeps its running maximum and
 // scores in the base-2 domain, scores pre-multiplied by log2(e)
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }

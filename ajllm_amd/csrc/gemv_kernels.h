@@ -207,8 +207,8 @@ __device__ __forceinline__ void dequant_gemv_body(
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         const int j = wave * 4 + c + u * kWaves * 4;  // float4 index inside the row
-        const bool live = 4 * j < ep.parts;
-        const float4 t = *reinterpret_cast<const float4*>(ep.ssq_in + (size_t)m * ep.parts + (live ? 4 * j : 0));
+        const bool live = 4 * j < ep.parts && m < M;  // (idle lanes re-read the first 16 bytes)
+        const float4 t = *reinterpret_cast<const float4*>(ep.ssq_in + (live ? (size_t)m * ep.parts + 4 * j : 0));
         ssq_share[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
       }
     }
@@ -291,11 +291,7 @@ __device__ __forceinline__ void dequant_gemv_body(
         ep.h_out[(size_t)m * N + n] = h;
         ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
       }
-      float sq = m < M ? h * h : 0.f;
-      sq += __shfl_xor(sq, 1);
-      sq += __shfl_xor(sq, 2);
-      sq += __shfl_xor(sq, 4);
-      sq += __shfl_xor(sq, 8);
+      const float sq = team_sum16(m < M ? h * h : 0.f);  // over the tile's 16 columns (one DPP row)
       if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt] = sq;
     }
     return;
@@ -306,7 +302,7 @@ __device__ __forceinline__ void dequant_gemv_body(
     for (int i = 0; i < kLive; ++i) {
       const int m = 4 * kc + i;
       const float v = sum[i] * cs * rstd[i];
-      const float other = __shfl_xor(v, 8);
+      const float other = row_ror<8>(v);  // the lane 8 columns away
       if (nl < 8 && m < M)
         reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + nt * 8 + nl] =
             f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);

@@ -113,6 +113,34 @@ def test_greedy_tokens_match_the_oracle_model(cuda, scheme, batch):
     assert int(disagree.sum()) <= max(1, disagree.numel() // 10)
 
 
+@pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
+def test_reference_medium_geometry_decodes_through_the_graph_decoder(cuda, scheme):
+    """The geometry of the reference's own configs/models/transformer_medium.yaml (d_model 768, 12 heads of
+    head_dim 64, d_ff 2048, RoPE, pre-norm RMSNorm, SwiGLU, tied embeddings; fewer layers and a smaller
+    vocabulary here): every Linear is swapped, and the graph-replayed decode over the model's own code gives
+    the eager loop's tokens.  The all-kernel FusedDecoder is built for head_dim 128 and an untied head and
+    says so instead of running something else."""
+    torch.manual_seed(21)
+    model = modeling.TransformerLM(vocab_size=1024, context_length=128, d_model=768, num_layers=3, num_heads=12,
+                                   d_ff=2048, tie_embeddings=True).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    swapped = [m for m in fast.modules() if isinstance(m, QuantLinear)]
+    assert len(swapped) == 3 * 7 and fast.lm_head is None
+    prompt = torch.randint(0, 1024, (2, 24), generator=torch.Generator().manual_seed(5)).to(cuda)
+    eager, margins = modeling.greedy_decode(fast, prompt, 32, return_margins=True)
+    dec = decoding.GraphDecoder(fast, 2, 64)
+    dec.prefill(prompt)
+    got = dec.generate(32)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 24, noise=1e-3)
+    assert not report["unexplained"], report
+    with torch.no_grad():
+        dense = model.to(cuda)(prompt).float()
+        quant = fast(prompt).float()
+    assert errors(quant.cpu(), dense.cpu())[1] <= (0.3 if scheme == "w4a16_g128" else 0.05)  # the quantization error itself
+    with pytest.raises(ValueError, match="head_dim 128"):
+        decoding.FusedDecoder(fast, 2, 64)
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 def test_graph_replayed_decoding_matches_eager_decoding(cuda, batch):
     """The decode step recorded into a HIP graph and replayed per token (with the program's own
