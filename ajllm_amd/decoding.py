@@ -284,7 +284,8 @@ class FusedDecoder(GraphDecoder):
     and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), the greedy pick
     with the embedding lookup and the step counters (``ajq_greedy_pick``).  Five launches per layer
     at batch 1 (q|k|v with the norm, attention, output projection with the merge of the attention's
-    row chunks, w1|w3 with the norm, w2 with the gate: ``launches_per_step``), up to nine at large batch.
+    row chunks, w1|w3 with the norm, w2 with the gate: ``launches_per_step``); six at batch 5-16, where the norm's
+    row scale, the residual add and the gate ride in the GEMVs' epilogues; up to nine beyond.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
