@@ -429,13 +429,19 @@ int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const u
                     int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
 #define AJQ_EPI(W, T, R) return launch_gemv_epi_cfg<W, T, R, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
   if (K == 2048) {
+    if (M <= 1) AJQ_EPI(8, 2, 1);
+    if (M <= 4) AJQ_EPI(8, 2, 4);
     if (M <= 8) AJQ_EPI(8, 2, 8);
     AJQ_EPI(8, 2, 16);
   }
   if (K == 4096) {
+    if (M <= 1) AJQ_EPI(8, 4, 1);
+    if (M <= 4) AJQ_EPI(8, 4, 4);
     if (M <= 8) AJQ_EPI(8, 4, 8);
     AJQ_EPI(8, 4, 16);
   }
+  if (M <= 1) AJQ_EPI(11, 4, 1);
+  if (M <= 4) AJQ_EPI(11, 4, 4);
   AJQ_EPI(11, 4, 8);
 #undef AJQ_EPI
 }
@@ -499,7 +505,20 @@ int launch_gemv_pro_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, 
   auto kernel = dequant_gemv_pro_kernel<kWaves, TPW, MROWS, kW4, kPro>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
-                     meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out, S);
+                     meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out, S, nullptr, nullptr, nullptr);
+  return AJQ_OK;
+}
+
+// the merge prologue with the residual epilogue (output projection of a decode step)
+template <int TPW, int MROWS, bool kW4>
+int launch_gemv_merge_resid_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N,
+                                const float* partial, int S, const float* h_in, const float* gain, float* h_out,
+                                uint16_t* xt, float* ssq, hipStream_t stream) {
+  constexpr size_t lds = gemv_pro_lds_bytes(8, TPW, MROWS);
+  auto kernel = dequant_gemv_pro_kernel<8, TPW, MROWS, kW4, kProMerge, true>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(8 * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, K,
+                     M | (1 << 8), N, nullptr, scales8, partial, nullptr, gain, 0.f, h_out, S, h_in, xt, ssq);
   return AJQ_OK;
 }
 
@@ -567,6 +586,40 @@ int launch_gemv_merge(int M, int K, const uint32_t* wq, const uint32_t* meta, co
   if (M <= 1) AJQ_MRG(4, 1);
   AJQ_MRG(4, 2);
 #undef AJQ_MRG
+}
+
+template <bool kW4>
+int launch_gemv_merge_resid(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N,
+                            const float* partial, int S, const float* h_in, const float* gain, float* h_out, uint16_t* xt,
+                            float* ssq, hipStream_t stream) {
+#define AJQ_MRG(T, R) \
+  return launch_gemv_merge_resid_cfg<T, R, kW4>(M, K, wq, meta, scales8, N, partial, S, h_in, gain, h_out, xt, ssq, stream)
+  if (K == 2048) {
+    if (M <= 1) AJQ_MRG(2, 1);
+    if (M <= 2) AJQ_MRG(2, 2);
+    AJQ_MRG(2, 4);
+  }
+  if (M <= 1) AJQ_MRG(4, 1);
+  AJQ_MRG(4, 2);
+#undef AJQ_MRG
+}
+
+template <bool kW4>
+int gemv_merge_residual(const char* name, const float* partial, int S, int M, int K, const uint32_t* wq, const void* aux,
+                        int N, const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                        void* stream) {
+  if (int s = check_matmul_args(name, partial, M, K, wq, aux, N, h_out, AJQ_OUT_F32, kGroup)) return s;
+  const int cap = gemv_merge_max_splits(M, K);
+  if (cap == 0 || S < 1 || S > cap)
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d, S=%d is not built (ajq_gemv_merge_max_splits gives %d)", name, M, K, S, cap);
+  if (!h_in || !gain || !xt_out || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (h_in == h_out) return fail(AJQ_ERR_NULL, "%s: h_out must be a buffer other than h_in", name);
+  const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
+  const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
+  if (int s = launch_gemv_merge_resid<kW4>(M, K, wq, meta, scales, N, partial, S, h_in, gain, h_out, xt_out, ssq_out,
+                                           (hipStream_t)stream))
+    return s;
+  return check_launch(name);
 }
 
 int check_pro(const char* name, int M, int K, const void* a, const void* b) {
@@ -723,6 +776,20 @@ int ajq_w8a16_gemv_merge(const float* partial, int S, int M, int K, const uint32
                                        (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemv_merge");
+}
+
+int ajq_w4a16_gemv_merge_residual(const float* partial, int S, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
+                                  const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
+                                  void* stream) {
+  return gemv_merge_residual<true>("ajq_w4a16_gemv_merge_residual", partial, S, M, K, wq, meta, N, h_in, gain, h_out, xt_out,
+                                   ssq_out, stream);
+}
+
+int ajq_w8a16_gemv_merge_residual(const float* partial, int S, int M, int K, const uint32_t* wq, const uint16_t* scales,
+                                  int N, const float* h_in, const float* gain, float* h_out, uint16_t* xt_out,
+                                  float* ssq_out, void* stream) {
+  return gemv_merge_residual<false>("ajq_w8a16_gemv_merge_residual", partial, S, M, K, wq, scales, N, h_in, gain, h_out,
+                                    xt_out, ssq_out, stream);
 }
 
 // --------------------------------------------------------------- GEMM -----

@@ -30,7 +30,10 @@ constexpr int merge_chunks_per_lane(int mrows, int tpw) {
   return 8 / (mrows * tpw) > 4 ? 4 : (8 / (mrows * tpw) < 1 ? 1 : 8 / (mrows * tpw));
 }
 
-template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
+// kResid (with the merge prologue): the output side of dequant_gemv_epi_kernel's kEpiResidual as well:
+// h_out = res_h_in + (x W^T), res_xt = bf16(h_out * gain) for the norm that follows, res_ssq[m][tile] the
+// sum of squares of h_out over this workgroup's 16 columns; y is not written.
+template <int kWaves, int TPW, int MROWS, bool kW4, int kPro, bool kResid = false>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -42,8 +45,11 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     const float* __restrict__ src1,        // norm: delta [M, K] or nullptr
     const float* __restrict__ gain,        // norm: [K]
     float eps,                             // norm
-    float* __restrict__ h_out,             // norm: h_in + delta [M, K]; must not alias h_in
-    int S) {                               // merge: row chunks per (row, head), 1 <= S <= 4 * merge_chunks_per_lane
+    float* __restrict__ h_out,             // norm: h_in + delta [M, K]; must not alias h_in.  kResid: [M, N]
+    int S,                                 // merge: row chunks per (row, head), 1 <= S <= 4 * merge_chunks_per_lane
+    const float* __restrict__ res_h_in,    // kResid: [M, N]
+    uint16_t* __restrict__ res_xt,         // kResid: bf16 [M, N]
+    float* __restrict__ res_ssq) {         // kResid: [16][N / 16]
   const int M = m_flags & 0xFF;
   const bool out_f32 = (m_flags >> 8) != 0;
   constexpr int kSlice = TPW * kGroup;
@@ -129,6 +135,13 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
 #pragma unroll
     for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
+  }
+  constexpr int kLiveRows = MROWS < 4 ? MROWS : 4;
+  float h_old[kLiveRows], gain_n = 0.f;
+  if (kResid) {  // behind the weights in issue order, used at the very end
+    gain_n = gain[nt * kTileN + nl];
+#pragma unroll
+    for (int i = 0; i < kLiveRows; ++i) h_old[i] = res_h_in[(size_t)min(4 * kc + i, M - 1) * N + nt * kTileN + nl];
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -289,6 +302,23 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   const int n = nt * kTileN + nl;
   float cs = 1.0f;
   if (!kW4) cs = f16_bits_to_f32(scales8[n]);
+  if (kResid) {
+    const int ntiles = N / kTileN;
+#pragma unroll
+    for (int i = 0; i < kLive; ++i) {
+      const int m = 4 * kc + i;
+      float v = sum[i] * cs;
+      asm volatile("" : "+v"(v));  // no fused multiply-add: bit for bit the plain output, then the add
+      const float h = h_old[i] + v;
+      if (m < M) {
+        h_out[(size_t)m * N + n] = h;
+        res_xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+      }
+      const float sq = team_sum16(m < M ? h * h : 0.f);
+      if (nl == 0 && m < M) res_ssq[(size_t)m * ntiles + nt] = sq;
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < kLive; ++i) {
     const int m = 4 * kc + i;

@@ -286,7 +286,9 @@ __device__ __forceinline__ void dequant_gemv_body(
 #pragma unroll
     for (int i = 0; i < kLive; ++i) {
       const int m = 4 * kc + i;
-      const float h = h_old[i] + sum[i] * cs * rstd[i];
+      float v = sum[i] * cs * rstd[i];
+      asm volatile("" : "+v"(v));  // no fused multiply-add: bit for bit the plain output, then the add
+      const float h = h_old[i] + v;
       if (m < M) {
         ep.h_out[(size_t)m * N + n] = h;
         ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);

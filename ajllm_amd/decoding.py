@@ -222,6 +222,16 @@ class _FusedLinear:
                       self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(),
                       _stream()), "gemv_residual")
 
+    def merge_residual(self, partial: torch.Tensor, splits: int, rows: int, h_in: torch.Tensor, gain: torch.Tensor,
+                       h_out: torch.Tensor, xt: torch.Tensor, ssq: torch.Tensor) -> None:
+        """``residual`` whose input is the attention output merged from ``splits`` partial results per (row, head) on
+        the way in (as ``after_merge``), one launch."""
+        lib = _lib.load()
+        fn = lib.ajq_w8a16_gemv_merge_residual if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_merge_residual
+        _lib.check(fn(partial.data_ptr(), splits, rows, self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(),
+                      _stream()), "gemv_merge_residual")
+
     def rowscaled(self, xt: torch.Tensor, ssq: torch.Tensor, eps: float, gated: torch.Tensor | None = None) -> torch.Tensor:
         """``self(RMSNorm(h) * gain)`` from ``xt = bf16(h * gain)`` and the sums of squares ``residual`` left,
         one launch; with ``gated`` (bf16 ``[rows, out / 2]``, for an ``interleaved_gate`` pair) the SwiGLU
@@ -359,13 +369,18 @@ class FusedDecoder(GraphDecoder):
         # is applied to the OUTPUTS of q|k|v, w1|w3 and the head instead, the output projection and w2 add
         # the residual and prepare the next norm on their way out, and w1|w3 (rows interleaved in blocks
         # of 8) applies the gate: six launches per layer instead of nine.
+        # At small batch as well, provided the output projection can merge the attention's row chunks on its way
+        # in (five launches per layer either way, and the epilogue forms cost less than the prologue forms:
+        # 3.9 against 4.8 us for q|k|v at batch 1, 4.3 against 6.7 at batch 4).
         self.fuse_epilogue = (
-            not self.fuse_norm and self.d_ff % 8 == 0 and d // 16 <= 256
+            (batch > 4 or self.fuse_merge) and self.d_ff % 8 == 0 and d // 16 <= 256
             and self.layers[0]["o"].in_features == d
             and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
             and self.head.epilogue_fusable(batch)
         )
         if self.fuse_epilogue:
+            self.first_norm_fused = self.fuse_norm   # the step's very first norm rides in layer 0's q|k|v where built
+            self.fuse_norm = self.fuse_gate = False
             for w, layer in zip(self.layers, model.layers):
                 w["w13i"] = _FusedLinear.interleaved_gate(layer.feed_forward.w1, layer.feed_forward.w3)
             self.xt = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
@@ -463,7 +478,7 @@ class FusedDecoder(GraphDecoder):
         lib = _lib.load()
         if self.fuse_epilogue:
             # q|k|v, attention (+ merge), output projection, w1|w3 with the gate, w2; the first norm, head, pick
-            return (5 if self.fuse_merge else 6) * len(self.layers) + 3
+            return (5 if self.fuse_merge else 6) * len(self.layers) + (2 if self.first_norm_fused else 3)
         per_layer = 2 if self.fuse_norm else 4           # q|k|v and w1|w3, each with or without its norm launch
         per_layer += 1                                   # attention
         if not self.fuse_merge:                          # merge of its row chunks (none if there is one chunk)
@@ -543,18 +558,34 @@ class FusedDecoder(GraphDecoder):
         lib, st = _lib.load(), _stream()
         b, d = self.batch, self.model.d_model
         first = self.layers[0]
-        _lib.check(lib.ajq_add_rmsnorm(self.embedded.data_ptr(), None, first["g1"].data_ptr(), first["eps1"],
-                                       self.normed.data_ptr(), b, d, st), "add_rmsnorm")
         cur = self.embedded
 
         def other() -> torch.Tensor:
             return self.hidden2 if cur is self.hidden else self.hidden
 
         for index, w in enumerate(self.layers):
-            qkv = w["qkv"](self.normed) if index == 0 else w["qkv"].rowscaled(self.xt, self.ssq, w["eps1"])
-            self._attention(index, w, qkv)
+            if index > 0:
+                qkv = w["qkv"].rowscaled(self.xt, self.ssq, w["eps1"])
+            elif self.first_norm_fused:
+                qkv = w["qkv"].after_norm(self.embedded, None, first["g1"], first["eps1"], self.hidden)
+                cur = self.hidden  # (a copy of the embedding row)
+            else:
+                _lib.check(lib.ajq_add_rmsnorm(self.embedded.data_ptr(), None, first["g1"].data_ptr(), first["eps1"],
+                                               self.normed.data_ptr(), b, d, st), "add_rmsnorm")
+                qkv = w["qkv"](self.normed)
             nxt = other()
-            w["o"].residual(self.attended, cur, w["g2"], nxt, self.xt, self.ssq)
+            if self.fuse_merge:
+                splits = ctypes.c_int(0)
+                _lib.check(lib.ajq_attn_step_partial(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
+                                                     self.cache.position.data_ptr(), self.cache.keys[index].data_ptr(),
+                                                     self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
+                                                     self.kv_heads, 128, self.max_len, self.merge_splits,
+                                                     ctypes.addressof(splits), self.attn_ws.data_ptr(),
+                                                     self.attn_ws_bytes, st), "attn_step_partial")
+                w["o"].merge_residual(self.attn_ws, splits.value, b, cur, w["g2"], nxt, self.xt, self.ssq)
+            else:
+                self._attention(index, w, qkv)
+                w["o"].residual(self.attended, cur, w["g2"], nxt, self.xt, self.ssq)
             cur = nxt
             w["w13i"].rowscaled(self.xt, self.ssq, w["eps2"], gated=self.gated)
             nxt = other()

@@ -130,7 +130,7 @@ int ajq_w4a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
                         void* y, int out_dtype, void* stream);
 int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                         void* y, int out_dtype, void* stream);
-/* The same GEMV with work around the matmul, for decode steps of several rows, where a launch of its own
+/* The same GEMV with work around the matmul, for decode steps, where a launch of its own
  * for the residual add, the RMSNorm or the SwiGLU gate costs more than the operation itself
  * (TransformerBlock.forward, src/ajllm/modeling/transformer.py:45-50; RMSNorm, layers.py:70-74; SwiGLU,
  * activations.py:24-25).  The row scale of an RMSNorm commutes with the matmul, so the pair below computes
@@ -161,6 +161,16 @@ int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, flo
 int ajq_w8a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
                             const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
                             void* stream);
+/*   _merge_residual: _residual whose x is the single-query attention output merged from the S partial results
+ *              per (row, head) in ajq_attn_step_partial's workspace, as in _merge below (same limits:
+ *              ajq_gemv_merge_max_splits): the output projection of a decode step at small batch, with the
+ *              merge on its way in and the residual add and the next norm's preparation on its way out. */
+int ajq_w4a16_gemv_merge_residual(const float* partial, int S, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                                  int N, const float* h_in, const float* gain, float* h_out, uint16_t* xt_out,
+                                  float* ssq_out, void* stream);
+int ajq_w8a16_gemv_merge_residual(const float* partial, int S, int M, int K, const uint32_t* wq, const uint16_t* scales,
+                                  int N, const float* h_in, const float* gain, float* h_out, uint16_t* xt_out,
+                                  float* ssq_out, void* stream);
 /*   _merge: x = bf16 of the single-query attention output [M, K] (K = heads * 128), merged from the S
  *          partial results per (row, head) that ajq_attn_step_partial left in its workspace -- the
  *          softmax-weighted value sum of scaled_dot_product_attention (src/ajllm/modeling/attention.py:20-33)

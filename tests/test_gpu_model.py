@@ -517,6 +517,20 @@ def test_output_projection_that_merges_the_attention_chunks(cuda, scheme, b, h, 
                              out_dtype=torch.float64)
     max_abs, rel = errors(got[:, :272], ref)
     assert rel <= 2e-3 and max_abs <= MAX_ABS_TOL, (max_abs, rel)
+    # the same launch with the residual epilogue: bit for bit h_in + (the merged product), its bf16 image
+    # times the next norm's gain, and the per-tile sums of squares
+    n16 = fused.rows16
+    h_in = torch.randn((b, n16), generator=g).to(cuda)
+    gain = (torch.rand(n16, generator=g) + 0.5).to(cuda)
+    h_out = torch.zeros_like(h_in)
+    xt = torch.zeros((b, n16), dtype=torch.bfloat16, device=cuda)
+    ssq = torch.zeros((16, n16 // 16), dtype=torch.float32, device=cuda)
+    fused.merge_residual(ws2, splits.value, b, h_in, gain, h_out, xt, ssq)
+    torch.cuda.synchronize()
+    assert torch.equal(h_out, h_in + got)
+    assert torch.equal(xt, (h_out * gain).to(torch.bfloat16))
+    tiles = h_out.double().square().reshape(b, n16 // 16, 16).sum(-1)
+    assert float((ssq[:b].double() - tiles).abs().max() / tiles.max()) <= 1e-6 and not ssq[b:].any()
 
 
 @pytest.mark.parametrize("scheme", ["w4a16_g128", "w8a16"])
@@ -670,19 +684,23 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
     _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
 
 
-@pytest.mark.parametrize("scheme,batch,d_ff", [("w4a16_g128", 8, 5632), ("w8a16", 13, 2048), ("w4a16_g128", 5, 4096)])
+@pytest.mark.parametrize("scheme,batch,d_ff", [("w4a16_g128", 8, 5632), ("w8a16", 13, 2048), ("w4a16_g128", 5, 4096),
+                                               ("w4a16_g128", 1, 5632), ("w8a16", 4, 2048), ("w4a16_g128", 2, 4096)])
 def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff):
-    """Batches above the prologue range on widths the epilogue GEMVs are built for (d_model 2048): no norm,
-    gate or residual launch inside a layer (the norm's row scale is applied to the matmul outputs, the
-    residual add and the next norm's preparation ride in the output projection and w2, w1|w3 applies the
-    gate on interleaved rows): six launches per layer."""
+    """Widths the epilogue GEMVs are built for (d_model 2048): no norm, gate or residual launch inside a layer
+    (the norm's row scale is applied to the matmul outputs, the residual add and the next norm's preparation
+    ride in the output projection and w2, w1|w3 applies the gate on interleaved rows): six launches per
+    layer above batch 4, five at small batch, where the output projection also merges the attention's row
+    chunks on its way in and the step's first norm rides in layer 0's q|k|v."""
     torch.manual_seed(18)
     model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=2048, num_layers=2, num_heads=16,
                                    d_ff=d_ff, num_kv_heads=4).eval()
 
     def configure(dec):
         assert dec.fuse_epilogue and not dec.fuse_norm and not dec.fuse_gate
-        assert dec.launches_per_step() == 6 * 2 + 3
+        small = batch <= 4
+        assert dec.fuse_merge == small and dec.first_norm_fused == small
+        assert dec.launches_per_step() == (5 * 2 + 2 if small else 6 * 2 + 3)
 
     _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
 
