@@ -645,6 +645,8 @@ def _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configur
     configure(dec)
     dec.prefill(prompt.to(cuda))
     got = dec.generate(new).cpu()
+    dec.prefill(prompt.to(cuda))
+    assert torch.equal(dec.generate(new).cpu(), got)            # sums run in a fixed order: run-to-run identical
     # teacher-forced: decode-step logits along the oracle's tokens
     dec.prefill(prompt.to(cuda))
     forced = []
