@@ -308,6 +308,77 @@ def cpu_baseline(m: int, n: int, k: int, budget_s: float = 15.0) -> dict:
     }
 
 
+def bench_gemv_forms(device, batches=(1, 4, 8), reps: int = 30) -> list[dict]:
+    """Microseconds per launch, in a graph chain over six distinct W4 weight sets, of the decode GEMV in its
+    plain form and with work folded in: the norm / gate PROLOGUE forms (every workgroup forms the
+    activations from the fp32 sources) against the row-scale / residual / gate EPILOGUE forms (a workgroup
+    touches its own 16 columns), on the 12-layer benchmark model's four projection shapes."""
+    from ajllm_amd import _lib, quantize_w4_g128, repack_w4
+
+    lib = _lib.load()
+    rows = []
+    for name, n, k in (("q|k|v", 6144, 2048), ("output", 2048, 2048), ("w1|w3", 11264, 2048), ("w2", 2048, 5632)):
+        weights = []
+        for _ in range(6):
+            q, s, z = quantize_w4_g128(torch.randn(n, k, device=device) * 0.02)
+            weights.append(repack_w4(q, s, z))
+        for m in batches:
+            x = torch.randn(m, k, device=device).to(torch.bfloat16)
+            y = torch.empty(m, n, device=device)
+            yg = torch.empty(m, n // 2, device=device, dtype=torch.bfloat16)
+            h, gain = torch.randn(m, n, device=device), torch.ones(n, device=device)
+            h2, xt = torch.empty_like(h), torch.empty(m, n, device=device, dtype=torch.bfloat16)
+            ssq_out, ssq_in = torch.zeros(16, n // 16, device=device), torch.rand(16, k // 16, device=device) + 1
+            hk, dk, gk = torch.randn(m, k, device=device), torch.randn(m, k, device=device), torch.ones(k, device=device)
+            hk2, ab = torch.empty_like(hk), torch.randn(m, 2 * k, device=device)
+            forms = {
+                "plain": lambda wq, meta, st: lib.ajq_w4a16_gemv(
+                    x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32, st),
+                "row_scale_epilogue": lambda wq, meta, st: lib.ajq_w4a16_gemv_rowscale(
+                    x.data_ptr(), ssq_in.data_ptr(), k // 16, 1e-5, m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(),
+                    _lib.AJQ_OUT_F32, 0, st),
+                "row_scale_and_gate_epilogue": lambda wq, meta, st: lib.ajq_w4a16_gemv_rowscale(
+                    x.data_ptr(), ssq_in.data_ptr(), k // 16, 1e-5, m, k, wq.data_ptr(), meta.data_ptr(), n, yg.data_ptr(),
+                    _lib.AJQ_OUT_BF16, 1, st),
+                "residual_epilogue": lambda wq, meta, st: lib.ajq_w4a16_gemv_residual(
+                    x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, h.data_ptr(), gain.data_ptr(), h2.data_ptr(),
+                    xt.data_ptr(), ssq_out.data_ptr(), st),
+            }
+            if lib.ajq_gemv_fused_supported(m, k):
+                forms["norm_prologue"] = lambda wq, meta, st: lib.ajq_w4a16_gemv_norm(
+                    hk.data_ptr(), dk.data_ptr(), gk.data_ptr(), 1e-5, hk2.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(),
+                    n, y.data_ptr(), _lib.AJQ_OUT_F32, st)
+                forms["gate_prologue"] = lambda wq, meta, st: lib.ajq_w4a16_gemv_gate(
+                    ab.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32, st)
+            launches = 8 * len(weights)
+            row = {"projection": name, "M": m, "N": n, "K": k}
+            for form, call in forms.items():
+                stream = torch.cuda.Stream()
+                torch.cuda.synchronize()
+                with torch.cuda.stream(stream):
+                    def chain():
+                        for i in range(launches):
+                            status = call(*weights[i % len(weights)], stream.cuda_stream)
+                            if status != 0:
+                                raise RuntimeError(f"{form}: status {status}")
+                    chain()
+                    stream.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=stream):
+                        chain()
+                    graph.replay()
+                    stream.synchronize()
+                    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    start.record(stream)
+                    for _ in range(reps):
+                        graph.replay()
+                    stop.record(stream)
+                    stop.synchronize()
+                row[form + "_us"] = round(start.elapsed_time(stop) * 1e3 / reps / launches, 2)
+            rows.append(row)
+    return rows
+
+
 # ------------------------------------------------------------------ main
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -321,6 +392,8 @@ def main() -> int:
                     help="also time the Llama-3-8B-shaped W8A16 stack (4 x 2048 prefill, batch-32 decode at context 2048)")
     ap.add_argument("--probes", action="store_true",
                     help="also time the alternatives to one launch per matrix for a chain of GEMVs (bench-only probes)")
+    ap.add_argument("--forms", action="store_true",
+                    help="also time the decode GEMV's prologue forms against its epilogue forms (norm, gate, residual)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="timed region only")
     ap.add_argument("--no-decode", action="store_true",
@@ -410,6 +483,10 @@ def main() -> int:
         extras["gemv_chain_launch_alternatives"] = bench_launch_alternatives()
         for row in extras["gemv_chain_launch_alternatives"]:
             log("probe", json.dumps(row))
+    if args.forms:
+        extras["decode_gemv_forms"] = bench_gemv_forms(device)
+        for row in extras["decode_gemv_forms"]:
+            log("forms", json.dumps(row))
     if args.stack:
         from ajllm_amd.stack_bench import bench_stack
 
