@@ -367,6 +367,20 @@ int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const
   return AJQ_OK;
 }
 
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi>
+int launch_skinny_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                          const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  constexpr size_t lds = skinny_epi_lds_bytes(kWaves, TPW, MROWS);
+  static_assert(lds <= 160 * 1024, "skinny configuration exceeds the 160 KiB LDS of a CU");
+  auto kernel = dequant_skinny_epi_kernel<kWaves, TPW, MROWS, NT, kW4, kEpi>;
+  if (int s = allow_big_lds(kernel, lds)) return s;
+  const int ntiles = N / kTileN;
+  const int ngroups = (ntiles + NT - 1) / NT, mblocks = (M + MROWS - 1) / MROWS;
+  hipLaunchKernelGGL(kernel, dim3(8 * ((ngroups + 7) / 8) * mblocks), dim3(kWaves * 64), lds, stream,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32, scales8, ep);
+  return AJQ_OK;
+}
+
 #ifndef AJQ_SKINNY_FORCE_NT
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
@@ -377,6 +391,38 @@ int launch_skinny_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const
 // rounds: the tile count with the smallest rounds x bytes wins (384 row tiles as 192 workgroups of
 // two run in one round instead of two: 14.7 -> 11.2 us at M = 32, K = 4096).  Wider row blocks
 // lose to more row tiles on the same count.
+// row tiles per workgroup of the weight-streaming kernel (see launch_skinny)
+template <bool kW4>
+int skinny_row_tiles(int M, int N) {
+  const int ntiles = N / kTileN;
+  const int mblocks = (M + 31) / 32;
+  int nt = 1;
+  long long best = 0;
+  for (int c = 1; c <= 4; c *= 2) {
+    const long long wgs = (long long)((ntiles + c - 1) / c) * mblocks;
+    const int slots = (c == 4 && (ntiles / 4) * mblocks >= 512) ? 512 : 256;  // four-wave workgroups share a CU
+    const long long cost = ((wgs + slots - 1) / slots) * (64 + (kW4 ? 8 : 16) * c);
+    if (c == 1 || cost < best) {
+      best = cost;
+      nt = c;
+    }
+  }
+  return AJQ_SKINNY_FORCE_NT ? AJQ_SKINNY_FORCE_NT : nt;
+}
+
+// the same choice of configuration for the kernel's epilogue forms (row scale / residual / gate)
+template <bool kW4, int kEpi>
+int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                      int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  const int nt = skinny_row_tiles<kW4>(M, N);
+  const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
+  if (nt == 1) return launch_skinny_epi_cfg<8, 2, 32, 1, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if (nt == 2) return launch_skinny_epi_cfg<8, 1, 32, 2, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if ((ntiles / 4) * mblocks >= 512)
+    return launch_skinny_epi_cfg<4, 1, 32, 4, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  return launch_skinny_epi_cfg<8, 1, 32, 4, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+}
+
 template <bool kW4>
 int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
@@ -418,8 +464,10 @@ int launch_gemv_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, con
   return AJQ_OK;
 }
 
+constexpr int kMaxEpiM = 255;  // above the GEMV range the weight-streaming kernel carries the same epilogues
 bool gemv_epi_supported(int M, int K) {
-  if (M < 1 || M > kMaxGemvM) return false;
+  if (M < 1 || M > kMaxEpiM) return false;
+  if (M > kMaxGemvM) return K % kGroup == 0;
   if (K == 2048 || K == 4096) return true;
   return K == 5632 && M <= 8;
 }
@@ -427,6 +475,7 @@ bool gemv_epi_supported(int M, int K) {
 template <bool kW4, int kEpi>
 int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                     int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  if (M > kMaxGemvM) return launch_skinny_epi<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
 #define AJQ_EPI(W, T, R) return launch_gemv_epi_cfg<W, T, R, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
   if (K == 2048) {
     if (M <= 1) AJQ_EPI(8, 2, 1);
@@ -458,7 +507,7 @@ int gemv_rowscale(const char* name, const uint16_t* xt, const float* ssq, int pa
   if (int s = check_matmul_args(name, xt, M, K, wq, aux, N, y, out_dtype, kGroup)) return s;
   if (int s = check_epi(name, M, K)) return s;
   if (!ssq || !aligned16(ssq)) return fail(ssq ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq must be non-null and 16-byte aligned", name);
-  const int waves = K == 5632 ? 11 : 8;
+  const int waves = (M <= kMaxGemvM && K == 5632) ? 11 : 8;
   if (parts < 4 || parts % 4 != 0 || parts > waves * 32)
     return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, %d]", name, parts, waves * 32);
   if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);

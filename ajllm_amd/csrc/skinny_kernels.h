@@ -30,13 +30,18 @@ struct SkinnyBatch {
   uint32_t m[NT][TPW];
 };
 
-template <int kWaves, int TPW, int MROWS, int NT, bool kW4>
-__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_kernel(
+// kEpi: the epilogue forms of dequant_gemv_epi_kernel (row scale of an RMSNorm applied to the outputs,
+// residual add with the next norm's preparation, SwiGLU gate on interleaved rows) for more rows than a GEMV
+// takes; ssq_in is [M][parts], ssq_out [M][N / 16].
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi>
+__device__ __forceinline__ void dequant_skinny_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
-    const uint16_t* __restrict__ scales8) {  // W8: fp16 [N]; W4: unused
+    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
+    const GemvEpilogue& ep) {
   static_assert(MROWS % 16 == 0, "row block is a whole number of MFMA tiles");
+  static_assert(kEpi == 0 || MROWS == 32, "the epilogue forms lay their row sums out for 32-row blocks");
   constexpr int MB = MROWS / 16;
   constexpr int kSlice = TPW * kGroup;     // k extent of one batch of one wave
   constexpr int kStride = kSlice + 8;      // padded LDS row, bf16 elements
@@ -188,9 +193,29 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
     }
   };
 
+  // row scale: this wave's share of the sums of squares of the block's 32 rows (lane -> row lane & 31, the two
+  // half-waves take alternate 16-byte pieces), requested behind the first batch of weights, used at the end
+  constexpr int kShareLoads = 32 / kWaves;  // 2 * kWaves * kShareLoads pieces of four: up to 256 parts
+  float4 ssq_share[kShareLoads];
+  float* red2 = reinterpret_cast<float*>(reinterpret_cast<uint16_t*>(smem_raw) + kWaves * kRegion);  // [32][kWaves]
+  auto epilogue_loads = [&]() {
+    if (kEpi & kEpiRowScale) {
+      const int m = m0 + (lane & 31), half = lane >> 5;
+#pragma unroll
+      for (int u = 0; u < kShareLoads; ++u) {
+        const int j = wave * 2 + half + u * kWaves * 2;
+        const bool live = 4 * j < ep.parts && m < M;  // (idle lanes re-read the first 16 bytes)
+        const float4 t = *reinterpret_cast<const float4*>(ep.ssq_in + (live ? (size_t)m * ep.parts + 4 * j : 0));
+        ssq_share[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  if (g_begin >= g_end) epilogue_loads();
   if (g_begin < g_end) {
     Batch b0, b1;
     load(b0, g_begin);
+    epilogue_loads();
     for (int g0 = g_begin; g0 < g_end; g0 += 2 * TPW) {
       const bool has1 = g0 + TPW < g_end;
       if (has1) load(b1, g0 + TPW);
@@ -212,6 +237,13 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int r = 0; r < MB; ++r) mine[(t * MB + r) * 64 + lane] = acc[t][r];
+  if (kEpi & kEpiRowScale) {
+    float sh = 0.f;
+#pragma unroll
+    for (int u = 0; u < kShareLoads; ++u) sh += (ssq_share[u].x + ssq_share[u].y) + (ssq_share[u].z + ssq_share[u].w);
+    sh += __shfl_xor(sh, 32);
+    if (lane < 32) red2[lane * kWaves + wave] = sh;
+  }
   __syncthreads();
   for (int u = wave; u < NT * MB; u += kWaves) {
     const int t = u / MB, r = u % MB;
@@ -226,23 +258,78 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
     const int n = (nt0 + t) * kTileN + nl;
     float cs = 1.0f;
     if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
+    float rstd[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (kEpi & kEpiRowScale) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m0 + 16 * r + 4 * kc + i;
-      if (m < M) {
-        const float v = sum[i] * cs;
-        if (out_f32)
-          reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
-        else
-          reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+      for (int i = 0; i < 4; ++i) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) total += red2[(16 * r + 4 * kc + i) * kWaves + w];
+        rstd[i] = rsqrtf(total * ep.inv_k + ep.eps);
+      }
+    }
+    if (kEpi & kEpiResidual) {
+      const float gain_n = ep.gain[n];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 16 * r + 4 * kc + i;
+        float v = sum[i] * cs * rstd[i];
+        asm volatile("" : "+v"(v));  // no fused multiply-add: bit for bit the plain output, then the add
+        const float h = (m < M ? ep.h_in[(size_t)m * N + n] : 0.f) + v;
+        if (m < M) {
+          ep.h_out[(size_t)m * N + n] = h;
+          ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+        }
+        const float sq = team_sum16(m < M ? h * h : 0.f);
+        if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt0 + t] = sq;
+      }
+    } else if (kEpi & kEpiGate) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 16 * r + 4 * kc + i;
+        const float v = sum[i] * cs * rstd[i];
+        const float other = row_ror<8>(v);  // the lane 8 columns away
+        if (nl < 8 && m < M)
+          reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + (nt0 + t) * 8 + nl] =
+              f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 16 * r + 4 * kc + i;
+        if (m < M) {
+          const float v = sum[i] * cs * rstd[i];
+          if (out_f32)
+            reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
+          else
+            reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+        }
       }
     }
   }
 }
 
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4>
+__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8) {
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, 0>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
+}
+
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi>
+__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_epi_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, kEpi>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
+}
+
 // LDS bytes of one workgroup of dequant_skinny_kernel<kWaves, TPW, MROWS, *>
 constexpr size_t skinny_lds_bytes(int waves, int tpw, int mrows) {
   return (size_t)waves * mrows * (tpw * kGroup + 8) * 2;
+}
+// ... of dequant_skinny_epi_kernel: the 32 rows' sums of squares, one share per wave, behind the waves' regions
+constexpr size_t skinny_epi_lds_bytes(int waves, int tpw, int mrows) {
+  return skinny_lds_bytes(waves, tpw, mrows) + (size_t)32 * waves * 4;
 }
 
 }  // namespace ajq

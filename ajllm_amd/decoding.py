@@ -294,8 +294,9 @@ class FusedDecoder(GraphDecoder):
     and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), the greedy pick
     with the embedding lookup and the step counters (``ajq_greedy_pick``).  Five launches per layer
     at batch 1 (q|k|v with the norm, attention, output projection with the merge of the attention's
-    row chunks, w1|w3 with the norm, w2 with the gate: ``launches_per_step``); six at batch 5-16, where the norm's
-    row scale, the residual add and the gate ride in the GEMVs' epilogues; up to nine beyond.
+    row chunks, w1|w3 with the gate, w2: ``launches_per_step``); six above batch 4, where the attention's merge is a
+    launch of its own.  The norm's row scale, the residual add and the gate ride in the matmuls' epilogues (GEMV kernel
+    up to 16 rows, weight-streaming kernel up to 255); nine launches per layer where those forms are not built.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
@@ -384,7 +385,7 @@ class FusedDecoder(GraphDecoder):
             for w, layer in zip(self.layers, model.layers):
                 w["w13i"] = _FusedLinear.interleaved_gate(layer.feed_forward.w1, layer.feed_forward.w3)
             self.xt = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
-            self.ssq = torch.zeros((16, d // 16), dtype=torch.float32, device=dev)
+            self.ssq = torch.zeros((max(16, batch), d // 16), dtype=torch.float32, device=dev)
         self.normed = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.attended = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)
         self.gated = torch.zeros((batch, self.d_ff), dtype=torch.bfloat16, device=dev)

@@ -137,7 +137,7 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
  *     h_out = h_in + x W1^T ;   y = (RMSNorm(h_out) * gain) W2^T
  * in two launches, without a norm kernel between them:
  *   _residual: h_out[M, N] = h_in + x W^T (fp32; h_out must not be h_in), xt_out = bf16(h_out * gain)
- *              (gain[N]: of the norm that follows) and ssq_out[16][N / 16]: per row, the sum of squares of
+ *              (gain[N]: of the norm that follows) and ssq_out[max(16, M)][N / 16]: per row, the sum of squares of
  *              h_out over each 16-column tile (rows >= M are not written);
  *   _rowscale: y = rstd[m] * (xt W^T) with rstd[m] = rsqrt(sum(ssq[m][0 .. parts)) / K + eps), ssq laid out
  *              [16][parts] as _residual leaves it (parts = K / 16; a multiple of 4, at most 256, 352 for
@@ -147,7 +147,8 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
  * xt is rounded to bf16 BEFORE the row scale is applied (the reference order rounds the normalised value);
  * both are one bf16 rounding of the same quantity up to the fp32 factor rstd.  Sums run in a fixed order:
  * results are run-to-run identical.  Built for the (M, K) that ajq_gemv_epilogue_supported reports: M <= 16
- * with K = 2048 or 4096, M <= 8 with K = 5632; AJQ_ERR_UNSUPPORTED otherwise. */
+ * with K = 2048 or 4096, M <= 8 with K = 5632 (the GEMV kernel), and 17 <= M <= 255 with any K % 128 == 0 (the
+ * weight-streaming kernel; ssq then has M rows instead of 16); AJQ_ERR_UNSUPPORTED otherwise. */
 int ajq_gemv_epilogue_supported(int M, int K);
 int ajq_w4a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                             const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,

@@ -687,7 +687,8 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
 
 
 @pytest.mark.parametrize("scheme,batch,d_ff", [("w4a16_g128", 8, 5632), ("w8a16", 13, 2048), ("w4a16_g128", 5, 4096),
-                                               ("w4a16_g128", 1, 5632), ("w8a16", 4, 2048), ("w4a16_g128", 2, 4096)])
+                                               ("w4a16_g128", 1, 5632), ("w8a16", 4, 2048), ("w4a16_g128", 2, 4096),
+                                               ("w8a16", 20, 2048), ("w4a16_g128", 33, 5632)])
 def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff):
     """Widths the epilogue GEMVs are built for (d_model 2048): no norm, gate or residual launch inside a layer
     (the norm's row scale is applied to the matmul outputs, the residual add and the next norm's preparation
