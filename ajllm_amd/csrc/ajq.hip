@@ -465,17 +465,16 @@ int launch_gemv_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, con
 }
 
 constexpr int kMaxEpiM = 255;  // above the GEMV range the weight-streaming kernel carries the same epilogues
-bool gemv_epi_supported(int M, int K) {
-  if (M < 1 || M > kMaxEpiM) return false;
-  if (M > kMaxGemvM) return K % kGroup == 0;
-  if (K == 2048 || K == 4096) return true;
-  return K == 5632 && M <= 8;
+// whether the GEMV kernel's straight-line configurations take (M, K); everything else goes to the streaming kernel
+bool gemv_epi_straight(int M, int K) {
+  return M <= kMaxGemvM && (K == 2048 || K == 4096 || (K == 5632 && M <= 8));
 }
+bool gemv_epi_supported(int M, int K) { return M >= 1 && M <= kMaxEpiM && K >= kGroup && K % kGroup == 0; }
 
 template <bool kW4, int kEpi>
 int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                     int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
-  if (M > kMaxGemvM) return launch_skinny_epi<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if (!gemv_epi_straight(M, K)) return launch_skinny_epi<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
 #define AJQ_EPI(W, T, R) return launch_gemv_epi_cfg<W, T, R, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
   if (K == 2048) {
     if (M <= 1) AJQ_EPI(8, 2, 1);
@@ -507,7 +506,7 @@ int gemv_rowscale(const char* name, const uint16_t* xt, const float* ssq, int pa
   if (int s = check_matmul_args(name, xt, M, K, wq, aux, N, y, out_dtype, kGroup)) return s;
   if (int s = check_epi(name, M, K)) return s;
   if (!ssq || !aligned16(ssq)) return fail(ssq ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq must be non-null and 16-byte aligned", name);
-  const int waves = (M <= kMaxGemvM && K == 5632) ? 11 : 8;
+  const int waves = (gemv_epi_straight(M, K) && K == 5632) ? 11 : 8;
   if (parts < 4 || parts % 4 != 0 || parts > waves * 32)
     return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, %d]", name, parts, waves * 32);
   if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);

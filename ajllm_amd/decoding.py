@@ -370,11 +370,10 @@ class FusedDecoder(GraphDecoder):
         # is applied to the OUTPUTS of q|k|v, w1|w3 and the head instead, the output projection and w2 add
         # the residual and prepare the next norm on their way out, and w1|w3 (rows interleaved in blocks
         # of 8) applies the gate: six launches per layer instead of nine.
-        # At small batch as well, provided the output projection can merge the attention's row chunks on its way
-        # in (five launches per layer either way, and the epilogue forms cost less than the prologue forms:
-        # 3.9 against 4.8 us for q|k|v at batch 1, 4.3 against 6.7 at batch 4).
+        # At small batch as well: the epilogue forms cost less than the prologue forms (3.3 against 4.8 us for
+        # q|k|v at batch 1, 4.2 against 6.7 at batch 4).
         self.fuse_epilogue = (
-            (batch > 4 or self.fuse_merge) and self.d_ff % 8 == 0 and d // 16 <= 256
+            self.d_ff % 8 == 0 and d // 16 <= 256
             and self.layers[0]["o"].in_features == d
             and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
             and self.head.epilogue_fusable(batch)
@@ -382,6 +381,10 @@ class FusedDecoder(GraphDecoder):
         if self.fuse_epilogue:
             self.first_norm_fused = self.fuse_norm   # the step's very first norm rides in layer 0's q|k|v where built
             self.fuse_norm = self.fuse_gate = False
+            # the merge prologue re-reads every chunk of every head in every workgroup: with the cheaper epilogue
+            # kernels around it, it only pays at batch 1 (measured: 0.41 / 0.50 / 0.52 ms per step with it at
+            # batch 2 / 3 / 4 against 0.41 / 0.45 / 0.48 with the merge as a launch of its own)
+            self.fuse_merge = self.fuse_merge and batch == 1
             for w, layer in zip(self.layers, model.layers):
                 w["w13i"] = _FusedLinear.interleaved_gate(layer.feed_forward.w1, layer.feed_forward.w3)
             self.xt = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)

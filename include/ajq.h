@@ -146,9 +146,9 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
  *              y[M, N / 2] = bf16(silu(a) * u), out_dtype AJQ_OUT_BF16.
  * xt is rounded to bf16 BEFORE the row scale is applied (the reference order rounds the normalised value);
  * both are one bf16 rounding of the same quantity up to the fp32 factor rstd.  Sums run in a fixed order:
- * results are run-to-run identical.  Built for the (M, K) that ajq_gemv_epilogue_supported reports: M <= 16
- * with K = 2048 or 4096, M <= 8 with K = 5632 (the GEMV kernel), and 17 <= M <= 255 with any K % 128 == 0 (the
- * weight-streaming kernel; ssq then has M rows instead of 16); AJQ_ERR_UNSUPPORTED otherwise. */
+ * results are run-to-run identical.  Built for the (M, K) that ajq_gemv_epilogue_supported reports: 1 <= M <= 255,
+ * K % 128 == 0 (the GEMV kernel for M <= 16 with K = 2048 or 4096 and M <= 8 with K = 5632, the weight-streaming
+ * kernel otherwise; ssq has max(16, M) rows); AJQ_ERR_UNSUPPORTED otherwise. */
 int ajq_gemv_epilogue_supported(int M, int K);
 int ajq_w4a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                             const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,

@@ -92,12 +92,11 @@ def test_shape_alignment_and_option_errors():
     need = lib.ajq_w4a16_gemm_workspace_bytes(2048, 4096)                    # a shape the tile kernel takes
     assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, None, 0, None) == -6
     assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, p, need - 1, None) == -6
-    # GEMVs with a residual / row-scale / gate epilogue: which (M, K) are built, and what is refused before any launch
+    # matmuls with a residual / row-scale / gate epilogue: which (M, K) are built, and what is refused before any launch
     assert lib.ajq_gemv_epilogue_supported(1, 2048) == 1 and lib.ajq_gemv_epilogue_supported(16, 4096) == 1
-    assert lib.ajq_gemv_epilogue_supported(8, 5632) == 1 and lib.ajq_gemv_epilogue_supported(9, 5632) == 0
-    assert lib.ajq_gemv_epilogue_supported(17, 2048) == 1 and lib.ajq_gemv_epilogue_supported(200, 14336) == 1   # streaming kernel
-    assert lib.ajq_gemv_epilogue_supported(256, 2048) == 0 and lib.ajq_gemv_epilogue_supported(1, 1024) == 0
-    assert lib.ajq_w4a16_gemv_rowscale(p, p, 128, 1e-5, 4, 1024, p, p, 16, p, 0, 0, None) == -4   # K = 1024 is not built
+    assert lib.ajq_gemv_epilogue_supported(9, 5632) == 1 and lib.ajq_gemv_epilogue_supported(200, 14336) == 1   # streaming kernel
+    assert lib.ajq_gemv_epilogue_supported(256, 2048) == 0 and lib.ajq_gemv_epilogue_supported(4, 1000) == 0
+    assert lib.ajq_w4a16_gemv_rowscale(p, p, 128, 1e-5, 300, 2048, p, p, 16, p, 0, 0, None) == -4   # more rows than built
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 130, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2   # parts not a multiple of 4
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 260, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2   # more parts than the waves cover
     assert lib.ajq_w4a16_gemv_rowscale(p, None, 128, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -1
