@@ -529,7 +529,7 @@ int gemv_residual(const char* name, const uint16_t* x, int M, int K, const uint3
                          const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out, void* stream) {
   if (int s = check_matmul_args(name, x, M, K, wq, aux, N, h_out, AJQ_OUT_F32, kGroup)) return s;
   if (int s = check_epi(name, M, K)) return s;
-  if (!h_in || !gain || !xt_out || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (!h_in || !gain || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
   if (h_in == h_out) return fail(AJQ_ERR_NULL, "%s: h_out must be a buffer other than h_in", name);
   GemvEpilogue ep{};
   ep.h_in = h_in;
@@ -544,13 +544,13 @@ int gemv_residual(const char* name, const uint16_t* x, int M, int K, const uint3
 }
 
 // ---- GEMV with the activations produced on the way in (norm / gate prologue)
-template <int kWaves, int TPW, int MROWS, bool kW4, int kPro>
+template <int kWaves, int TPW, int MROWS, bool kW4, int kPro, int kOut = 0>
 int launch_gemv_pro_cfg(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
                         int out_f32, const float* src0, const float* src1, const float* gain, float eps, float* h_out,
                         hipStream_t stream, int S = 0) {
   constexpr size_t lds = gemv_pro_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_gemv_pro_kernel<kWaves, TPW, MROWS, kW4, kPro>;
+  auto kernel = dequant_gemv_pro_kernel<kWaves, TPW, MROWS, kW4, kPro, kOut>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
                      meta, K, M | (out_f32 << 8), N, y, scales8, src0, src1, gain, eps, h_out, S, nullptr, nullptr, nullptr);
@@ -563,7 +563,7 @@ int launch_gemv_merge_resid_cfg(int M, int K, const uint32_t* wq, const uint32_t
                                 const float* partial, int S, const float* h_in, const float* gain, float* h_out,
                                 uint16_t* xt, float* ssq, hipStream_t stream) {
   constexpr size_t lds = gemv_pro_lds_bytes(8, TPW, MROWS);
-  auto kernel = dequant_gemv_pro_kernel<8, TPW, MROWS, kW4, kProMerge, true>;
+  auto kernel = dequant_gemv_pro_kernel<8, TPW, MROWS, kW4, kProMerge, kOutResid>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(8 * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, K,
                      M | (1 << 8), N, nullptr, scales8, partial, nullptr, gain, 0.f, h_out, S, h_in, xt, ssq);
@@ -580,12 +580,13 @@ bool gemv_pro_supported(int M, int K) {
   return false;
 }
 
-template <bool kW4, int kPro>
+template <bool kW4, int kPro, int kOut = 0>
 int launch_gemv_pro(int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8, int N, void* y,
                     int out_f32, const float* src0, const float* src1, const float* gain, float eps, float* h_out,
-                    hipStream_t stream) {
-#define AJQ_PRO(W, T, R) \
-  return launch_gemv_pro_cfg<W, T, R, kW4, kPro>(M, K, wq, meta, scales8, N, y, out_f32, src0, src1, gain, eps, h_out, stream)
+                    hipStream_t stream, int S = 0) {
+#define AJQ_PRO(W, T, R)                                                                                              \
+  return launch_gemv_pro_cfg<W, T, R, kW4, kPro, kOut>(M, K, wq, meta, scales8, N, y, out_f32, src0, src1, gain, eps, \
+                                                       h_out, stream, S)
   if (K == 1024) {
     if (M <= 1) AJQ_PRO(8, 1, 1);
     if (M <= 4) AJQ_PRO(8, 1, 4);
@@ -660,13 +661,34 @@ int gemv_merge_residual(const char* name, const float* partial, int S, int M, in
   const int cap = gemv_merge_max_splits(M, K);
   if (cap == 0 || S < 1 || S > cap)
     return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d, S=%d is not built (ajq_gemv_merge_max_splits gives %d)", name, M, K, S, cap);
-  if (!h_in || !gain || !xt_out || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
+  if (!h_in || !gain || !ssq_out) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
   if (h_in == h_out) return fail(AJQ_ERR_NULL, "%s: h_out must be a buffer other than h_in", name);
   const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
   const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
   if (int s = launch_gemv_merge_resid<kW4>(M, K, wq, meta, scales, N, partial, S, h_in, gain, h_out, xt_out, ssq_out,
                                            (hipStream_t)stream))
     return s;
+  return check_launch(name);
+}
+
+template <bool kW4>
+int gemv_norm_sums(const char* name, const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
+                   const uint32_t* wq, const void* aux, int N, void* y, int out_dtype, int gate, void* stream) {
+  if (int s = check_matmul_args(name, h, M, K, wq, aux, N, y, out_dtype, kGroup)) return s;
+  if (!gemv_pro_supported(M, K))
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d is not built (ajq_gemv_fused_supported)", name, M, K);
+  if (!ssq || !gain || !aligned16(ssq) || !aligned16(gain))
+    return fail(ssq && gain ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq and gain must be non-null and 16-byte aligned", name);
+  if (parts < 4 || parts % 4 != 0 || parts > 256)
+    return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, 256]", name, parts);
+  if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);
+  const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
+  const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
+  const int s = gate ? launch_gemv_pro<kW4, kProNormSums, kOutGate>(M, K, wq, meta, scales, N, y, 0, h, ssq, gain, eps, nullptr,
+                                                                    (hipStream_t)stream, parts)
+                     : launch_gemv_pro<kW4, kProNormSums>(M, K, wq, meta, scales, N, y, out_dtype == AJQ_OUT_F32, h, ssq, gain,
+                                                          eps, nullptr, (hipStream_t)stream, parts);
+  if (s) return s;
   return check_launch(name);
 }
 
@@ -731,6 +753,20 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1 : 0; }
 
 int ajq_gemv_epilogue_supported(int M, int K) { return gemv_epi_supported(M, K) ? 1 : 0; }
+
+int ajq_w4a16_gemv_norm_sums(const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
+                             const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, int gate,
+                             void* stream) {
+  return gemv_norm_sums<true>("ajq_w4a16_gemv_norm_sums", h, ssq, parts, gain, eps, M, K, wq, meta, N, y, out_dtype, gate,
+                              stream);
+}
+
+int ajq_w8a16_gemv_norm_sums(const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
+                             const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
+                             void* stream) {
+  return gemv_norm_sums<false>("ajq_w8a16_gemv_norm_sums", h, ssq, parts, gain, eps, M, K, wq, scales, N, y, out_dtype, gate,
+                               stream);
+}
 
 int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K, const uint32_t* wq,
                             const uint32_t* meta, int N, void* y, int out_dtype, int gate, void* stream) {

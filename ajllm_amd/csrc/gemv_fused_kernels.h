@@ -23,17 +23,24 @@
 
 namespace ajq {
 
-constexpr int kProNorm = 1, kProGate = 2, kProMerge = 3;
+constexpr int kProNorm = 1, kProGate = 2, kProMerge = 3, kProNormSums = 4;
+// kProNormSums: x = bf16( (h / rms) * gain ) as kProNorm forms it, with rms taken from sums of squares that the
+// PRODUCER of h left behind (src1 = ssq[rows][parts], per row the sums over 16-column tiles; S = parts): nothing
+// is added to h, no workgroup barrier sits in front of the matmul (a wave adds the parts of its rows itself), and the
+// activations are rounded exactly where the separate norm kernel rounds them.
+// kOut: 0 plain output; kOutResid the residual epilogue (see dequant_gemv_epi_kernel); kOutGate the SwiGLU gate on
+// rows interleaved in blocks of 8, y = bf16 [M, N / 2].
+constexpr int kOutResid = 1, kOutGate = 2;
 
 // chunks of one (row, head) a lane of the merge prologue takes (the 4 lane quarters take every 4th chunk)
 constexpr int merge_chunks_per_lane(int mrows, int tpw) {
   return 8 / (mrows * tpw) > 4 ? 4 : (8 / (mrows * tpw) < 1 ? 1 : 8 / (mrows * tpw));
 }
 
-// kResid (with the merge prologue): the output side of dequant_gemv_epi_kernel's kEpiResidual as well:
-// h_out = res_h_in + (x W^T), res_xt = bf16(h_out * gain) for the norm that follows, res_ssq[m][tile] the
-// sum of squares of h_out over this workgroup's 16 columns; y is not written.
-template <int kWaves, int TPW, int MROWS, bool kW4, int kPro, bool kResid = false>
+// kOutResid (with the merge prologue): h_out = res_h_in + (x W^T), res_xt = bf16(h_out * gain) for the norm that
+// follows (skipped if null), res_ssq[m][tile] the sum of squares of h_out over this workgroup's 16 columns; y is
+// not written.
+template <int kWaves, int TPW, int MROWS, bool kW4, int kPro, int kOut = 0>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -100,11 +107,11 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     const int v = min(lane + 64 * i, kVecs - 1);
     const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
     const int k = g0 * kGroup + 8 * c;
-    if (kPro == kProNorm) {
+    if (kPro == kProNorm || kPro == kProNormSums) {
       const float4* ph = reinterpret_cast<const float4*>(src0 + (size_t)m * K + k);
       a0[i][0] = ph[0];
       a0[i][1] = ph[1];
-      if (src1) {
+      if (kPro == kProNorm && src1) {
         const float4* pd = reinterpret_cast<const float4*>(src1 + (size_t)m * K + k);
         a1[i][0] = pd[0];
         a1[i][1] = pd[1];
@@ -123,6 +130,20 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       a1[i][1] = pu[1];
     }
   }
+  // kProNormSums: the 64 / MROWS lanes of a row share the parts of its sum of squares
+  constexpr int kLanesPerRow = 64 / MROWS;
+  constexpr int kPartLoads = kPro == kProNormSums ? (64 + kLanesPerRow - 1) / kLanesPerRow : 1;  // up to 256 parts
+  float4 sums[kPartLoads];
+  if (kPro == kProNormSums) {
+    const int row = lane / kLanesPerRow, piece = lane % kLanesPerRow;
+#pragma unroll
+    for (int u = 0; u < kPartLoads; ++u) {
+      const int j = piece + u * kLanesPerRow;
+      const bool live = 4 * j < S && row < M;  // (idle lanes re-read the first 16 bytes)
+      const float4 t = *reinterpret_cast<const float4*>(src1 + (live ? (size_t)row * S + 4 * j : 0));
+      sums[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
   {
     const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
 #pragma unroll
@@ -136,6 +157,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
 #pragma unroll
     for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
   }
+  constexpr bool kResid = kOut == kOutResid;
   constexpr int kLiveRows = MROWS < 4 ? MROWS : 4;
   float h_old[kLiveRows], gain_n = 0.f;
   if (kResid) {  // behind the weights in issue order, used at the very end
@@ -181,6 +203,24 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       xv[i][2] = (xv[i][2] / rms) * g0v.z; xv[i][3] = (xv[i][3] / rms) * g0v.w;
       xv[i][4] = (xv[i][4] / rms) * g1v.x; xv[i][5] = (xv[i][5] / rms) * g1v.y;
       xv[i][6] = (xv[i][6] / rms) * g1v.z; xv[i][7] = (xv[i][7] / rms) * g1v.w;
+    }
+  } else if (kPro == kProNormSums) {
+    // a row's total in its first lane, then through the wave's own LDS words to whoever holds a piece of the row
+    float total = 0.f;
+#pragma unroll
+    for (int u = 0; u < kPartLoads; ++u) total += (sums[u].x + sums[u].y) + (sums[u].z + sums[u].w);
+#pragma unroll
+    for (int off = kLanesPerRow / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    if (lane % kLanesPerRow == 0) ssq[(lane / kLanesPerRow) * kWaves + wave] = total;
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = min(lane + 64 * i, kVecs - 1);
+      const float rms = sqrtf(ssq[(v / kVecPerRow) * kWaves + wave] / (float)K + eps);
+      const float4 h0 = a0[i][0], h1 = a0[i][1], g0v = a2[i][0], g1v = a2[i][1];
+      xv[i][0] = (h0.x / rms) * g0v.x; xv[i][1] = (h0.y / rms) * g0v.y;
+      xv[i][2] = (h0.z / rms) * g0v.z; xv[i][3] = (h0.w / rms) * g0v.w;
+      xv[i][4] = (h1.x / rms) * g1v.x; xv[i][5] = (h1.y / rms) * g1v.y;
+      xv[i][6] = (h1.z / rms) * g1v.z; xv[i][7] = (h1.w / rms) * g1v.w;
     }
   } else if (kPro == kProGate) {
 #pragma unroll
@@ -312,10 +352,23 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       const float h = h_old[i] + v;
       if (m < M) {
         h_out[(size_t)m * N + n] = h;
-        res_xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+        if (res_xt) res_xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
       }
       const float sq = team_sum16(m < M ? h * h : 0.f);
       if (nl == 0 && m < M) res_ssq[(size_t)m * ntiles + nt] = sq;
+    }
+    return;
+  }
+  if (kOut == kOutGate) {
+    // columns 0..7 of the tile are gate projections, 8..15 the matching up projections
+#pragma unroll
+    for (int i = 0; i < kLive; ++i) {
+      const int m = 4 * kc + i;
+      const float v = sum[i] * cs;
+      const float other = row_ror<8>(v);  // the lane 8 columns away
+      if (nl < 8 && m < M)
+        reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + nt * 8 + nl] =
+            f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);
     }
     return;
   }

@@ -291,7 +291,7 @@ __device__ __forceinline__ void dequant_gemv_body(
       const float h = h_old[i] + v;
       if (m < M) {
         ep.h_out[(size_t)m * N + n] = h;
-        ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+        if (ep.xt) ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
       }
       const float sq = team_sum16(m < M ? h * h : 0.f);  // over the tile's 16 columns (one DPP row)
       if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt] = sq;

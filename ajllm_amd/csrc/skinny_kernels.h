@@ -278,7 +278,7 @@ __device__ __forceinline__ void dequant_skinny_body(
         const float h = (m < M ? ep.h_in[(size_t)m * N + n] : 0.f) + v;
         if (m < M) {
           ep.h_out[(size_t)m * N + n] = h;
-          ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+          if (ep.xt) ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
         }
         const float sq = team_sum16(m < M ? h * h : 0.f);
         if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt0 + t] = sq;

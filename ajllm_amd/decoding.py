@@ -213,24 +213,42 @@ class _FusedLinear:
         return bool(_lib.load().ajq_gemv_epilogue_supported(batch, self.in_features))
 
     def residual(self, x_bf16: torch.Tensor, h_in: torch.Tensor, gain: torch.Tensor, h_out: torch.Tensor,
-                 xt: torch.Tensor, ssq: torch.Tensor) -> None:
-        """``h_out = h_in + self(x)``, ``xt = bf16(h_out * gain)`` and the per-tile sums of squares of
-        ``h_out`` in ``ssq`` (what the next ``rowscaled`` needs in place of a norm), one launch."""
+                 xt: torch.Tensor | None, ssq: torch.Tensor) -> None:
+        """``h_out = h_in + self(x)``, ``xt = bf16(h_out * gain)`` (skipped if None) and the per-tile sums of squares
+        of ``h_out`` in ``ssq`` (what the next ``normed_from_sums`` / ``rowscaled`` needs in place of a norm), one launch."""
         lib = _lib.load()
         fn = lib.ajq_w8a16_gemv_residual if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_residual
         _lib.check(fn(x_bf16.data_ptr(), x_bf16.shape[0], self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
-                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(),
-                      _stream()), "gemv_residual")
+                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(),
+                      xt.data_ptr() if xt is not None else None, ssq.data_ptr(), _stream()), "gemv_residual")
 
     def merge_residual(self, partial: torch.Tensor, splits: int, rows: int, h_in: torch.Tensor, gain: torch.Tensor,
-                       h_out: torch.Tensor, xt: torch.Tensor, ssq: torch.Tensor) -> None:
+                       h_out: torch.Tensor, xt: torch.Tensor | None, ssq: torch.Tensor) -> None:
         """``residual`` whose input is the attention output merged from ``splits`` partial results per (row, head) on
         the way in (as ``after_merge``), one launch."""
         lib = _lib.load()
         fn = lib.ajq_w8a16_gemv_merge_residual if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_merge_residual
         _lib.check(fn(partial.data_ptr(), splits, rows, self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
-                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(),
-                      _stream()), "gemv_merge_residual")
+                      self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(),
+                      xt.data_ptr() if xt is not None else None, ssq.data_ptr(), _stream()), "gemv_merge_residual")
+
+    def normed_from_sums(self, h: torch.Tensor, ssq: torch.Tensor, gain: torch.Tensor, eps: float,
+                         gated: torch.Tensor | None = None) -> torch.Tensor:
+        """``self(bf16(RMSNorm(h) * gain))`` with the norm's sums of squares taken from what ``residual`` left in
+        ``ssq``: the activations are rounded exactly where a separate norm kernel rounds them.  One launch; ``gated``
+        as in ``rowscaled``."""
+        lib = _lib.load()
+        rows = h.shape[0]
+        fn = lib.ajq_w8a16_gemv_norm_sums if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_norm_sums
+        if gated is None:
+            y = torch.empty((rows, self.rows16), dtype=torch.float32, device=h.device)
+            dtype, gate = _lib.AJQ_OUT_F32, 0
+        else:
+            y, dtype, gate = gated, _lib.AJQ_OUT_BF16, 1
+        _lib.check(fn(h.data_ptr(), ssq.data_ptr(), ssq.shape[1], gain.data_ptr(), eps, rows, self.in_features,
+                      self.wq.data_ptr(), self.meta.data_ptr(), self.rows16, y.data_ptr(), dtype, gate, _stream()),
+                   "gemv_norm_sums")
+        return y
 
     def rowscaled(self, xt: torch.Tensor, ssq: torch.Tensor, eps: float, gated: torch.Tensor | None = None) -> torch.Tensor:
         """``self(RMSNorm(h) * gain)`` from ``xt = bf16(h * gain)`` and the sums of squares ``residual`` left,
@@ -304,8 +322,10 @@ class FusedDecoder(GraphDecoder):
     torch.bfloat16 (keys and values rounded to nearest even on write, half the cache traffic)."""
 
     def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int,
-                 kv_dtype: torch.dtype | None = None) -> None:
+                 kv_dtype: torch.dtype | None = None, activation_rounding: str = "reference") -> None:
         super().__init__(model, batch, max_len, kv_dtype)
+        if activation_rounding not in ("reference", "before_scale"):
+            raise ValueError('activation_rounding must be "reference" or "before_scale"')
         cache_dtype = self.cache.keys[0].dtype
         if cache_dtype not in (torch.float32, torch.bfloat16):
             raise ValueError("the KV cache must be float32 or bfloat16")
@@ -372,8 +392,20 @@ class FusedDecoder(GraphDecoder):
         # of 8) applies the gate: six launches per layer instead of nine.
         # At small batch as well: the epilogue forms cost less than the prologue forms (3.3 against 4.8 us for
         # q|k|v at batch 1, 4.2 against 6.7 at batch 4).
+        # Where the normed activations are rounded to bf16.  "reference": exactly where the model code rounds them,
+        # bf16((h / rms) * gain) (the consumer is the GEMV with a norm prologue, fed with the producer's sums of
+        # squares; built for the batches and widths ``fusable`` reports).  "before_scale": bf16(h * gain), the row
+        # scale applied to the matmul's outputs (one rounding of the same quantity at a different point: the
+        # logits move by about as much again as bf16 activations move them at all); built for every batch.
+        # The reference-order consumer reads the fp32 stream of all batch rows in every workgroup, like any prologue
+        # form: measured on the 12-layer model it beats the unfolded step up to batch 4 (0.37 / 0.46 / 0.45 / 0.53 ms
+        # against 0.38 / 0.51 / 0.60 / 0.62 at batch 1 - 4) and loses from batch 5 (0.63 against 0.53), so above
+        # batch 4 "reference" means the unfolded step; "before_scale" folds at every batch (0.34 / 0.42 / 0.60 ms at
+        # batch 1 / 4 / 8).
+        self.exact_norm = activation_rounding == "reference"
+        rounding_built = (batch <= 4 and self.head.fusable(batch)) if self.exact_norm else True
         self.fuse_epilogue = (
-            self.d_ff % 8 == 0 and d // 16 <= 256
+            rounding_built and self.d_ff % 8 == 0 and d // 16 <= 256
             and self.layers[0]["o"].in_features == d
             and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
             and self.head.epilogue_fusable(batch)
@@ -567,9 +599,17 @@ class FusedDecoder(GraphDecoder):
         def other() -> torch.Tensor:
             return self.hidden2 if cur is self.hidden else self.hidden
 
+        xt = None if self.exact_norm else self.xt   # the producers' bf16 image is only read by the row-scale form
+
+        def normed(linear: _FusedLinear, gain: torch.Tensor, eps: float, gated: torch.Tensor | None = None) -> torch.Tensor:
+            """linear(RMSNorm(cur) * gain), the norm taken from the sums of squares cur's producer left."""
+            if self.exact_norm:
+                return linear.normed_from_sums(cur, self.ssq, gain, eps, gated)
+            return linear.rowscaled(self.xt, self.ssq, eps, gated)
+
         for index, w in enumerate(self.layers):
             if index > 0:
-                qkv = w["qkv"].rowscaled(self.xt, self.ssq, w["eps1"])
+                qkv = normed(w["qkv"], w["g1"], w["eps1"])
             elif self.first_norm_fused:
                 qkv = w["qkv"].after_norm(self.embedded, None, first["g1"], first["eps1"], self.hidden)
                 cur = self.hidden  # (a copy of the embedding row)
@@ -586,17 +626,17 @@ class FusedDecoder(GraphDecoder):
                                                      self.kv_heads, 128, self.max_len, self.merge_splits,
                                                      ctypes.addressof(splits), self.attn_ws.data_ptr(),
                                                      self.attn_ws_bytes, st), "attn_step_partial")
-                w["o"].merge_residual(self.attn_ws, splits.value, b, cur, w["g2"], nxt, self.xt, self.ssq)
+                w["o"].merge_residual(self.attn_ws, splits.value, b, cur, w["g2"], nxt, xt, self.ssq)
             else:
                 self._attention(index, w, qkv)
-                w["o"].residual(self.attended, cur, w["g2"], nxt, self.xt, self.ssq)
+                w["o"].residual(self.attended, cur, w["g2"], nxt, xt, self.ssq)
             cur = nxt
-            w["w13i"].rowscaled(self.xt, self.ssq, w["eps2"], gated=self.gated)
+            normed(w["w13i"], w["g2"], w["eps2"], gated=self.gated)
             nxt = other()
             gain = self.layers[index + 1]["g1"] if index + 1 < len(self.layers) else self.final_gain
-            w["w2"].residual(self.gated, cur, gain, nxt, self.xt, self.ssq)
+            w["w2"].residual(self.gated, cur, gain, nxt, xt, self.ssq)
             cur = nxt
-        self.logits_full = self.head.rowscaled(self.xt, self.ssq, self.final_eps)
+        self.logits_full = normed(self.head, self.final_gain, self.final_eps)
         return self.logits_full[:, : self.vocab]
 
 

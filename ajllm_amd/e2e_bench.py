@@ -109,6 +109,20 @@ def bench_decode_short(device, log=print, batches=(1, 8), scheme: str = "w4a16_g
         torch.cuda.synchronize()
         t_bf16 = time.perf_counter() - t0
         r["bf16_kv_cache"] = {"decode_tok/s": batch * steps / t_bf16, "ms_per_step": t_bf16 / steps * 1e3}
+        # the decoder's faster folding: normed activations rounded to bf16 BEFORE the norm's row scale, which is then
+        # applied to the matmul outputs (fp32 cache; not the reference's rounding point)
+        del dec
+        dec = decoding.FusedDecoder(model, batch, PROMPT_LEN + NEW_TOKENS, activation_rounding="before_scale")
+        dec.prefill(prompt, fused=True)
+        dec.generate(8)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.generate(NEW_TOKENS)
+        torch.cuda.synchronize()
+        t_fold = time.perf_counter() - t0
+        r["activations_rounded_before_norm_scale"] = {"decode_tok/s": batch * steps / t_fold,
+                                                      "ms_per_step": t_fold / steps * 1e3,
+                                                      "launches_per_step": dec.launches_per_step()}
         log("decode", r)
         results.append(r)
         del dec

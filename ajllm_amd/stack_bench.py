@@ -189,5 +189,19 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
         torch.cuda.synchronize()
         t16 = (time.perf_counter() - t0) / decode_steps
         result["decode_bf16_kv_cache"] = {"ms_per_step": t16 * 1e3, "tok/s": batch / t16}
+        # the decoder's folded step (norms, residual adds and the gate in the matmuls' epilogues, six launches per
+        # layer; the normed activations are rounded to bf16 before the norm's row scale), fp32 cache
+        del dec16
+        torch.cuda.empty_cache()
+        decf = decoding.FusedDecoder(model, batch, context + decode_steps + 8, activation_rounding="before_scale")
+        decf.prefill(prompt, rows_per_pass=PREFILL_ROWS, fused=True)
+        decf.generate(4)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        decf.generate(4 + decode_steps)
+        torch.cuda.synchronize()
+        tf = (time.perf_counter() - t0) / decode_steps
+        result["decode_activations_rounded_before_norm_scale"] = {"ms_per_step": tf * 1e3, "tok/s": batch / tf,
+                                                                  "launches_per_step": decf.launches_per_step()}
     log("stack", result)
     return result

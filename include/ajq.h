@@ -162,6 +162,18 @@ int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, flo
 int ajq_w8a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
                             const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
                             void* stream);
+/*   _norm_sums: y = (RMSNorm(h) * gain) W^T with the activations rounded exactly where the reference rounds them,
+ *              bf16((h / rms) * gain) (layers.py:70-74 then the bf16 input of the quantized linear), rms taken from
+ *              the sums of squares that _residual left in ssq ([rows][parts], parts = K / 16 <= 256): the GEMV with a
+ *              norm prologue (ajq_w*a16_gemv_norm) without the add, without the reduction and without its
+ *              workgroup barrier.  h is _residual's h_out (fp32 [M, K]); gate as in _rowscale.  Built for the (M, K)
+ *              of ajq_gemv_fused_supported.  _residual's xt_out may be NULL when only this consumer follows. */
+int ajq_w4a16_gemv_norm_sums(const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
+                             const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, int gate,
+                             void* stream);
+int ajq_w8a16_gemv_norm_sums(const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
+                             const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
+                             void* stream);
 /*   _merge_residual: _residual whose x is the single-query attention output merged from the S partial results
  *              per (row, head) in ajq_attn_step_partial's workspace, as in _merge below (same limits:
  *              ajq_gemv_merge_max_splits): the output projection of a decode step at small batch, with the

@@ -439,6 +439,26 @@ def test_gemv_residual_then_rowscale_against_the_oracle(cuda, scheme, m, k1, d, 
     # (two independent bf16 roundings of every activation: 2^-9 / sqrt(3) each, relative, which does not
     # average out over K; the bound is twice the expected 1.6e-3)
     assert errors(y, ordered)[1] <= 3.2e-3
+    # the same consumer with the activations rounded where the reference rounds them (ajq_w*a16_gemv_norm_sums: the
+    # norm prologue fed with the producer's sums of squares): against the reference order within fp32 noise, up
+    # to a few activations that a differently ordered sum of squares moves to the neighbouring bf16 value
+    if lib.ajq_gemv_fused_supported(m, d):
+        ns_fn = lib.ajq_w4a16_gemv_norm_sums if scheme == "w4" else lib.ajq_w8a16_gemv_norm_sums
+        h_dev = h_out.to(cuda)
+        ssq_dev = ssq.to(cuda)
+        y_ns = torch.empty((m, n2), dtype=torch.float32, device=cuda)
+        _lib.check(ns_fn(h_dev.data_ptr(), ssq_dev.data_ptr(), d // 16, gg.data_ptr(), eps, m, d, wq2.data_ptr(),
+                         meta2.data_ptr(), n2, y_ns.data_ptr(), _lib.AJQ_OUT_F32, 0, st), "gemv_norm_sums")
+        yg_ns = torch.empty((m, n2 // 2), dtype=torch.bfloat16, device=cuda)
+        _lib.check(ns_fn(h_dev.data_ptr(), ssq_dev.data_ptr(), d // 16, gg.data_ptr(), eps, m, d, wq2.data_ptr(),
+                         meta2.data_ptr(), n2, yg_ns.data_ptr(), _lib.AJQ_OUT_BF16, 1, st), "gemv_norm_sums gate")
+        torch.cuda.synchronize()
+        x_own = ((h_out / torch.sqrt(h_out.square().mean(-1, keepdim=True) + eps)) * gain).to(torch.bfloat16)
+        own = qspec.quant_linear(x_own, w2_hat, accumulate=torch.float64, out_dtype=torch.float64)
+        assert errors(y_ns.cpu(), own)[1] <= 2e-4
+        pairs_ns = y_ns.cpu().reshape(m, n2 // 16, 2, 8)
+        gate_ns = (torch.nn.functional.silu(pairs_ns[:, :, 0].double()) * pairs_ns[:, :, 1].double()).reshape(m, n2 // 2)
+        assert bf16_rounding_excess(yg_ns.cpu(), gate_ns, 4e-6 * float(gate_ns.abs().max())) <= 0
     # the gate: tiles of 8 gate rows and 8 up rows
     pairs = y.reshape(m, n2 // 16, 2, 8)
     gate = (torch.nn.functional.silu(pairs[:, :, 0].double()) * pairs[:, :, 1].double()).reshape(m, n2 // 2)

@@ -255,20 +255,30 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         assert errors(got_g, want_g.cpu())[1] <= 3e-3
 
 
-@pytest.mark.parametrize("scheme,batch,kv_heads,kv_dtype", [
-    ("w4a16_g128", 1, 2, None), ("w4a16_g128", 5, 2, None), ("w8a16", 2, 2, None), ("w8a16", 32, 1, None),
-    ("w4a16_g128", 20, 1, None), ("w4a16_g128", 3, 2, torch.bfloat16), ("w8a16", 24, 1, torch.bfloat16)])
-def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_dtype):
+@pytest.mark.parametrize("scheme,batch,kv_heads,kv_dtype,folded", [
+    ("w4a16_g128", 1, 2, None, True), ("w4a16_g128", 5, 2, None, True), ("w8a16", 2, 2, None, True),
+    ("w8a16", 32, 1, None, True), ("w4a16_g128", 20, 1, None, True), ("w4a16_g128", 3, 2, torch.bfloat16, True),
+    ("w8a16", 24, 1, torch.bfloat16, True), ("w4a16_g128", 5, 2, None, False), ("w8a16", 32, 1, None, False),
+    ("w4a16_g128", 1, 1, None, False)])
+def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_dtype, folded):
     """The all-kernel decode step (FusedDecoder) against the eager model loop, replayed from a
     graph; differences only below the eager run's own logit-margin noise.  Batches above 16 take
-    the batched-decode matmul; one key/value head under two query heads is grouped-query attention."""
+    the batched-decode matmul; one key/value head under two query heads is grouped-query attention.
+    ``folded`` True: norms, gates and residual adds in the matmuls' epilogues with the activations rounded before the
+    norm's row scale (the only folded form built for this model's d_model 256); False: every norm, gate, merge and
+    residual add as a launch of its own."""
     torch.manual_seed(4)
     model = modeling.TransformerLM(vocab_size=512, context_length=96, d_model=256, num_layers=3, num_heads=2,
                                    d_ff=640, num_kv_heads=kv_heads).eval()
     fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
     prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(10)).to(cuda)
     eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True, kv_dtype=kv_dtype)
-    dec = decoding.FusedDecoder(fast, batch, 60, kv_dtype)
+    dec = decoding.FusedDecoder(fast, batch, 60, kv_dtype, activation_rounding="before_scale" if folded else "reference")
+    if folded:
+        assert dec.fuse_epilogue and not dec.exact_norm   # (d_model 256: the reference-order consumer is not built)
+    else:
+        dec.fuse_epilogue = dec.fuse_norm = dec.fuse_gate = dec.fuse_merge = False
+        assert dec.launches_per_step() == 9 * 3 + 4
     dec.prefill(prompt, rows_per_pass=8 if batch > 16 else None)
     first = dec.generate(10)
     torch.cuda.synchronize()
@@ -288,7 +298,7 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
             eager_logits = fast(eager[row:row + 1, : 20 + step], fast.new_cache(1, 60, dtype=kv_dtype))[0, -1].float()
         gap = float((fused_logits - eager_logits).abs().max())
         print("row", row, "step", step, "eager margin", margin, "logit difference", gap)
-        assert gap <= 1e-2 and margin <= 2 * gap, (row, step, margin, gap)
+        assert gap <= (2e-2 if folded else 1e-2) and margin <= 2 * gap, (row, step, margin, gap)
     # logits of one fused step against the eager model on the same context
     dec.prefill(prompt)
     with torch.no_grad():
@@ -297,7 +307,10 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
         fast(prompt, cache)
         logits_eager = fast(dec.token, cache)[:, -1, :]
     max_abs, rel = errors(logits_fused, logits_eager.cpu())
-    assert rel <= 1e-3, (max_abs, rel)
+    # unfolded, both loops round the same bf16 activations and differ by summation order only; folded, the norm's
+    # row scale is applied after the matmul, so every normed activation is rounded at a different point (2^-9
+    # relative each, independent of the eager loop's rounding): a few 1e-3 on this 3-layer model
+    assert rel <= (6e-3 if folded else 1e-3), (max_abs, rel)
 
 
 @pytest.mark.parametrize("batch", [1, 3])
@@ -580,6 +593,7 @@ def test_fused_decoder_with_gemv_prologues(cuda, scheme, batch):
     dec = decoding.FusedDecoder(fast, batch, 60)
     assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
     dec.fuse_norm = dec.fuse_gate = True  # also at the batches where the decoder would not choose them
+    dec.fuse_epilogue, dec.fuse_merge = False, dec.merge_splits > 0   # (it prefers the epilogue forms where both are built)
     dec.prefill(prompt)
     got = dec.generate(30)
     report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 20, noise=2e-3)
@@ -623,7 +637,7 @@ def test_fused_decoder_tokens_match_the_oracle_model(cuda):
     assert report["identical_rows"] + len(report["attributable"]) == 4
 
 
-def _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure):
+def _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure, rounding="reference"):
     """The graph-replayed tokens of a FusedDecoder (set up by ``configure``) against the CPU oracle model,
     and the decode-step logits of every step along the oracle's tokens against the oracle's logits."""
     ref = _oracle_model(model, scheme)
@@ -641,7 +655,7 @@ def _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configur
     ref_new, ref_logits = torch.cat(ref_new, 1), torch.stack(ref_logits, 1)
     top2 = torch.topk(ref_logits, 2, dim=-1).values
     margins = top2[..., 0] - top2[..., 1]
-    dec = decoding.FusedDecoder(fast, batch, 48 + new)
+    dec = decoding.FusedDecoder(fast, batch, 48 + new, activation_rounding=rounding)
     configure(dec)
     dec.prefill(prompt.to(cuda))
     got = dec.generate(new).cpu()
@@ -682,14 +696,17 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
     def configure(dec):
         assert dec.head.fusable(batch) and dec.layers[0]["w2"].fusable(batch)
         dec.fuse_norm = dec.fuse_gate = True
+        dec.fuse_epilogue, dec.fuse_merge = False, dec.merge_splits > 0   # (it prefers the epilogue forms where both are built)
 
     _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
 
 
-@pytest.mark.parametrize("scheme,batch,d_ff", [("w4a16_g128", 8, 5632), ("w8a16", 13, 2048), ("w4a16_g128", 5, 4096),
-                                               ("w4a16_g128", 1, 5632), ("w8a16", 4, 2048), ("w4a16_g128", 2, 4096),
-                                               ("w8a16", 20, 2048), ("w4a16_g128", 33, 5632), ("w4a16_g128", 12, 5632)])
-def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff):
+@pytest.mark.parametrize("scheme,batch,d_ff,rounding", [
+    ("w4a16_g128", 1, 5632, "reference"), ("w8a16", 4, 2048, "reference"), ("w4a16_g128", 2, 4096, "reference"),
+    ("w8a16", 3, 5632, "reference"), ("w4a16_g128", 8, 5632, "before_scale"), ("w8a16", 13, 2048, "before_scale"),
+    ("w4a16_g128", 5, 4096, "before_scale"), ("w8a16", 1, 2048, "before_scale"), ("w4a16_g128", 12, 5632, "before_scale"),
+    ("w8a16", 20, 2048, "before_scale"), ("w4a16_g128", 33, 5632, "before_scale")])
+def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff, rounding):
     """Widths the epilogue GEMVs are built for (d_model 2048): no norm, gate or residual launch inside a layer
     (the norm's row scale is applied to the matmul outputs, the residual add and the next norm's preparation
     ride in the output projection and w2, w1|w3 applies the gate on interleaved rows): six launches per
@@ -702,10 +719,11 @@ def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme
 
     def configure(dec):
         assert dec.fuse_epilogue and not dec.fuse_norm and not dec.fuse_gate
+        assert dec.exact_norm == (rounding == "reference")
         assert dec.fuse_merge == (batch == 1) and dec.first_norm_fused == (batch <= 4)
         assert dec.launches_per_step() == (5 if batch == 1 else 6) * 2 + (2 if batch <= 4 else 3)
 
-    _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure)
+    _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure, rounding)
 
 
 def test_quantized_checkpoint_round_trip(cuda, tmp_path):
