@@ -118,8 +118,15 @@ def test_config4_greedy_tokens_against_the_oracle_model(config4, cuda, batch):
     ref_tokens, ref_logits = _oracle_greedy(ref, prompt, NEW)
     top2 = torch.topk(ref_logits, 2, dim=-1).values
     margins = top2[..., 0] - top2[..., 1]                       # [B, NEW]
-    _beat(f"config 4 batch {batch}: fused decoder")
-    dec = decoding.FusedDecoder(fast, batch, PROMPT + NEW)
+    # the decoder's default (the reference's rounding point) and its faster folding (normed activations rounded
+    # before the norm's row scale): same criteria, one report each
+    for rounding, suffix in (("reference", ""), ("before_scale", "_before_scale")):
+        _config4_decoder_against_the_oracle(fast, cuda, batch, prompt, ref_tokens, ref_logits, margins, rounding, suffix)
+
+
+def _config4_decoder_against_the_oracle(fast, cuda, batch, prompt, ref_tokens, ref_logits, margins, rounding, suffix):
+    _beat(f"config 4 batch {batch}: fused decoder, activation rounding {rounding}")
+    dec = decoding.FusedDecoder(fast, batch, PROMPT + NEW, activation_rounding=rounding)
     dec.prefill(prompt.to(cuda))
     got = torch.cat((prompt, dec.generate(NEW).cpu()), dim=1)
     # replayed once more from the recorded graph: the same tokens, bit for bit
@@ -160,13 +167,14 @@ def test_config4_greedy_tokens_against_the_oracle_model(config4, cuda, batch):
                 unexplained.append(row)
         rows.append(row)
     report = {"config": CONFIG4, "scheme": "w4a16_g128", "batch": batch, "prompt": PROMPT, "new_tokens": NEW,
+              "activation_rounding": rounding, "launches_per_step": dec.launches_per_step(),
               "logits_relative_frobenius_error": rel, "logits_max_abs_error": noise,
               "teacher_forced_top1_agreement": float((~disagree).float().mean()),
               "teacher_forced_disagreements": int(disagree.sum()),
               "largest_oracle_gap_at_a_disagreement": float(gap[disagree].max()) if bool(disagree.any()) else 0.0,
               "rows": rows}
     OUT_DIR.mkdir(exist_ok=True)
-    (OUT_DIR / f"config4_tokens_b{batch}.json").write_text(json.dumps(report, indent=1))
+    (OUT_DIR / f"config4_tokens_b{batch}{suffix}.json").write_text(json.dumps(report, indent=1))
     print(json.dumps(report))
     assert not unexplained, unexplained
     # the choices agree on all but a few near-ties
