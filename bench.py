@@ -311,8 +311,9 @@ def cpu_baseline(m: int, n: int, k: int, budget_s: float = 15.0) -> dict:
 def bench_gemv_forms(device, batches=(1, 4, 8), reps: int = 30) -> list[dict]:
     """Microseconds per launch, in a graph chain over six distinct W4 weight sets, of the decode GEMV in its
     plain form and with work folded in: the norm / gate PROLOGUE forms (every workgroup forms the
-    activations from the fp32 sources) against the row-scale / residual / gate EPILOGUE forms (a workgroup
-    touches its own 16 columns), on the 12-layer benchmark model's four projection shapes."""
+    activations from the fp32 sources; "from sums": the norm's sums of squares come from the producer) against
+    the row-scale / residual / gate EPILOGUE forms (a workgroup touches its own 16 columns), on the 12-layer
+    benchmark model's four projection shapes."""
     from ajllm_amd import _lib, quantize_w4_g128, repack_w4
 
     lib = _lib.load()
@@ -350,6 +351,10 @@ def bench_gemv_forms(device, batches=(1, 4, 8), reps: int = 30) -> list[dict]:
                     n, y.data_ptr(), _lib.AJQ_OUT_F32, st)
                 forms["gate_prologue"] = lambda wq, meta, st: lib.ajq_w4a16_gemv_gate(
                     ab.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32, st)
+            if lib.ajq_gemv_fused_supported(m, k) and k // 16 <= 256:
+                forms["norm_from_sums_prologue"] = lambda wq, meta, st: lib.ajq_w4a16_gemv_norm_sums(
+                    hk.data_ptr(), ssq_in.data_ptr(), k // 16, gk.data_ptr(), 1e-5, m, k, wq.data_ptr(), meta.data_ptr(),
+                    n, y.data_ptr(), _lib.AJQ_OUT_F32, 0, st)
             launches = 8 * len(weights)
             row = {"projection": name, "M": m, "N": n, "K": k}
             for form, call in forms.items():
