@@ -209,13 +209,20 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     float total = 0.f;
 #pragma unroll
     for (int u = 0; u < kPartLoads; ++u) total += (sums[u].x + sums[u].y) + (sums[u].z + sums[u].w);
+    if (kLanesPerRow >= 16) {
+      total = team_sum16(total);  // DPP row rotates inside each 16 lanes, then the crossbar for whole rows of 16
 #pragma unroll
-    for (int off = kLanesPerRow / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
-    if (lane % kLanesPerRow == 0) ssq[(lane / kLanesPerRow) * kWaves + wave] = total;
+      for (int off = 16; off < kLanesPerRow; off <<= 1) total += __shfl_xor(total, off);
+    } else {
+#pragma unroll
+      for (int off = kLanesPerRow / 2; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    }
+    if (MROWS > 1 && lane % kLanesPerRow == 0) ssq[(lane / kLanesPerRow) * kWaves + wave] = total;
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = min(lane + 64 * i, kVecs - 1);
-      const float rms = sqrtf(ssq[(v / kVecPerRow) * kWaves + wave] / (float)K + eps);
+      // one row: every lane already holds its total
+      const float rms = sqrtf((MROWS > 1 ? ssq[(v / kVecPerRow) * kWaves + wave] : total) / (float)K + eps);
       const float4 h0 = a0[i][0], h1 = a0[i][1], g0v = a2[i][0], g1v = a2[i][1];
       xv[i][0] = (h0.x / rms) * g0v.x; xv[i][1] = (h0.y / rms) * g0v.y;
       xv[i][2] = (h0.z / rms) * g0v.z; xv[i][3] = (h0.w / rms) * g0v.w;
