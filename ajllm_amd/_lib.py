@@ -92,6 +92,8 @@ SIGNATURES: dict[str, tuple] = {
                                         c_void_p, c_void_p, c_void_p]),
     "ajq_w8a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p]),
+    "ajq_w4a16_gemv_gated": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
+    "ajq_w8a16_gemv_gated": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p]),
     "ajq_w4a16_gemv_norm_sums": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p,
                                          c_int, c_void_p, c_int, c_int, c_void_p]),
     "ajq_w8a16_gemv_norm_sums": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p,

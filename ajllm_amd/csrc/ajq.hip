@@ -525,6 +525,17 @@ int gemv_rowscale(const char* name, const uint16_t* xt, const float* ssq, int pa
 }
 
 template <bool kW4>
+int gemv_gated(const char* name, const uint16_t* x, int M, int K, const uint32_t* wq, const void* aux, int N, void* y,
+               void* stream) {
+  if (int s = check_matmul_args(name, x, M, K, wq, aux, N, y, AJQ_OUT_BF16, kGroup)) return s;
+  if (int s = check_epi(name, M, K)) return s;
+  const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
+  const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
+  if (int s = launch_gemv_epi<kW4, kEpiGate>(x, M, K, wq, meta, scales, N, y, 0, GemvEpilogue{}, (hipStream_t)stream)) return s;
+  return check_launch(name);
+}
+
+template <bool kW4>
 int gemv_residual(const char* name, const uint16_t* x, int M, int K, const uint32_t* wq, const void* aux, int N,
                          const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out, void* stream) {
   if (int s = check_matmul_args(name, x, M, K, wq, aux, N, h_out, AJQ_OUT_F32, kGroup)) return s;
@@ -753,6 +764,16 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1 : 0; }
 
 int ajq_gemv_epilogue_supported(int M, int K) { return gemv_epi_supported(M, K) ? 1 : 0; }
+
+int ajq_w4a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                         void* stream) {
+  return gemv_gated<true>("ajq_w4a16_gemv_gated", x, M, K, wq, meta, N, y, stream);
+}
+
+int ajq_w8a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                         void* stream) {
+  return gemv_gated<false>("ajq_w8a16_gemv_gated", x, M, K, wq, scales, N, y, stream);
+}
 
 int ajq_w4a16_gemv_norm_sums(const float* h, const float* ssq, int parts, const float* gain, float eps, int M, int K,
                              const uint32_t* wq, const uint32_t* meta, int N, void* y, int out_dtype, int gate,

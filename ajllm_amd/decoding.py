@@ -232,6 +232,14 @@ class _FusedLinear:
                       self.rows16, h_in.data_ptr(), gain.data_ptr(), h_out.data_ptr(),
                       xt.data_ptr() if xt is not None else None, ssq.data_ptr(), _stream()), "gemv_merge_residual")
 
+    def gated_interleaved(self, x_bf16: torch.Tensor, gated: torch.Tensor) -> torch.Tensor:
+        """``bf16(silu(a) * u)`` into ``gated`` for an ``interleaved_gate`` pair and plain bf16 activations, one launch."""
+        lib = _lib.load()
+        fn = lib.ajq_w8a16_gemv_gated if self.scheme == "w8a16" else lib.ajq_w4a16_gemv_gated
+        _lib.check(fn(x_bf16.data_ptr(), x_bf16.shape[0], self.in_features, self.wq.data_ptr(), self.meta.data_ptr(),
+                      self.rows16, gated.data_ptr(), _stream()), "gemv_gated")
+        return gated
+
     def normed_from_sums(self, h: torch.Tensor, ssq: torch.Tensor, gain: torch.Tensor, eps: float,
                          gated: torch.Tensor | None = None) -> torch.Tensor:
         """``self(bf16(RMSNorm(h) * gain))`` with the norm's sums of squares taken from what ``residual`` left in
@@ -403,15 +411,19 @@ class FusedDecoder(GraphDecoder):
         # batch 4 "reference" means the unfolded step; "before_scale" folds at every batch (0.34 / 0.42 / 0.60 ms at
         # batch 1 / 4 / 8).
         self.exact_norm = activation_rounding == "reference"
-        rounding_built = (batch <= 4 and self.head.fusable(batch)) if self.exact_norm else True
+        # reference rounding above batch 4 (or where that consumer is not built): the norm is a launch of its own
+        # again, the residual adds and the gate stay in the epilogues (they move no rounding point): eight
+        # launches per layer instead of nine
+        self.norm_launch = self.exact_norm and not (batch <= 4 and self.head.fusable(batch))
         self.fuse_epilogue = (
-            rounding_built and self.d_ff % 8 == 0 and d // 16 <= 256
+            self.d_ff % 8 == 0 and d // 16 <= 256
             and self.layers[0]["o"].in_features == d
             and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
             and self.head.epilogue_fusable(batch)
         )
         if self.fuse_epilogue:
-            self.first_norm_fused = self.fuse_norm   # the step's very first norm rides in layer 0's q|k|v where built
+            # the step's very first norm rides in layer 0's q|k|v where built
+            self.first_norm_fused = self.fuse_norm and not self.norm_launch
             self.fuse_norm = self.fuse_gate = False
             # the merge prologue re-reads every chunk of every head in every workgroup: with the cheaper epilogue
             # kernels around it, it only pays at batch 1 (measured: 0.41 / 0.50 / 0.52 ms per step with it at
@@ -514,7 +526,10 @@ class FusedDecoder(GraphDecoder):
         lib = _lib.load()
         if self.fuse_epilogue:
             # q|k|v, attention (+ merge), output projection, w1|w3 with the gate, w2; the first norm, head, pick
-            return (5 if self.fuse_merge else 6) * len(self.layers) + (2 if self.first_norm_fused else 3)
+            per_layer = 5 if self.fuse_merge else 6
+            if self.norm_launch:  # both norms of a layer and the final one as launches
+                return (per_layer + 2) * len(self.layers) + 3
+            return per_layer * len(self.layers) + (2 if self.first_norm_fused else 3)
         per_layer = 2 if self.fuse_norm else 4           # q|k|v and w1|w3, each with or without its norm launch
         per_layer += 1                                   # attention
         if not self.fuse_merge:                          # merge of its row chunks (none if there is one chunk)
@@ -603,12 +618,16 @@ class FusedDecoder(GraphDecoder):
 
         def normed(linear: _FusedLinear, gain: torch.Tensor, eps: float, gated: torch.Tensor | None = None) -> torch.Tensor:
             """linear(RMSNorm(cur) * gain), the norm taken from the sums of squares cur's producer left."""
+            if self.norm_launch:
+                _lib.check(lib.ajq_add_rmsnorm(cur.data_ptr(), None, gain.data_ptr(), eps, self.normed.data_ptr(), b, d, st),
+                           "add_rmsnorm")
+                return linear(self.normed) if gated is None else linear.gated_interleaved(self.normed, gated)
             if self.exact_norm:
                 return linear.normed_from_sums(cur, self.ssq, gain, eps, gated)
             return linear.rowscaled(self.xt, self.ssq, eps, gated)
 
         for index, w in enumerate(self.layers):
-            if index > 0:
+            if index > 0 or self.norm_launch:
                 qkv = normed(w["qkv"], w["g1"], w["eps1"])
             elif self.first_norm_fused:
                 qkv = w["qkv"].after_norm(self.embedded, None, first["g1"], first["eps1"], self.hidden)

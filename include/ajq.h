@@ -162,6 +162,12 @@ int ajq_w4a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, flo
 int ajq_w8a16_gemv_rowscale(const uint16_t* xt, const float* ssq, int parts, float eps, int M, int K,
                             const uint32_t* wq, const uint16_t* scales, int N, void* y, int out_dtype, int gate,
                             void* stream);
+/*   _gated:    y[M, N / 2] = bf16(silu(a) * u) for the plain bf16 activations x, the rows of W interleaved as for
+ *              _rowscale's gate: w1|w3 with SwiGLU's product in its epilogue (activations.py:24-25), no row scale. */
+int ajq_w4a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
+                         void* stream);
+int ajq_w8a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N, void* y,
+                         void* stream);
 /*   _norm_sums: y = (RMSNorm(h) * gain) W^T with the activations rounded exactly where the reference rounds them,
  *              bf16((h / rms) * gain) (layers.py:70-74 then the bf16 input of the quantized linear), rms taken from
  *              the sums of squares that _residual left in ssq ([rows][parts], parts = K / 16 <= 256): the GEMV with a

@@ -703,7 +703,8 @@ def test_fused_decoder_with_gemv_prologues_matches_the_oracle_model(cuda, scheme
 
 @pytest.mark.parametrize("scheme,batch,d_ff,rounding", [
     ("w4a16_g128", 1, 5632, "reference"), ("w8a16", 4, 2048, "reference"), ("w4a16_g128", 2, 4096, "reference"),
-    ("w8a16", 3, 5632, "reference"), ("w4a16_g128", 8, 5632, "before_scale"), ("w8a16", 13, 2048, "before_scale"),
+    ("w8a16", 3, 5632, "reference"), ("w4a16_g128", 8, 5632, "reference"), ("w8a16", 13, 2048, "reference"),
+    ("w4a16_g128", 8, 5632, "before_scale"), ("w8a16", 13, 2048, "before_scale"),
     ("w4a16_g128", 5, 4096, "before_scale"), ("w8a16", 1, 2048, "before_scale"), ("w4a16_g128", 12, 5632, "before_scale"),
     ("w8a16", 20, 2048, "before_scale"), ("w4a16_g128", 33, 5632, "before_scale")])
 def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme, batch, d_ff, rounding):
@@ -711,7 +712,8 @@ def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme
     (the norm's row scale is applied to the matmul outputs, the residual add and the next norm's preparation
     ride in the output projection and w2, w1|w3 applies the gate on interleaved rows): six launches per
     layer, five at batch 1, where the output projection also merges the attention's row chunks on its way in; up
-    to batch 4 the step's first norm rides in layer 0's q|k|v.  Above 16 rows, and for shapes the GEMV kernel's
+    to batch 4 the step's first norm rides in layer 0's q|k|v.  With the reference's rounding point above batch 4 the
+    norms are launches of their own (eight per layer), the residual adds and the gate stay folded.  Above 16 rows, and for shapes the GEMV kernel's
     straight-line configurations do not cover (12 rows on K = 5632), the weight-streaming kernel carries the epilogues."""
     torch.manual_seed(18)
     model = modeling.TransformerLM(vocab_size=2048, context_length=128, d_model=2048, num_layers=2, num_heads=16,
@@ -720,8 +722,13 @@ def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme
     def configure(dec):
         assert dec.fuse_epilogue and not dec.fuse_norm and not dec.fuse_gate
         assert dec.exact_norm == (rounding == "reference")
+        # reference rounding above batch 4: the norms are launches of their own again (eight per layer)
+        assert dec.norm_launch == (rounding == "reference" and batch > 4)
         assert dec.fuse_merge == (batch == 1) and dec.first_norm_fused == (batch <= 4)
-        assert dec.launches_per_step() == (5 if batch == 1 else 6) * 2 + (2 if batch <= 4 else 3)
+        if dec.norm_launch:
+            assert dec.launches_per_step() == 8 * 2 + 3
+        else:
+            assert dec.launches_per_step() == (5 if batch == 1 else 6) * 2 + (2 if batch <= 4 else 3)
 
     _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure, rounding)
 
