@@ -1030,11 +1030,21 @@ int attn_splits(int B, int Hkv, int max_len) {
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
 }
 
+// Caches of a launch above this many bytes (keys + values as allocated) are streamed: non-temporal loads,
+// rows dealt to the chunks in blocks.  Below it they are read with ordinary loads, chunk by chunk, and
+// stay in the 256 MB last-level cache between steps.  Measured on a 12-layer model's decode step: 12.6 MB
+// per layer is 4 % slower streamed, 19 MB 1 % faster, 25 MB 3 % faster, 100 MB 5 % faster (the
+// attention launch itself: 15-20 %).
+constexpr long long kAttnStreamBytes = 16ll << 20;
+
 template <int R, typename CacheT, bool kStep>
 void launch_attn(const float* q, void* kcache, void* vcache, const long long* pos, int B, int H, int Hkv, int max_len,
                  float scale, int S, float* partial, uint16_t* out, const float* cosine, const float* sine,
                  hipStream_t stream) {
-  hipLaunchKernelGGL((attn_decode_kernel<R, CacheT, kStep>), dim3(B * Hkv, S), dim3(256), 0, stream, q,
+  const long long cache_bytes = 2ll * B * Hkv * max_len * 128 * (long long)sizeof(CacheT);
+  auto kernel = cache_bytes > kAttnStreamBytes ? attn_decode_kernel<R, CacheT, kStep, true>
+                                                    : attn_decode_kernel<R, CacheT, kStep, false>;
+  hipLaunchKernelGGL(kernel, dim3(B * Hkv, S), dim3(256), 0, stream, q,
                      reinterpret_cast<CacheT*>(kcache), reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale,
                      partial, out, cosine, sine);
   if (S > 1 && out != nullptr)  // out == nullptr: the caller merges the chunks itself (ajq_w*a16_gemv_merge)

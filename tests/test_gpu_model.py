@@ -255,6 +255,56 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         assert errors(got_g, want_g.cpu())[1] <= 3e-3
 
 
+@pytest.mark.parametrize("b,heads,kv_heads,max_len,cache_dtype", [
+    (4, 8, 8, 1100, torch.float32), (8, 8, 4, 2100, torch.bfloat16), (16, 8, 2, 1500, torch.float32),
+    (6, 16, 4, 1400, torch.bfloat16)])
+def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads, max_len, cache_dtype):
+    """Caches above 16 MB per launch take the kernel's streaming form (non-temporal loads, rows dealt to the row
+    chunks in blocks of 32): ajq_attn_decode and ajq_attn_step against the model code's attention, at positions on
+    both sides of block and chunk boundaries, with scores spread widely enough that the running reference exponent
+    of the grouped-head form has to move many times."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    hd = 128
+    assert 2 * b * kv_heads * max_len * hd * (4 if cache_dtype == torch.float32 else 2) > 16 << 20
+    g = torch.Generator().manual_seed(b * 1000 + max_len)
+    att = modeling.MultiHeadSelfAttention(heads * hd, heads, max_len, "rope", 10000.0, num_kv_heads=kv_heads).to(cuda)
+    kv_flag = _lib.AJQ_KV_BF16 if cache_dtype == torch.bfloat16 else _lib.AJQ_KV_F32
+    kc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
+    vc = torch.randn((b, kv_heads, max_len, hd), generator=g).to(cuda).to(cache_dtype)
+    qkv = torch.randn((b, (heads + 2 * kv_heads) * hd), generator=g).to(cuda)
+    qkv[:, : heads * hd] *= 4.0     # scores with a standard deviation of 4: exponents 17 apart are common
+    ws_bytes = lib.ajq_attn_step_workspace_bytes(b, heads)
+    ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
+    rep = heads // kv_heads
+    for p in (0, 31, 32, 63, 64, 500, max_len - 33, max_len - 1):
+        pos = torch.tensor([p], device=cuda)
+        k2, v2 = kc.clone(), vc.clone()
+        got = torch.zeros((b, heads * hd), dtype=torch.bfloat16, device=cuda)
+        _lib.check(lib.ajq_attn_step(qkv.data_ptr(), att.rope.cosine.data_ptr(), att.rope.sine.data_ptr(), pos.data_ptr(),
+                                     k2.data_ptr(), v2.data_ptr(), kv_flag, b, heads, kv_heads, hd, max_len,
+                                     got.data_ptr(), ws.data_ptr(), ws_bytes, st), "attn_step")
+        pp = pos.view(1, 1, 1)
+        q_rot = att.rope(qkv[:, : heads * hd].view(b, heads, 1, hd), pp.expand(b, heads, 1))[:, :, 0].contiguous()
+        k_new = att.rope(qkv[:, heads * hd: (heads + kv_heads) * hd].view(b, kv_heads, 1, hd), pp.expand(b, kv_heads, 1))
+        v_new = qkv[:, (heads + kv_heads) * hd:].view(b, kv_heads, hd)
+        untouched = torch.ones(max_len, dtype=torch.bool); untouched[p] = False
+        assert torch.equal(k2[:, :, untouched], kc[:, :, untouched]) and torch.equal(v2[:, :, untouched], vc[:, :, untouched])
+        assert torch.equal(v2[:, :, p], v_new.to(cache_dtype))
+        assert (k2[:, :, p].float() - k_new[:, :, 0]).abs().max() <= 2 ** -7 * k_new.abs().max()
+        keys = k2[:, :, : p + 1].float().repeat_interleave(rep, dim=1)
+        vals = v2[:, :, : p + 1].float().repeat_interleave(rep, dim=1)
+        want = modeling.scaled_dot_product_attention(q_rot.unsqueeze(2), keys, vals)[:, :, 0].reshape(b, heads * hd)
+        assert (got.float() - want).abs().max() <= 2e-2 and errors(got, want.cpu())[1] <= 3e-3, p
+        # the attention alone over the cache the step left (ajq_attn_decode: every row comes from memory)
+        got2 = torch.zeros((b, heads * hd), dtype=torch.bfloat16, device=cuda)
+        _lib.check(lib.ajq_attn_decode(q_rot.data_ptr(), k2.data_ptr(), v2.data_ptr(), kv_flag, pos.data_ptr(), b, heads,
+                                       kv_heads, hd, max_len, got2.data_ptr(), ws.data_ptr(), ws_bytes, st), "attn")
+        assert (got2.float() - want).abs().max() <= 2e-2 and errors(got2, want.cpu())[1] <= 3e-3, p
+        assert (got2.float() - got.float()).abs().max() <= 2 ** -6
+
+
 @pytest.mark.parametrize("scheme,batch,kv_heads,kv_dtype,folded", [
     ("w4a16_g128", 1, 2, None, True), ("w4a16_g128", 5, 2, None, True), ("w8a16", 2, 2, None, True),
     ("w8a16", 32, 1, None, True), ("w4a16_g128", 20, 1, None, True), ("w4a16_g128", 3, 2, torch.bfloat16, True),
