@@ -54,6 +54,7 @@ SIGNATURES: dict[str, tuple] = {
          c_int, c_void_p],
     ),
     "ajq_attn_decode_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "ajq_attn_row_chunks": (c_int, [c_int, c_int, c_int]),
     "ajq_rope_prefill": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,

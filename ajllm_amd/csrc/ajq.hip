@@ -1015,16 +1015,21 @@ int ajq_w8a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, con
 
 // --------------------------------------------------- decode-step operators -----
 namespace {
-#ifndef AJQ_ATTN_WGS
-#define AJQ_ATTN_WGS 640
-#endif
 constexpr int kAttnMaxSplits = 16;
-// Row chunks per cache head.  Measured on (batch x cache heads) = 32 ... 256 at contexts 640 ... 4096: the
-// kernel is fastest with 500-800 workgroups in all (two to three per CU); more chunks only add start-up,
-// in-workgroup merges and partial results.  A chunk keeps at least 32 rows.
+// Row chunks per cache head.  Measured on (batch x cache heads) = 32 ... 256 at contexts 640 ... 8192: the
+// kernel is fastest with 500-800 workgroups in all (two to three per CU; targets of 512 ... 1024 are within
+// 5 % of each other); more chunks only add start-up, in-workgroup merges and partial results.  A chunk keeps
+// at least 32 rows.
+constexpr int kAttnTargetWorkgroups = 768;
+// From one (sequence, cache head) pair per CU on, one 1024-thread workgroup per pair reads the whole head:
+// the chip is occupied without row chunks, and the merge launch and its partial results go away (256 pairs:
+// 5-7 % faster than three chunks and a merge; 128 pairs: 8 % slower than six chunks and a merge).
+constexpr int kAttnWholeHeadPairs = 256;
+bool attn_whole_heads(int B, int Hkv) { return B * Hkv >= kAttnWholeHeadPairs; }
 int attn_splits(int B, int Hkv, int max_len) {
   const int pairs = B * Hkv;
-  int s = (AJQ_ATTN_WGS + pairs / 2) / pairs;
+  if (attn_whole_heads(B, Hkv)) return 1;
+  int s = (kAttnTargetWorkgroups + pairs / 2) / pairs;
   const int by_rows = max_len / 32;
   if (s > by_rows) s = by_rows;
   return s < 1 ? 1 : (s > kAttnMaxSplits ? kAttnMaxSplits : s);
@@ -1042,8 +1047,14 @@ void launch_attn(const float* q, void* kcache, void* vcache, const long long* po
                  float scale, int S, float* partial, uint16_t* out, const float* cosine, const float* sine,
                  hipStream_t stream) {
   const long long cache_bytes = 2ll * B * Hkv * max_len * 128 * (long long)sizeof(CacheT);
-  auto kernel = cache_bytes > kAttnStreamBytes ? attn_decode_kernel<R, CacheT, kStep, true>
-                                                    : attn_decode_kernel<R, CacheT, kStep, false>;
+  const bool streamed = cache_bytes > kAttnStreamBytes;
+  if (attn_whole_heads(B, Hkv)) {  // S == 1 by attn_splits
+    auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 16> : attn_decode_kernel<R, CacheT, kStep, false, 16>;
+    hipLaunchKernelGGL(kernel, dim3(B * Hkv, 1), dim3(1024), 0, stream, q, reinterpret_cast<CacheT*>(kcache),
+                       reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale, partial, out, cosine, sine);
+    return;
+  }
+  auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 4> : attn_decode_kernel<R, CacheT, kStep, false, 4>;
   hipLaunchKernelGGL(kernel, dim3(B * Hkv, S), dim3(256), 0, stream, q,
                      reinterpret_cast<CacheT*>(kcache), reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale,
                      partial, out, cosine, sine);
@@ -1125,6 +1136,11 @@ size_t ajq_attn_decode_workspace_bytes(int B, int H) {
   if (B < 1 || H < 1) return 0;
   // sized for the largest split count: the number of cache heads is not known here
   return (size_t)B * H * kAttnMaxSplits * kAttnPartialStride * sizeof(float);
+}
+
+int ajq_attn_row_chunks(int B, int Hkv, int max_len) {
+  if (B < 1 || Hkv < 1 || max_len < 1) return 0;
+  return attn_splits(B, Hkv, max_len);
 }
 
 int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype, const int64_t* pos, int B,

@@ -129,10 +129,10 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
 }
 
 // Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * Hkv, S): a
-// workgroup of 4 waves takes chunk s of the rows of one cache head and serves the R = H / Hkv
+// workgroup of kWaves waves takes chunk s of the rows of one cache head and serves the R = H / Hkv
 // query heads that share it, so a cache row is read once whatever R is.  Sixteen lanes share
 // one cache row (a lane holds 8 of the 128 dimensions), so a wave works on four rows at a time
-// and a workgroup on sixteen, two rounds in flight; every 16-lane team keeps a reference
+// and a workgroup on 4 kWaves, two rounds in flight; every 16-lane team keeps a reference
 // exponent, denominator and weighted value sum of its rows per query head.  The teams are
 // merged through LDS.  With S == 1 the result is normalised and written as bf16 [B, H * 128];
 // otherwise (max, denominator, 128 sums) go to `partial` for the merge kernel.  A bf16 cache
@@ -144,6 +144,9 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
 // a cache head sweep one region of memory together instead of S regions far apart.  Without it
 // a chunk is a contiguous run of rows and the loads are ordinary ones: a small cache (batch 1)
 // stays in the last-level cache from one step to the next.
+//
+// kWaves = 16 is for launches with enough cache heads to occupy the chip on their own (S = 1): one
+// 1024-thread workgroup per cache head writes the finished output, no partial results and no merge launch.
 struct KvRow8 {
   float4 a, b;
 };
@@ -218,8 +221,8 @@ __device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <int R, typename CacheT, bool kStep, bool kStream>
-__global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restrict__ q, CacheT* __restrict__ kcache,
+template <int R, typename CacheT, bool kStep, bool kStream, int kWaves>
+__global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* __restrict__ q, CacheT* __restrict__ kcache,
                                                           CacheT* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
                                                           float scale, float* __restrict__ partial, uint16_t* __restrict__ out,
@@ -229,7 +232,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
   const int bk = blockIdx.x, S = gridDim.y, s = blockIdx.y;
   const int b = bk / Hkv, hk = bk % Hkv;
   const int bh0 = b * H + hk * R;  // first of the R query heads
-  const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // 16 teams of 16 lanes
+  static_assert(kWaves == 4 || kWaves == 16, "4 waves (row chunks, merged by a second kernel) or 16 (one workgroup per cache head)");
+  constexpr int kTeams = 4 * kWaves;
+  const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // teams of 16 lanes
   const long long p = min(max(*pos, 0LL), (long long)max_len - 1);  // held inside the cache (device data, unchecked by the host)
   const int rows = (int)p + 1;
   const int per = (rows + S - 1) / S;
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     }
   };
   // the step's own row: the chunk that owns it rotates the key, stores both and attends from registers (team 0)
-  const bool own = kStream ? (((int)p >> 5) % S) == s : (t_begin <= (int)p && (int)p < t_end);
+  const bool own = kStream ? (((int)p / (2 * kTeams)) % S) == s : (t_begin <= (int)p && (int)p < t_end);
   if (kStep && own) {
     t_end = (int)p;
     if (team == 0) {
@@ -335,13 +340,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
     }
   }
   // rows first .. limit-1 in steps of `stride`, two rows per team in flight
-  const int first = kStream ? 32 * s + team : t_begin + team;
+  const int first = kStream ? 2 * kTeams * s + team : t_begin + team;
   const int limit = kStream ? ((kStep && own) ? (int)p : rows) : t_end;
-  const int stride = kStream ? 32 * S : 32;
+  const int stride = kStream ? 2 * kTeams * S : 2 * kTeams;
   for (int t = first; t < limit; t += stride) {
-    if (t + 16 < limit) {
-      const KvRow8 k0 = load_row8<kStream>(kbase + (size_t)t * hd), k1 = load_row8<kStream>(kbase + (size_t)(t + 16) * hd);
-      const KvRow8 v0 = load_row8<kStream>(vbase + (size_t)t * hd), v1 = load_row8<kStream>(vbase + (size_t)(t + 16) * hd);
+    if (t + kTeams < limit) {
+      const KvRow8 k0 = load_row8<kStream>(kbase + (size_t)t * hd), k1 = load_row8<kStream>(kbase + (size_t)(t + kTeams) * hd);
+      const KvRow8 v0 = load_row8<kStream>(vbase + (size_t)t * hd), v1 = load_row8<kStream>(vbase + (size_t)(t + kTeams) * hd);
       row(k0.a, k0.b, v0.a, v0.b);
       row(k1.a, k1.b, v1.a, v1.b);
     } else {
@@ -349,18 +354,39 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float* __restric
       row(k0.a, k0.b, v0.a, v0.b);
     }
   }
+  // Sixteen partial results meet in LDS: the 16 teams of a 4-wave workgroup, or the 16 waves of the large one,
+  // whose four teams are first merged inside the wave (lanes 16 and 32 apart hold the same dimensions).
+  if constexpr (kWaves == 16) {
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float mo = __shfl_xor(m[r], off), lo = __shfl_xor(l[r], off);
+        const float mn = fmaxf(m[r], mo);
+        const float cs = m[r] == -INFINITY ? 0.f : exp2_hw(m[r] - mn);   // a team without rows weighs nothing
+        const float co = mo == -INFINITY ? 0.f : exp2_hw(mo - mn);
+        l[r] = l[r] * cs + lo * co;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[r][i] = acc[r][i] * cs + __shfl_xor(acc[r][i], off) * co;
+        m[r] = mn;
+      }
+    }
+  }
   __shared__ float sm[R][16], sl[R][16];
   __shared__ float sacc[R][16][hd];
+  const int entry = kWaves == 16 ? (int)(threadIdx.x >> 6) : team;
+  if (kWaves == 4 || (threadIdx.x & 48) == 0) {
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    if (c == 0) { sm[r][team] = m[r]; sl[r][team] = l[r]; }
+    for (int r = 0; r < R; ++r) {
+      if (c == 0) { sm[r][entry] = m[r]; sl[r][entry] = l[r]; }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) sacc[r][team][LD::dim(c, i)] = acc[r][i];
+      for (int i = 0; i < 8; ++i) sacc[r][entry][LD::dim(c, i)] = acc[r][i];
+    }
   }
   __syncthreads();
-  // wave w merges query heads w, w + 4, ...; two dimensions per lane from here on
+  // wave w merges query heads w, w + kWaves, ...; two dimensions per lane from here on
   const int lane = threadIdx.x & 63;
-  for (int r = threadIdx.x >> 6; r < R; r += 4) {
+  for (int r = threadIdx.x >> 6; r < R; r += kWaves) {
     float M16 = sm[r][0];
 #pragma unroll
     for (int w = 1; w < 16; ++w) M16 = fmaxf(M16, sm[r][w]);

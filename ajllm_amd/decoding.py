@@ -521,18 +521,25 @@ class FusedDecoder(GraphDecoder):
                                                self.step_index.data_ptr(), self.counters.data_ptr(),
                                                self.ticket.data_ptr(), _stream()), "greedy_pick")
 
+    @property
+    def merge_launch(self) -> bool:
+        """Whether the attention's row chunks are merged by a launch of their own (not by the output projection's
+        prologue, and there are several chunks)."""
+        chunks = _lib.load().ajq_attn_row_chunks(self.batch, self.kv_heads, self.max_len)
+        return not self.fuse_merge and chunks > 1
+
     def launches_per_step(self) -> int:
         """Kernel launches of one decode step as this decoder is configured."""
         lib = _lib.load()
         if self.fuse_epilogue:
             # q|k|v, attention (+ merge), output projection, w1|w3 with the gate, w2; the first norm, head, pick
-            per_layer = 5 if self.fuse_merge else 6
+            per_layer = 6 if self.merge_launch else 5
             if self.norm_launch:  # both norms of a layer and the final one as launches
                 return (per_layer + 2) * len(self.layers) + 3
             return per_layer * len(self.layers) + (2 if self.first_norm_fused else 3)
         per_layer = 2 if self.fuse_norm else 4           # q|k|v and w1|w3, each with or without its norm launch
         per_layer += 1                                   # attention
-        if not self.fuse_merge:                          # merge of its row chunks (none if there is one chunk)
+        if self.merge_launch:                            # merge of its row chunks (none if there is one chunk)
             per_layer += 1
         per_layer += 1                                   # output projection
         per_layer += 1 if self.fuse_gate else 2          # w2 with or without the gate launch

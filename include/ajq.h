@@ -257,6 +257,10 @@ int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, f
  * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of
  * them).  head_dim 128 only.  The workspace holds the partial results of up to 16 row chunks. */
 size_t ajq_attn_decode_workspace_bytes(int B, int H);
+/* Row chunks per cache head that ajq_attn_decode and ajq_attn_step use for this shape (0: bad shape).  With 1
+ * the attention is a single launch (no merge kernel; the workspace is not touched): any shape with at least 256
+ * (sequence, cache head) pairs, where one workgroup reads a whole head. */
+int ajq_attn_row_chunks(int B, int Hkv, int max_len);
 int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int cache_dtype,
                     const int64_t* pos, int B, int H, int Hkv, int head_dim, int max_len, uint16_t* out,
                     void* workspace, size_t workspace_bytes, void* stream);

@@ -112,6 +112,17 @@ def test_shape_alignment_and_option_errors():
         _lib.check(-5, "probe")
 
 
+def test_attention_row_chunk_query():
+    """Host-side only: how many row chunks per cache head the decode attention uses (1 = a single launch)."""
+    lib = _lib.load()
+    assert lib.ajq_attn_row_chunks(0, 8, 128) == 0 and lib.ajq_attn_row_chunks(1, 0, 128) == 0
+    assert lib.ajq_attn_row_chunks(1, 16, 768) == 16          # few heads: as many chunks as the merge takes
+    assert lib.ajq_attn_row_chunks(1, 16, 64) == 2            # a chunk keeps at least 32 rows
+    assert lib.ajq_attn_row_chunks(8, 16, 768) == 6           # about 768 workgroups in all
+    assert lib.ajq_attn_row_chunks(32, 8, 2176) == 1          # a cache head per CU: whole heads, no merge
+    assert lib.ajq_attn_row_chunks(100, 16, 4096) == 1
+
+
 def test_python_layer_refuses_cpu_tensors():
     """There is no CPU fallback: the host API raises instead of computing elsewhere."""
     import torch

@@ -177,7 +177,7 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
     g = torch.Generator().manual_seed(21)
-    for b, heads, kv_heads in ((1, 4, 2), (3, 4, 4), (8, 4, 1), (32, 8, 2)):
+    for b, heads, kv_heads in ((1, 4, 2), (3, 4, 4), (8, 4, 1), (32, 8, 2), (64, 4, 4)):  # the last: a workgroup per whole cache head
         d, hd, max_len, ff = heads * 128, 128, 40, 384
         # residual add + RMSNorm
         hidden = torch.randn((b, d), generator=g).to(cuda)
@@ -257,12 +257,14 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
 
 @pytest.mark.parametrize("b,heads,kv_heads,max_len,cache_dtype", [
     (4, 8, 8, 1100, torch.float32), (8, 8, 4, 2100, torch.bfloat16), (16, 8, 2, 1500, torch.float32),
-    (6, 16, 4, 1400, torch.bfloat16)])
+    (6, 16, 4, 1400, torch.bfloat16), (32, 8, 8, 300, torch.float32), (64, 16, 4, 520, torch.bfloat16),
+    (128, 4, 2, 200, torch.float32)])
 def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads, max_len, cache_dtype):
     """Caches above 16 MB per launch take the kernel's streaming form (non-temporal loads, rows dealt to the row
-    chunks in blocks of 32): ajq_attn_decode and ajq_attn_step against the model code's attention, at positions on
-    both sides of block and chunk boundaries, with scores spread widely enough that the running reference exponent
-    of the grouped-head form has to move many times."""
+    chunks in blocks of 32), and from 256 (sequence, cache head) pairs on one 1024-thread workgroup reads a whole
+    head (the last three cases): ajq_attn_decode and ajq_attn_step against the model code's attention, at positions
+    on both sides of block and chunk boundaries, with scores spread widely enough that the running reference
+    exponent of the grouped-head form has to move many times."""
     from ajllm_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
@@ -278,7 +280,7 @@ def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads
     ws_bytes = lib.ajq_attn_step_workspace_bytes(b, heads)
     ws = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device=cuda)
     rep = heads // kv_heads
-    for p in (0, 31, 32, 63, 64, 500, max_len - 33, max_len - 1):
+    for p in (0, 31, 32, 63, 64, 127, 128, max_len // 2, max_len - 33, max_len - 1):
         pos = torch.tensor([p], device=cuda)
         k2, v2 = kc.clone(), vc.clone()
         got = torch.zeros((b, heads * hd), dtype=torch.bfloat16, device=cuda)
