@@ -1042,32 +1042,38 @@ int attn_splits(int B, int Hkv, int max_len) {
 // attention launch itself: 15-20 %).
 constexpr long long kAttnStreamBytes = 16ll << 20;
 
-template <int R, typename CacheT, bool kStep>
+template <int R, typename CacheT, bool kStep, int HD>
 void launch_attn(const float* q, void* kcache, void* vcache, const long long* pos, int B, int H, int Hkv, int max_len,
                  float scale, int S, float* partial, uint16_t* out, const float* cosine, const float* sine,
                  hipStream_t stream) {
-  const long long cache_bytes = 2ll * B * Hkv * max_len * 128 * (long long)sizeof(CacheT);
+  const long long cache_bytes = 2ll * B * Hkv * max_len * HD * (long long)sizeof(CacheT);
   const bool streamed = cache_bytes > kAttnStreamBytes;
   if (attn_whole_heads(B, Hkv)) {  // S == 1 by attn_splits
-    auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 16> : attn_decode_kernel<R, CacheT, kStep, false, 16>;
+    auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 16, HD>
+                           : attn_decode_kernel<R, CacheT, kStep, false, 16, HD>;
     hipLaunchKernelGGL(kernel, dim3(B * Hkv, 1), dim3(1024), 0, stream, q, reinterpret_cast<CacheT*>(kcache),
                        reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale, partial, out, cosine, sine);
     return;
   }
-  auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 4> : attn_decode_kernel<R, CacheT, kStep, false, 4>;
+  auto kernel = streamed ? attn_decode_kernel<R, CacheT, kStep, true, 4, HD> : attn_decode_kernel<R, CacheT, kStep, false, 4, HD>;
   hipLaunchKernelGGL(kernel, dim3(B * Hkv, S), dim3(256), 0, stream, q,
                      reinterpret_cast<CacheT*>(kcache), reinterpret_cast<CacheT*>(vcache), pos, H, Hkv, max_len, scale,
                      partial, out, cosine, sine);
   if (S > 1 && out != nullptr)  // out == nullptr: the caller merges the chunks itself (ajq_w*a16_gemv_merge)
-    hipLaunchKernelGGL(attn_merge_kernel, dim3(B * H), dim3(64), 0, stream, partial, S, out);
+    hipLaunchKernelGGL(attn_merge_kernel<HD>, dim3(B * H), dim3(64), 0, stream, partial, S, out);
 }
 
-template <bool kStep>
-auto pick_attn(int R, int cache_dtype) {
+template <bool kStep, int HD>
+auto pick_attn_hd(int R, int cache_dtype) {
   if (cache_dtype == AJQ_KV_F32)
-    return R == 1 ? launch_attn<1, float, kStep> : R == 2 ? launch_attn<2, float, kStep> : launch_attn<4, float, kStep>;
-  return R == 1 ? launch_attn<1, uint16_t, kStep>
-                : R == 2 ? launch_attn<2, uint16_t, kStep> : launch_attn<4, uint16_t, kStep>;
+    return R == 1 ? launch_attn<1, float, kStep, HD>
+                  : R == 2 ? launch_attn<2, float, kStep, HD> : launch_attn<4, float, kStep, HD>;
+  return R == 1 ? launch_attn<1, uint16_t, kStep, HD>
+                : R == 2 ? launch_attn<2, uint16_t, kStep, HD> : launch_attn<4, uint16_t, kStep, HD>;
+}
+template <bool kStep>
+auto pick_attn(int R, int cache_dtype, int head_dim) {
+  return head_dim == 64 ? pick_attn_hd<kStep, 64>(R, cache_dtype) : pick_attn_hd<kStep, 128>(R, cache_dtype);
 }
 }  // namespace
 
@@ -1147,7 +1153,8 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
                     int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace, size_t workspace_bytes,
                     void* stream) {
   if (!q || !kcache || !vcache || !pos || !out) return fail(AJQ_ERR_NULL, "ajq_attn_decode: null pointer argument");
-  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (only 128 is built)", head_dim);
+  if (head_dim != 128 && head_dim != 64)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (128 and 64 are built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_attn_decode: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
   const int R = H / Hkv;
@@ -1162,7 +1169,7 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: cache_dtype %d is neither AJQ_KV_F32 nor AJQ_KV_BF16", cache_dtype);
   if (!aligned16(kcache) || !aligned16(vcache) || !aligned16(q))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_decode: q and the caches must be 16-byte aligned");
-  pick_attn<false>(R, cache_dtype)(q, const_cast<void*>(kcache), const_cast<void*>(vcache),
+  pick_attn<false>(R, cache_dtype, head_dim)(q, const_cast<void*>(kcache), const_cast<void*>(vcache),
                                    reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len, scale, S,
                                    reinterpret_cast<float*>(workspace), out, nullptr, nullptr, (hipStream_t)stream);
   return check_launch("ajq_attn_decode");
@@ -1180,7 +1187,9 @@ int attn_step_impl(const char* name, const float* qkv, const float* cosine, cons
                    void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len,
                    uint16_t* out, int max_splits, int* splits, void* workspace, size_t workspace_bytes, void* stream) {
   if (!qkv || !cosine || !sine || !pos || !kcache || !vcache) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
-  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "%s: head_dim %d (only 128 is built)", name, head_dim);
+  if (head_dim != 128 && !(head_dim == 64 && out))
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: head_dim %d (128 is built%s)", name, head_dim,
+                out ? ", and 64" : "; unmerged partial results are read by ajq_w*a16_gemv_merge, which assumes it");
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "%s: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", name, B, H, Hkv, max_len);
   const int R = H / Hkv;
@@ -1197,7 +1206,7 @@ int attn_step_impl(const char* name, const float* qkv, const float* cosine, cons
                 ajq_attn_step_workspace_bytes(B, H), workspace_bytes);
   if (splits) *splits = S;
   const float scale = 1.0f / sqrtf((float)head_dim);
-  pick_attn<true>(R, cache_dtype)(qkv, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len,
+  pick_attn<true>(R, cache_dtype, head_dim)(qkv, kcache, vcache, reinterpret_cast<const long long*>(pos), B, H, Hkv, max_len,
                                   scale, S, reinterpret_cast<float*>(workspace), out, cosine, sine,
                                   (hipStream_t)stream);
   return check_launch(name);

@@ -128,16 +128,15 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
     store_pair(kcache + (((size_t)b * Hkv + (head - H)) * max_len + p) * hd + 2 * i, r);
 }
 
-// Single-query attention over cache rows 0 .. *pos for head_dim 128.  Grid (B * Hkv, S): a
+// Single-query attention over cache rows 0 .. *pos for head_dim HD = 128 or 64.  Grid (B * Hkv, S): a
 // workgroup of kWaves waves takes chunk s of the rows of one cache head and serves the R = H / Hkv
 // query heads that share it, so a cache row is read once whatever R is.  Sixteen lanes share
-// one cache row (a lane holds 8 of the 128 dimensions), so a wave works on four rows at a time
+// one cache row (a lane holds HD / 16 of its dimensions), so a wave works on four rows at a time
 // and a workgroup on 4 kWaves, two rounds in flight; every 16-lane team keeps a reference
 // exponent, denominator and weighted value sum of its rows per query head.  The teams are
-// merged through LDS.  With S == 1 the result is normalised and written as bf16 [B, H * 128];
-// otherwise (max, denominator, 128 sums) go to `partial` for the merge kernel.  A bf16 cache
-// row is 256 B: one 128-bit load per lane and operand, widened to fp32 in registers; all
-// arithmetic is fp32 either way.
+// merged through LDS.  With S == 1 the result is normalised and written as bf16 [B, H * HD];
+// otherwise (max, denominator, HD sums) go to `partial` for the merge kernel.  bf16 cache rows are
+// widened to fp32 in registers; all arithmetic is fp32 either way.
 //
 // kStream (caches too large to stay in the last-level cache between steps): rows are fetched with
 // non-temporal loads and dealt to the S chunks in blocks of 32 rows, round-robin, so the chunks of
@@ -147,152 +146,188 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
 //
 // kWaves = 16 is for launches with enough cache heads to occupy the chip on their own (S = 1): one
 // 1024-thread workgroup per cache head writes the finished output, no partial results and no merge launch.
-struct KvRow8 {
-  float4 a, b;
-};
-// One partial result of a row chunk: (maximum, denominator, 0, 0, 128 weighted value sums); the
+
+// One partial result of a row chunk: (maximum, denominator, 0, 0, HD weighted value sums); the
 // sums start on a 16-byte boundary so that a GEMV prologue can fetch them with 128-bit loads.
-constexpr int kAttnPartialStride = 132;
-// Which 8 of a row's 128 dimensions lane c of a team holds.  bf16 rows (256 B): 8c .. 8c+7, one 128-bit
-// load.  fp32 rows (512 B): 4c .. 4c+3 and 64+4c .. 64+4c+3, so each of a team's two 128-bit loads covers
-// 256 contiguous bytes.
-template <typename CacheT> struct LaneDims {
-  static constexpr bool split = sizeof(CacheT) == 4;
-  static constexpr int per_lane = split ? 4 : 8;   // the lane's first dimension = per_lane * c
-  static constexpr int second = split ? 64 : 4;    // its second four start this many dimensions later
+constexpr int attn_partial_stride(int hd) { return 4 + hd; }
+constexpr int kAttnPartialStride = attn_partial_stride(128);
+// Which HD / 16 of a row's dimensions lane c of a team holds (DPL of them, 8 or 4), and how it fetches them.
+// 8 per lane, bf16 rows (256 B): 8c .. 8c+7, one 128-bit load.  8 per lane, fp32 rows (512 B): 4c .. 4c+3
+// and 64+4c .. 64+4c+3, so each of a team's two 128-bit loads covers 256 contiguous bytes.  4 per lane:
+// 4c .. 4c+3, one 128-bit (fp32) or 64-bit (bf16) load.
+template <typename CacheT, int HD> struct LaneDims {
+  static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+  static constexpr int DPL = HD / 16;
+  static constexpr bool split = sizeof(CacheT) == 4 && DPL == 8;
+  static constexpr int per_lane = split ? 4 : DPL;   // the lane's first dimension = per_lane * c
+  static constexpr int second = split ? 64 : 4;      // DPL == 8: its second four start this many dimensions later
   __device__ static __forceinline__ int dim(int c, int i) { return per_lane * c + (i < 4 ? i : second + i - 4); }
 };
-template <bool kStream>
-__device__ __forceinline__ u32x4_t load_kv16(const u32x4_t* p) {
+template <int DPL> struct KvRow {
+  float v[DPL];
+};
+template <bool kStream, typename T>
+__device__ __forceinline__ T load_kv(const T* p) {
   if constexpr (kStream) return __builtin_nontemporal_load(p);
   return *p;
 }
-__device__ __forceinline__ float4 as_float4(u32x4_t v) {
-  return float4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+__device__ __forceinline__ void widen2(uint32_t w, float& lo, float& hi) {  // two bf16 -> two fp32
+  lo = __uint_as_float(w << 16);
+  hi = __uint_as_float(w & 0xFFFF0000u);
 }
 // p: the lane's first dimension of the row
-template <bool kStream>
-__device__ __forceinline__ KvRow8 load_row8(const float* p) {
-  const u32x4_t* p4 = reinterpret_cast<const u32x4_t*>(p);
-  return KvRow8{as_float4(load_kv16<kStream>(p4)), as_float4(load_kv16<kStream>(p4 + LaneDims<float>::second / 4))};
-}
-template <bool kStream>
-__device__ __forceinline__ KvRow8 load_row8(const uint16_t* p) {
-  const u32x4_t v = load_kv16<kStream>(reinterpret_cast<const u32x4_t*>(p));
-  KvRow8 r;
-  r.a = float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u), __uint_as_float(v.y << 16),
-               __uint_as_float(v.y & 0xFFFF0000u)};
-  r.b = float4{__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xFFFF0000u), __uint_as_float(v.w << 16),
-               __uint_as_float(v.w & 0xFFFF0000u)};
+template <bool kStream, int HD>
+__device__ __forceinline__ KvRow<HD / 16> load_row(const float* p) {
+  using LD = LaneDims<float, HD>;
+  KvRow<HD / 16> r;
+  const u32x4_t a = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p));
+  r.v[0] = __uint_as_float(a.x); r.v[1] = __uint_as_float(a.y); r.v[2] = __uint_as_float(a.z); r.v[3] = __uint_as_float(a.w);
+  if constexpr (LD::DPL == 8) {
+    const u32x4_t b = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p + LD::second));
+    r.v[4] = __uint_as_float(b.x); r.v[5] = __uint_as_float(b.y); r.v[6] = __uint_as_float(b.z); r.v[7] = __uint_as_float(b.w);
+  }
   return r;
+}
+template <bool kStream, int HD>
+__device__ __forceinline__ KvRow<HD / 16> load_row(const uint16_t* p) {
+  KvRow<HD / 16> r;
+  if constexpr (HD / 16 == 8) {
+    const u32x4_t v = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p));
+    widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]); widen2(v.z, r.v[4], r.v[5]); widen2(v.w, r.v[6], r.v[7]);
+  } else {
+    const u32x2_t v = load_kv<kStream>(reinterpret_cast<const u32x2_t*>(p));
+    widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]);
+  }
+  return r;
+}
+// the step's own key / value row into the cache; a bf16 cache rounds and hands the rounded values back (what a
+// later read of the cache would give)
+template <int HD>
+__device__ __forceinline__ void store_row(float* p, KvRow<HD / 16>& r) {
+  using LD = LaneDims<float, HD>;
+  *reinterpret_cast<float4*>(p) = float4{r.v[0], r.v[1], r.v[2], r.v[3]};
+  if constexpr (LD::DPL == 8) *reinterpret_cast<float4*>(p + LD::second) = float4{r.v[4], r.v[5], r.v[6], r.v[7]};
+}
+template <int HD>
+__device__ __forceinline__ void store_row(uint16_t* p, KvRow<HD / 16>& r) {
+  if constexpr (HD / 16 == 8) {
+    u32x4_t v;
+    v.x = pack2_bf16(r.v[0], r.v[1]); v.y = pack2_bf16(r.v[2], r.v[3]);
+    v.z = pack2_bf16(r.v[4], r.v[5]); v.w = pack2_bf16(r.v[6], r.v[7]);
+    *reinterpret_cast<u32x4_t*>(p) = v;
+    widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]); widen2(v.z, r.v[4], r.v[5]); widen2(v.w, r.v[6], r.v[7]);
+  } else {
+    u32x2_t v;
+    v.x = pack2_bf16(r.v[0], r.v[1]); v.y = pack2_bf16(r.v[2], r.v[3]);
+    *reinterpret_cast<u32x2_t*>(p) = v;
+    widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]);
+  }
 }
 
 // kStep: the whole attention part of a decode step in one launch.  `q` is then the fused
-// projection output qkv [B, (H + 2 Hkv) * 128] (query heads, key heads, value heads): the
+// projection output qkv [B, (H + 2 Hkv) * HD] (query heads, key heads, value heads): the
 // workgroup rotates its R query heads itself (interleaved pairs, the tables' row *pos); the
 // workgroup whose chunk holds row *pos also rotates the new key, writes it and the new value
 // into the caches and attends to them from registers.  (Merging the S partial results in the
 // workgroup that finishes last was tried and lost: the device-scope fences it needs write back
 // and invalidate the XCD's L2, several microseconds per launch; the merge stays a launch.)
-__device__ __forceinline__ void rotate4(float4& v, const float4 c, const float4 s) {
-  // pairs (x, y) and (z, w) with the angles of c.x/s.x and c.y/s.y
-  v = float4{v.x * c.x - v.y * s.x, v.x * s.x + v.y * c.x, v.z * c.y - v.w * s.y, v.z * s.y + v.w * c.y};
-}
-__device__ __forceinline__ void store_row8(float* p, float4& a, float4& b) {
-  reinterpret_cast<float4*>(p)[0] = a;
-  reinterpret_cast<float4*>(p)[LaneDims<float>::second / 4] = b;
-}
-__device__ __forceinline__ void store_row8(uint16_t* p, float4& a, float4& b) {
-  // rounds to bf16 and hands the rounded values back: what a later read of the cache would give
-  u32x4_t v;
-  v.x = pack2_bf16(a.x, a.y);
-  v.y = pack2_bf16(a.z, a.w);
-  v.z = pack2_bf16(b.x, b.y);
-  v.w = pack2_bf16(b.z, b.w);
-  *reinterpret_cast<u32x4_t*>(p) = v;
-  a = float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u), __uint_as_float(v.y << 16),
-             __uint_as_float(v.y & 0xFFFF0000u)};
-  b = float4{__uint_as_float(v.z << 16), __uint_as_float(v.z & 0xFFFF0000u), __uint_as_float(v.w << 16),
-             __uint_as_float(v.w & 0xFFFF0000u)};
-}
 
 // 2^x by the hardware instruction (1 ulp); the softmax below keeps its running maximum and
 // scores in the base-2 domain, scores pre-multiplied by log2(e)
 __device__ __forceinline__ float exp2_hw(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float kLog2e = 1.4426950408889634f;
 
-template <int R, typename CacheT, bool kStep, bool kStream, int kWaves>
+template <int R, typename CacheT, bool kStep, bool kStream, int kWaves, int HD>
 __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* __restrict__ q, CacheT* __restrict__ kcache,
                                                           CacheT* __restrict__ vcache,
                                                           const long long* __restrict__ pos, int H, int Hkv, int max_len,
                                                           float scale, float* __restrict__ partial, uint16_t* __restrict__ out,
                                                           const float* __restrict__ cosine,
                                                           const float* __restrict__ sine) {
-  constexpr int hd = 128;
+  static_assert(kWaves == 4 || kWaves == 16, "4 waves (row chunks, merged by a second kernel) or 16 (one workgroup per cache head)");
+  constexpr int hd = HD;
+  constexpr int kTeams = 4 * kWaves;
+  using LD = LaneDims<CacheT, HD>;
+  constexpr int DPL = LD::DPL;
+  using Row = KvRow<DPL>;
   const int bk = blockIdx.x, S = gridDim.y, s = blockIdx.y;
   const int b = bk / Hkv, hk = bk % Hkv;
   const int bh0 = b * H + hk * R;  // first of the R query heads
-  static_assert(kWaves == 4 || kWaves == 16, "4 waves (row chunks, merged by a second kernel) or 16 (one workgroup per cache head)");
-  constexpr int kTeams = 4 * kWaves;
   const int team = threadIdx.x >> 4, c = threadIdx.x & 15;  // teams of 16 lanes
   const long long p = min(max(*pos, 0LL), (long long)max_len - 1);  // held inside the cache (device data, unchecked by the host)
   const int rows = (int)p + 1;
   const int per = (rows + S - 1) / S;
   const int t_begin = s * per;
   int t_end = min(rows, t_begin + per);
-  using LD = LaneDims<CacheT>;
-  constexpr int sec4 = LD::second / 4;  // the lane's second float4, in float4 units from its first
   const int d0 = LD::per_lane * c;      // the lane's first dimension
-  float4 qa[R], qb[R];
-  float4 ca, cb, sa, sb;  // kStep: cosines / sines of this lane's four pairs, two per float4 half
+  // kStep: cosines / sines of the lane's DPL / 2 pairs (interleaved pairs never straddle a lane's four)
+  float cs[DPL / 2], sn[DPL / 2];
   const float* qkv_row = q + (size_t)b * (H + 2 * Hkv) * hd + d0;  // kStep only
   if (kStep) {
-    const float2 c0 = *reinterpret_cast<const float2*>(cosine + p * (hd / 2) + d0 / 2);
-    const float2 c1 = *reinterpret_cast<const float2*>(cosine + p * (hd / 2) + (d0 + LD::second) / 2);
-    const float2 s0 = *reinterpret_cast<const float2*>(sine + p * (hd / 2) + d0 / 2);
-    const float2 s1 = *reinterpret_cast<const float2*>(sine + p * (hd / 2) + (d0 + LD::second) / 2);
-    ca = float4{c0.x, c0.y, 0.f, 0.f}; cb = float4{c1.x, c1.y, 0.f, 0.f};
-    sa = float4{s0.x, s0.y, 0.f, 0.f}; sb = float4{s1.x, s1.y, 0.f, 0.f};
+#pragma unroll
+    for (int h2 = 0; h2 < DPL / 4; ++h2) {
+      const int pair0 = (d0 + h2 * LD::second) / 2;
+      const float2 c2 = *reinterpret_cast<const float2*>(cosine + p * (hd / 2) + pair0);
+      const float2 s2 = *reinterpret_cast<const float2*>(sine + p * (hd / 2) + pair0);
+      cs[2 * h2] = c2.x; cs[2 * h2 + 1] = c2.y;
+      sn[2 * h2] = s2.x; sn[2 * h2 + 1] = s2.y;
+    }
   }
+  auto rotate = [&](Row& r) {
+#pragma unroll
+    for (int i = 0; i < DPL / 2; ++i) {
+      const float e = r.v[2 * i], o = r.v[2 * i + 1];
+      r.v[2 * i] = e * cs[i] - o * sn[i];
+      r.v[2 * i + 1] = e * sn[i] + o * cs[i];
+    }
+  };
+  // a row of fp32 activations (queries, the step's own key and value) in the lane's dimensions
+  auto load_act = [&](const float* src) {
+    Row r;
+    const float4 a = *reinterpret_cast<const float4*>(src);
+    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
+    if constexpr (DPL == 8) {
+      const float4 b4 = *reinterpret_cast<const float4*>(src + LD::second);
+      r.v[4] = b4.x; r.v[5] = b4.y; r.v[6] = b4.z; r.v[7] = b4.w;
+    }
+    return r;
+  };
+  Row qr[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const float4* q4 = reinterpret_cast<const float4*>(kStep ? qkv_row + (size_t)(hk * R + r) * hd
-                                                             : q + (size_t)(bh0 + r) * hd + d0);
-    qa[r] = q4[0];
-    qb[r] = q4[sec4];
-    if (kStep) {
-      rotate4(qa[r], ca, sa);
-      rotate4(qb[r], cb, sb);
-    }
+    qr[r] = load_act(kStep ? qkv_row + (size_t)(hk * R + r) * hd : q + (size_t)(bh0 + r) * hd + d0);
+    if (kStep) rotate(qr[r]);
   }
   const CacheT* kbase = kcache + (size_t)bk * max_len * hd + d0;
   const CacheT* vbase = vcache + (size_t)bk * max_len * hd + d0;
   const float scale2 = scale * kLog2e;  // maxima and the partial results' maxima are base-2 exponents
-  float m[R], l[R], acc[R][8];
+  float m[R], l[R], acc[R][DPL];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     m[r] = -INFINITY;
     l[r] = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[r][i] = 0.f;
+    for (int i = 0; i < DPL; ++i) acc[r][i] = 0.f;
   }
+  auto dot = [&](const Row& a, const Row& k) {
+    float d = a.v[0] * k.v[0];
+#pragma unroll
+    for (int i = 1; i < DPL; ++i) d += a.v[i] * k.v[i];
+    return team_sum16(d) * scale2;
+  };
   // One cache row against the R queries.  One query head: the textbook running maximum.  Several: the
   // reference exponent m[r] of a team moves only when a new weight would pass 2^12 (always on the team's
   // first row: m = -inf gives +inf); then, for the whole wave, it becomes the running maximum and the sums
-  // are rescaled.  Otherwise a row costs its dot product, one exponential and nine FMAs per head instead of
-  // two exponentials and seventeen (12 % faster at R = 4 on a bf16 cache, 1 % slower at R = 1: the vote).
-  auto row = [&](const float4& ka, const float4& kb, const float4& va, const float4& vb) {
+  // are rescaled.  Otherwise a row costs its dot product, one exponential and DPL + 1 FMAs per head instead of
+  // two exponentials and twice the FMAs (12 % faster at R = 4 on a bf16 cache, 1 % slower at R = 1: the vote).
+  auto row = [&](const Row& k, const Row& v) {
     if constexpr (R == 1) {
-      float d = qa[0].x * ka.x + qa[0].y * ka.y + qa[0].z * ka.z + qa[0].w * ka.w + qb[0].x * kb.x + qb[0].y * kb.y +
-                qb[0].z * kb.z + qb[0].w * kb.w;
-      const float sc = team_sum16(d) * scale2;
+      const float sc = dot(qr[0], k);
       const float m_new = fmaxf(m[0], sc);
       const float corr = exp2_hw(m[0] - m_new), w = exp2_hw(sc - m_new);
       l[0] = l[0] * corr + w;
-      acc[0][0] = acc[0][0] * corr + w * va.x; acc[0][1] = acc[0][1] * corr + w * va.y;
-      acc[0][2] = acc[0][2] * corr + w * va.z; acc[0][3] = acc[0][3] * corr + w * va.w;
-      acc[0][4] = acc[0][4] * corr + w * vb.x; acc[0][5] = acc[0][5] * corr + w * vb.y;
-      acc[0][6] = acc[0][6] * corr + w * vb.z; acc[0][7] = acc[0][7] * corr + w * vb.w;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) acc[0][i] = acc[0][i] * corr + w * v.v[i];
       m[0] = m_new;
       return;
     }
@@ -300,9 +335,7 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
     bool far = false;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      float d = qa[r].x * ka.x + qa[r].y * ka.y + qa[r].z * ka.z + qa[r].w * ka.w + qb[r].x * kb.x + qb[r].y * kb.y +
-                qb[r].z * kb.z + qb[r].w * kb.w;
-      sc[r] = team_sum16(d) * scale2;
+      sc[r] = dot(qr[r], k);
       far |= !(sc[r] - m[r] <= 12.0f);
     }
     if (__builtin_amdgcn_ballot_w64(far) != 0) {
@@ -312,7 +345,7 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
         const float corr = exp2_hw(m[r] - m_new);
         l[r] *= corr;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[r][i] *= corr;
+        for (int i = 0; i < DPL; ++i) acc[r][i] *= corr;
         m[r] = m_new;
       }
     }
@@ -320,8 +353,8 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
     for (int r = 0; r < R; ++r) {
       const float w = exp2_hw(sc[r] - m[r]);
       l[r] += w;
-      acc[r][0] += w * va.x; acc[r][1] += w * va.y; acc[r][2] += w * va.z; acc[r][3] += w * va.w;
-      acc[r][4] += w * vb.x; acc[r][5] += w * vb.y; acc[r][6] += w * vb.z; acc[r][7] += w * vb.w;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) acc[r][i] += w * v.v[i];
     }
   };
   // the step's own row: the chunk that owns it rotates the key, stores both and attends from registers (team 0)
@@ -329,14 +362,12 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
   if (kStep && own) {
     t_end = (int)p;
     if (team == 0) {
-      const float4* k4 = reinterpret_cast<const float4*>(qkv_row + (size_t)(H + hk) * hd);
-      const float4* v4 = reinterpret_cast<const float4*>(qkv_row + (size_t)(H + Hkv + hk) * hd);
-      float4 ka = k4[0], kb = k4[sec4], va = v4[0], vb = v4[sec4];
-      rotate4(ka, ca, sa);
-      rotate4(kb, cb, sb);
-      store_row8(kcache + ((size_t)bk * max_len + p) * hd + d0, ka, kb);
-      store_row8(vcache + ((size_t)bk * max_len + p) * hd + d0, va, vb);
-      row(ka, kb, va, vb);
+      Row kn = load_act(qkv_row + (size_t)(H + hk) * hd);
+      Row vn = load_act(qkv_row + (size_t)(H + Hkv + hk) * hd);
+      rotate(kn);
+      store_row<HD>(kcache + ((size_t)bk * max_len + p) * hd + d0, kn);
+      store_row<HD>(vcache + ((size_t)bk * max_len + p) * hd + d0, vn);
+      row(kn, vn);
     }
   }
   // rows first .. limit-1 in steps of `stride`, two rows per team in flight
@@ -345,13 +376,13 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
   const int stride = kStream ? 2 * kTeams * S : 2 * kTeams;
   for (int t = first; t < limit; t += stride) {
     if (t + kTeams < limit) {
-      const KvRow8 k0 = load_row8<kStream>(kbase + (size_t)t * hd), k1 = load_row8<kStream>(kbase + (size_t)(t + kTeams) * hd);
-      const KvRow8 v0 = load_row8<kStream>(vbase + (size_t)t * hd), v1 = load_row8<kStream>(vbase + (size_t)(t + kTeams) * hd);
-      row(k0.a, k0.b, v0.a, v0.b);
-      row(k1.a, k1.b, v1.a, v1.b);
+      const Row k0 = load_row<kStream, HD>(kbase + (size_t)t * hd), k1 = load_row<kStream, HD>(kbase + (size_t)(t + kTeams) * hd);
+      const Row v0 = load_row<kStream, HD>(vbase + (size_t)t * hd), v1 = load_row<kStream, HD>(vbase + (size_t)(t + kTeams) * hd);
+      row(k0, v0);
+      row(k1, v1);
     } else {
-      const KvRow8 k0 = load_row8<kStream>(kbase + (size_t)t * hd), v0 = load_row8<kStream>(vbase + (size_t)t * hd);
-      row(k0.a, k0.b, v0.a, v0.b);
+      const Row k0 = load_row<kStream, HD>(kbase + (size_t)t * hd), v0 = load_row<kStream, HD>(vbase + (size_t)t * hd);
+      row(k0, v0);
     }
   }
   // Sixteen partial results meet in LDS: the 16 teams of a 4-wave workgroup, or the 16 waves of the large one,
@@ -363,11 +394,11 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
       for (int r = 0; r < R; ++r) {
         const float mo = __shfl_xor(m[r], off), lo = __shfl_xor(l[r], off);
         const float mn = fmaxf(m[r], mo);
-        const float cs = m[r] == -INFINITY ? 0.f : exp2_hw(m[r] - mn);   // a team without rows weighs nothing
+        const float cs_ = m[r] == -INFINITY ? 0.f : exp2_hw(m[r] - mn);   // a team without rows weighs nothing
         const float co = mo == -INFINITY ? 0.f : exp2_hw(mo - mn);
-        l[r] = l[r] * cs + lo * co;
+        l[r] = l[r] * cs_ + lo * co;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[r][i] = acc[r][i] * cs + __shfl_xor(acc[r][i], off) * co;
+        for (int i = 0; i < DPL; ++i) acc[r][i] = acc[r][i] * cs_ + __shfl_xor(acc[r][i], off) * co;
         m[r] = mn;
       }
     }
@@ -380,12 +411,13 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
     for (int r = 0; r < R; ++r) {
       if (c == 0) { sm[r][entry] = m[r]; sl[r][entry] = l[r]; }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) sacc[r][entry][LD::dim(c, i)] = acc[r][i];
+      for (int i = 0; i < DPL; ++i) sacc[r][entry][LD::dim(c, i)] = acc[r][i];
     }
   }
   __syncthreads();
-  // wave w merges query heads w, w + kWaves, ...; two dimensions per lane from here on
+  // wave w merges query heads w, w + kWaves, ...; two dimensions per lane from here on (the first HD / 2 lanes)
   const int lane = threadIdx.x & 63;
+  const int dl = min(lane, hd / 2 - 1);
   for (int r = threadIdx.x >> 6; r < R; r += kWaves) {
     float M16 = sm[r][0];
 #pragma unroll
@@ -396,14 +428,15 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
     for (int w = 0; w < 16; ++w) {
       const float cw = sm[r][w] == -INFINITY ? 0.f : exp2_hw(sm[r][w] - M16);
       L += sl[r][w] * cw;
-      A.x += sacc[r][w][2 * lane] * cw;
-      A.y += sacc[r][w][2 * lane + 1] * cw;
+      A.x += sacc[r][w][2 * dl] * cw;
+      A.y += sacc[r][w][2 * dl + 1] * cw;
     }
+    if (2 * lane >= hd) continue;
     if (S == 1 && out != nullptr) {
       const uint32_t o = pack2_bf16(A.x / L, A.y / L);
       reinterpret_cast<uint32_t*>(out + (size_t)(bh0 + r) * hd)[lane] = o;
     } else {  // several chunks, or a caller that merges them itself (out == nullptr)
-      float* dst = partial + ((size_t)(bh0 + r) * S + s) * kAttnPartialStride;
+      float* dst = partial + ((size_t)(bh0 + r) * S + s) * attn_partial_stride(hd);
       if (lane == 0) *reinterpret_cast<float4*>(dst) = float4{M16, L, 0.f, 0.f};
       *reinterpret_cast<float2*>(dst + 4 + 2 * lane) = A;
     }
@@ -411,19 +444,21 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
 }
 
 // merge of the S <= 16 partial results of attn_decode_kernel: one wave per (b, h).  Lane s
-// fetches chunk s's maximum and denominator and every lane its two dimensions of all chunks
-// at once, so the kernel is one memory round trip, not one per chunk.
+// fetches chunk s's maximum and denominator and every lane (the first HD / 2) its two dimensions of all
+// chunks at once, so the kernel is one memory round trip, not one per chunk.
+template <int HD>
 __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ partial, int S,
                                                         uint16_t* __restrict__ out) {
-  constexpr int hd = 128;
+  constexpr int hd = HD, stride = attn_partial_stride(HD);
   const int bh = blockIdx.x, lane = threadIdx.x;
-  const float* src = partial + (size_t)bh * S * kAttnPartialStride;
+  const int dl = min(lane, hd / 2 - 1);
+  const float* src = partial + (size_t)bh * S * stride;
   const int sl = min(lane & 15, S - 1);
-  const float2 ml = *reinterpret_cast<const float2*>(src + sl * kAttnPartialStride);  // (max, denominator) of chunk lane % 16
+  const float2 ml = *reinterpret_cast<const float2*>(src + sl * stride);  // (max, denominator) of chunk lane % 16
   float2 a[16];
 #pragma unroll
   for (int s = 0; s < 16; ++s)
-    a[s] = *reinterpret_cast<const float2*>(src + min(s, S - 1) * kAttnPartialStride + 4 + 2 * lane);
+    a[s] = *reinterpret_cast<const float2*>(src + min(s, S - 1) * stride + 4 + 2 * dl);
   float M = ml.x;
 #pragma unroll
   for (int off = 8; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
@@ -439,6 +474,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict_
       A.y += a[s].y * c;
     }
   }
+  if (2 * lane >= hd) return;
   const uint32_t o = pack2_bf16(A.x / L, A.y / L);
   reinterpret_cast<uint32_t*>(out + (size_t)bh * hd)[lane] = o;
 }

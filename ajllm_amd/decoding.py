@@ -325,8 +325,10 @@ class FusedDecoder(GraphDecoder):
     up to 16 rows, weight-streaming kernel up to 255); nine launches per layer where those forms are not built.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
-    head_dim 128, 1, 2 or 4 query heads per cache head, an untied quantized ``lm_head``, every
-    linear a QuantLinear.  ``kv_dtype``: torch.float32 (default, the model's own dtype) or
+    head_dim 128 or 64 (64: the geometry of the reference's configs/models/transformer_medium.yaml; the attention's
+    merge is then always a launch of its own and ``prefill(fused=True)`` is refused), 1, 2 or 4 query heads per
+    cache head, a quantized ``lm_head`` of its own (``quantize_model_(..., untie_head=True)`` for tied embeddings),
+    every linear a QuantLinear.  ``kv_dtype``: torch.float32 (default, the model's own dtype) or
     torch.bfloat16 (keys and values rounded to nearest even on write, half the cache traffic)."""
 
     def __init__(self, model: modeling.TransformerLM, batch: int, max_len: int,
@@ -343,17 +345,18 @@ class FusedDecoder(GraphDecoder):
             model.position_encoding == "rope" and first.norm_placement == "pre"
             and isinstance(first.norm1, modeling.RMSNorm) and isinstance(first.feed_forward, modeling.SwiGLU)
             and isinstance(model.final_norm, modeling.RMSNorm) and isinstance(model.lm_head, QuantLinear)
-            and model.d_model // model.num_heads == 128 and model.num_heads // model.num_kv_heads in (1, 2, 4)
+            and model.d_model // model.num_heads in (128, 64) and model.num_heads // model.num_kv_heads in (1, 2, 4)
             and all(isinstance(m, QuantLinear) for layer in model.layers
                     for m in (layer.attention.q_proj, layer.attention.k_proj, layer.attention.v_proj,
                               layer.attention.output_proj, layer.feed_forward.w1, layer.feed_forward.w2,
                               layer.feed_forward.w3))
         )
         if not ok:
-            raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128 and "
-                             "quantized linears everywhere (untied lm_head included)")
+            raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128 or 64 and "
+                             "quantized linears everywhere (an lm_head of its own included: quantize_model_(..., "
+                             "untie_head=True) gives a model with tied embeddings one)")
         dev, d = self.device, model.d_model
-        self.heads, self.kv_heads, self.head_dim = model.num_heads, model.num_kv_heads, 128
+        self.heads, self.kv_heads, self.head_dim = model.num_heads, model.num_kv_heads, d // model.num_heads
         self.d_ff = first.feed_forward.w1.out_features
         self.layers = []
         for layer in model.layers:
@@ -392,7 +395,8 @@ class FusedDecoder(GraphDecoder):
                           and self.layers[0]["w13"].rows16 == 2 * self.d_ff)
         # the output projection merges the attention's row chunks on its way in where that is built
         # (small batches; one launch less per layer)
-        self.merge_splits = self.layers[0]["o"].merge_splits(batch) if self.layers[0]["o"].in_features == d else 0
+        self.merge_splits = (self.layers[0]["o"].merge_splits(batch)
+                             if self.layers[0]["o"].in_features == d and self.head_dim == 128 else 0)
         self.fuse_merge = self.merge_splits > 0
         # Larger batches (every workgroup would re-read the fp32 sources of all rows): the norm's row scale
         # is applied to the OUTPUTS of q|k|v, w1|w3 and the head instead, the output projection and w2 add
@@ -448,6 +452,8 @@ class FusedDecoder(GraphDecoder):
         if not fused:
             super().prefill(prompt, rows_per_pass)
         else:
+            if self.head_dim != 128:
+                raise ValueError("the library's prefill attention is built for head_dim 128; use fused=False")
             if prompt.shape[0] != self.batch or prompt.shape[1] >= self.max_len:
                 raise ValueError("prompt must be [batch, T] with T < max_len")
             prompt = prompt.to(self.device)
@@ -581,14 +587,14 @@ class FusedDecoder(GraphDecoder):
                 _lib.check(lib.ajq_attn_step_partial(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
                                                      pos.data_ptr(), self.cache.keys[index].data_ptr(),
                                                      self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
-                                                     self.kv_heads, 128, self.max_len, self.merge_splits,
+                                                     self.kv_heads, self.head_dim, self.max_len, self.merge_splits,
                                                      ctypes.addressof(splits), self.attn_ws.data_ptr(),
                                                      self.attn_ws_bytes, st), "attn_step_partial")
                 delta = w["o"].after_merge(self.attn_ws, splits.value, b)
             else:
                 _lib.check(lib.ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), pos.data_ptr(),
                                              self.cache.keys[index].data_ptr(), self.cache.values[index].data_ptr(),
-                                             self.kv_flag, b, self.heads, self.kv_heads, 128, self.max_len,
+                                             self.kv_flag, b, self.heads, self.kv_heads, self.head_dim, self.max_len,
                                              self.attended.data_ptr(), self.attn_ws.data_ptr(), self.attn_ws_bytes, st),
                            "attn_step")
                 delta = w["o"](self.attended)
@@ -607,7 +613,7 @@ class FusedDecoder(GraphDecoder):
         _lib.check(_lib.load().ajq_attn_step(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
                                              self.cache.position.data_ptr(), self.cache.keys[index].data_ptr(),
                                              self.cache.values[index].data_ptr(), self.kv_flag, self.batch, self.heads,
-                                             self.kv_heads, 128, self.max_len, self.attended.data_ptr(),
+                                             self.kv_heads, self.head_dim, self.max_len, self.attended.data_ptr(),
                                              self.attn_ws.data_ptr(), self.attn_ws_bytes, _stream()), "attn_step")
 
     def _logits_epilogue(self) -> torch.Tensor:
@@ -649,7 +655,7 @@ class FusedDecoder(GraphDecoder):
                 _lib.check(lib.ajq_attn_step_partial(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(),
                                                      self.cache.position.data_ptr(), self.cache.keys[index].data_ptr(),
                                                      self.cache.values[index].data_ptr(), self.kv_flag, b, self.heads,
-                                                     self.kv_heads, 128, self.max_len, self.merge_splits,
+                                                     self.kv_heads, self.head_dim, self.max_len, self.merge_splits,
                                                      ctypes.addressof(splits), self.attn_ws.data_ptr(),
                                                      self.attn_ws_bytes, st), "attn_step_partial")
                 w["o"].merge_residual(self.attn_ws, splits.value, b, cur, w["g2"], nxt, xt, self.ssq)

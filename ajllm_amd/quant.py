@@ -326,15 +326,25 @@ def _is_reference_linear(module: nn.Module) -> bool:
 
 
 @torch.no_grad()
-def quantize_model_(model: nn.Module, scheme: str = "w4a16_g128", skip: tuple[str, ...] = ()) -> nn.Module:
+def quantize_model_(model: nn.Module, scheme: str = "w4a16_g128", skip: tuple[str, ...] = (),
+                    untie_head: bool = False) -> nn.Module:
     """Swap every bias-free linear of ``model`` for a :class:`QuantLinear`, in place.
 
     Matches by duck type, so it finds the reference's ``q_proj/k_proj/v_proj/output_proj``
     (src/ajllm/modeling/attention.py:82-85), ``w1/w2/w3`` (activations.py:20-22) and
-    ``lm_head`` (transformer.py:108).  Embeddings are not linears and stay dense."""
+    ``lm_head`` (transformer.py:108).  Embeddings are not linears and stay dense.
+
+    A model with tied embeddings has no ``lm_head`` module: its logits are ``hidden @ embedding.T``
+    (transformer.py:116-118) and stay a dense product.  With ``untie_head`` such a model gets a
+    quantized ``lm_head`` made from the embedding matrix (the embedding itself stays dense for the
+    look-up) and stops being tied: the head then runs through the library like every other linear."""
     for parent in list(model.modules()):
         for name, child in list(parent.named_children()):
             if name in skip or not _is_reference_linear(child):
                 continue
             setattr(parent, name, QuantLinear.from_linear(child, scheme))
+    if (untie_head and getattr(model, "tie_embeddings", False) and getattr(model, "lm_head", None) is None
+            and hasattr(model, "token_embeddings") and "lm_head" not in skip):
+        model.lm_head = QuantLinear.from_weight(model.token_embeddings.weight.data, scheme)
+        model.tie_embeddings = False
     return model

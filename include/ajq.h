@@ -255,7 +255,8 @@ int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, f
 /* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
  * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
  * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of
- * them).  head_dim 128 only.  The workspace holds the partial results of up to 16 row chunks. */
+ * them).  head_dim 128 or 64 (the reference's configs/models/transformer_medium.yaml: 768 / 12 heads).
+ * The workspace holds the partial results of up to 16 row chunks. */
 size_t ajq_attn_decode_workspace_bytes(int B, int H);
 /* Row chunks per cache head that ajq_attn_decode and ajq_attn_step use for this shape (0: bad shape).  With 1
  * the attention is a single launch (no merge kernel; the workspace is not touched): any shape with at least 256
@@ -266,7 +267,7 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two operators above in one kernel: qkv as for ajq_rope_cache; the step's key and value
- * rows are written to row *pos of the caches and attended to from registers. */
+ * rows are written to row *pos of the caches and attended to from registers.  head_dim 128 or 64. */
 size_t ajq_attn_step_workspace_bytes(int B, int H);
 int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
                   void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
@@ -276,7 +277,8 @@ int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, cons
  * head) stay in the workspace as records of 132 floats (maximum as a base-2 exponent, denominator,
  * two pad words, 128 weighted value sums) for ajq_w*a16_gemv_merge, the output projection that
  * merges them on its way in (one launch less per layer).  At most max_splits chunks are used (what
- * ajq_gemv_merge_max_splits allows for the batch); *splits (host memory) receives S. */
+ * ajq_gemv_merge_max_splits allows for the batch); *splits (host memory) receives S.  head_dim 128 only
+ * (the record layout ajq_w*a16_gemv_merge reads). */
 int ajq_attn_step_partial(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
                           void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
                           int max_len, int max_splits, int* splits, void* workspace, size_t workspace_bytes,

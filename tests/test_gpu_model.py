@@ -137,8 +137,46 @@ def test_reference_medium_geometry_decodes_through_the_graph_decoder(cuda, schem
         dense = model.to(cuda)(prompt).float()
         quant = fast(prompt).float()
     assert errors(quant.cpu(), dense.cpu())[1] <= (0.3 if scheme == "w4a16_g128" else 0.05)  # the quantization error itself
+    with pytest.raises(ValueError, match="lm_head of its own"):
+        decoding.FusedDecoder(fast, 2, 64)   # tied embeddings: the head is a dense product of the model code
+
+
+@pytest.mark.parametrize("scheme,batch,kv_dtype", [("w4a16_g128", 1, None), ("w8a16", 3, None), ("w4a16_g128", 8, torch.bfloat16)])
+def test_reference_medium_geometry_decodes_through_the_fused_decoder(cuda, scheme, batch, kv_dtype):
+    """The same geometry (head_dim 64, d_model 768, tied embeddings) with the head untied into a quantized
+    linear of its own (``untie_head``): the all-kernel decoder gives the eager loop's tokens, and the untied
+    quantized head's logits differ from the tied dense head's by the quantization error only."""
+    torch.manual_seed(22)
+    model = modeling.TransformerLM(vocab_size=1024, context_length=128, d_model=768, num_layers=3, num_heads=12,
+                                   d_ff=2048, tie_embeddings=True).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme, untie_head=True)
+    assert isinstance(fast.lm_head, QuantLinear) and not fast.tie_embeddings
+    assert len([m for m in fast.modules() if isinstance(m, QuantLinear)]) == 3 * 7 + 1
+    prompt = torch.randint(0, 1024, (batch, 24), generator=torch.Generator().manual_seed(6)).to(cuda)
+    with torch.no_grad():
+        tied = quantize_model_(copy.deepcopy(model).to(cuda), scheme)(prompt).float()
+        untied = fast(prompt).float()
+    assert errors(untied.cpu(), tied.cpu())[1] <= (0.15 if scheme == "w4a16_g128" else 0.02)
+    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True, kv_dtype=kv_dtype)
+    dec = decoding.FusedDecoder(fast, batch, 80, kv_dtype=kv_dtype)
+    assert dec.head_dim == 64 and not dec.fuse_merge
     with pytest.raises(ValueError, match="head_dim 128"):
-        decoding.FusedDecoder(fast, 2, 64)
+        dec.prefill(prompt, fused=True)
+    dec.prefill(prompt)
+    got = dec.generate(40)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 24, noise=2e-3)
+    assert not report["unexplained"], report
+    assert report["identical_rows"] + len(report["attributable"]) == batch
+    # logits of one fused step against the eager model on the same context: the same bf16 activations up to the few
+    # that a differently ordered sum of squares in a norm moves to the neighbouring bf16 value (2^-8 relative each),
+    # and different summation orders in the matmuls
+    dec.prefill(prompt)
+    with torch.no_grad():
+        logits_fused = dec._logits()
+        cache = fast.new_cache(batch, 80, dtype=kv_dtype)
+        fast(prompt, cache)
+        logits_eager = fast(dec.token, cache)[:, -1, :]
+    assert errors(logits_fused, logits_eager.cpu())[1] <= 3e-3
 
 
 @pytest.mark.parametrize("batch", [1, 3])
@@ -255,20 +293,20 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         assert errors(got_g, want_g.cpu())[1] <= 3e-3
 
 
-@pytest.mark.parametrize("b,heads,kv_heads,max_len,cache_dtype", [
-    (4, 8, 8, 1100, torch.float32), (8, 8, 4, 2100, torch.bfloat16), (16, 8, 2, 1500, torch.float32),
-    (6, 16, 4, 1400, torch.bfloat16), (32, 8, 8, 300, torch.float32), (64, 16, 4, 520, torch.bfloat16),
-    (128, 4, 2, 200, torch.float32)])
-def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads, max_len, cache_dtype):
+@pytest.mark.parametrize("b,heads,kv_heads,max_len,cache_dtype,hd", [
+    (4, 8, 8, 1100, torch.float32, 128), (8, 8, 4, 2100, torch.bfloat16, 128), (16, 8, 2, 1500, torch.float32, 128),
+    (6, 16, 4, 1400, torch.bfloat16, 128), (32, 8, 8, 300, torch.float32, 128), (64, 16, 4, 520, torch.bfloat16, 128),
+    (128, 4, 2, 200, torch.float32, 128), (16, 8, 8, 1100, torch.float32, 64), (64, 16, 4, 600, torch.bfloat16, 64),
+    (12, 12, 12, 900, torch.bfloat16, 64)])
+def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads, max_len, cache_dtype, hd):
     """Caches above 16 MB per launch take the kernel's streaming form (non-temporal loads, rows dealt to the row
     chunks in blocks of 32), and from 256 (sequence, cache head) pairs on one 1024-thread workgroup reads a whole
-    head (the last three cases): ajq_attn_decode and ajq_attn_step against the model code's attention, at positions
+    head (256 pairs and more); head_dim 128 and 64: ajq_attn_decode and ajq_attn_step against the model code's attention, at positions
     on both sides of block and chunk boundaries, with scores spread widely enough that the running reference
     exponent of the grouped-head form has to move many times."""
     from ajllm_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
-    hd = 128
     assert 2 * b * kv_heads * max_len * hd * (4 if cache_dtype == torch.float32 else 2) > 16 << 20
     g = torch.Generator().manual_seed(b * 1000 + max_len)
     att = modeling.MultiHeadSelfAttention(heads * hd, heads, max_len, "rope", 10000.0, num_kv_heads=kv_heads).to(cuda)
@@ -330,7 +368,10 @@ def test_fused_decoder_matches_eager_decoding(cuda, scheme, batch, kv_heads, kv_
         assert dec.fuse_epilogue and not dec.exact_norm   # (d_model 256: the reference-order consumer is not built)
     else:
         dec.fuse_epilogue = dec.fuse_norm = dec.fuse_gate = dec.fuse_merge = False
-        assert dec.launches_per_step() == 9 * 3 + 4
+        # nine per layer, eight where the attention has a single row chunk and so no merge launch (60 rows here)
+        from ajllm_amd import _lib
+        chunks = _lib.load().ajq_attn_row_chunks(batch, kv_heads, 60)
+        assert dec.launches_per_step() == (9 if chunks > 1 else 8) * 3 + 4
     dec.prefill(prompt, rows_per_pass=8 if batch > 16 else None)
     first = dec.generate(10)
     torch.cuda.synchronize()
