@@ -22,17 +22,19 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // hidden[b, :] += delta[b, :] (when delta != nullptr; written back), then
 // out[b, :] = bf16( (hidden / sqrt(mean(hidden^2) + eps)) * gain ).
-// One 256-thread workgroup per row; D % 4 == 0.
+// One 256-thread workgroup per row; D % 4 == 0.  The first 4096 elements of a row (four float4 per thread)
+// and their gains stay in registers between the two passes: one memory round trip for the usual widths.
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hidden, const float* __restrict__ delta,
                                                           const float* __restrict__ gain, float eps,
                                                           uint16_t* __restrict__ out, int D) {
+  constexpr int kKeep = 4;
   const int b = blockIdx.x;
   float4* h4 = reinterpret_cast<float4*>(hidden + (size_t)b * D);
   const float4* d4 = delta ? reinterpret_cast<const float4*>(delta + (size_t)b * D) : nullptr;
   const float4* g4 = reinterpret_cast<const float4*>(gain);
   const int n4 = D >> 2;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < n4; i += 256) {
+  auto take = [&](int i) {
     float4 v = h4[i];
     if (d4) {
       const float4 d = d4[i];
@@ -40,7 +42,18 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
       h4[i] = v;
     }
     ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    return v;
+  };
+  float4 keep[kKeep], g[kKeep];
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < n4) {
+      keep[j] = take(i);
+      g[j] = g4[i];
+    }
   }
+  for (int i = threadIdx.x + 256 * kKeep; i < n4; i += 256) take(i);
   ss = wave_sum(ss);
   __shared__ float part[4];
   if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
@@ -48,13 +61,17 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
   ss = (part[0] + part[1]) + (part[2] + part[3]);
   const float rms = sqrtf(ss / (float)D + eps);
   uint2* o2 = reinterpret_cast<uint2*>(out + (size_t)b * D);
-  for (int i = threadIdx.x; i < n4; i += 256) {
-    const float4 v = h4[i];  // own writes above: same thread, same addresses
-    const float4 g = g4[i];
-    const uint32_t lo = pack2_bf16((v.x / rms) * g.x, (v.y / rms) * g.y);
-    const uint32_t hi = pack2_bf16((v.z / rms) * g.z, (v.w / rms) * g.w);
+  auto put = [&](int i, const float4& v, const float4& gg) {
+    const uint32_t lo = pack2_bf16((v.x / rms) * gg.x, (v.y / rms) * gg.y);
+    const uint32_t hi = pack2_bf16((v.z / rms) * gg.z, (v.w / rms) * gg.w);
     o2[i] = uint2{lo, hi};
+  };
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < n4) put(i, keep[j], g[j]);
   }
+  for (int i = threadIdx.x + 256 * kKeep; i < n4; i += 256) put(i, h4[i], g4[i]);  // own writes above: same thread, same addresses
 }
 
 // qkv [B, (H + 2 Hkv) * hd] fp32 (q heads, then k heads, then v heads) -> rotated q

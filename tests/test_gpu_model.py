@@ -293,6 +293,30 @@ def test_decode_step_operators_match_their_pytorch_statement(cuda):
         assert errors(got_g, want_g.cpu())[1] <= 3e-3
 
 
+@pytest.mark.parametrize("d", [4, 132, 1024, 2048, 4096, 4100, 5632, 12292])
+def test_add_rmsnorm_over_widths(cuda, d):
+    """ajq_add_rmsnorm at widths on both sides of what a workgroup keeps in registers between its two passes
+    (4096 elements), with and without the residual add, against the model code's RMSNorm (layers.py:70-74)."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(d)
+    for b in (1, 5):
+        hidden = (torch.randn((b, d), generator=g) * 2).to(cuda)
+        delta = torch.randn((b, d), generator=g).to(cuda)
+        norm = modeling.RMSNorm(d).to(cuda)
+        norm.weight.data = torch.rand(d, generator=g).to(cuda) + 0.5
+        for with_delta in (True, False):
+            h2 = hidden.clone()
+            out = torch.zeros((b, d), dtype=torch.bfloat16, device=cuda)
+            _lib.check(lib.ajq_add_rmsnorm(h2.data_ptr(), delta.data_ptr() if with_delta else None, norm.weight.data_ptr(),
+                                           norm.epsilon, out.data_ptr(), b, d, st), "add_rmsnorm")
+            summed = hidden + delta if with_delta else hidden
+            assert torch.equal(h2, summed)
+            want = norm(summed).to(torch.bfloat16)
+            assert errors(out, want.cpu())[1] <= 3e-3 and (out.float() - want.float()).abs().max() <= 2 ** -5
+
+
 @pytest.mark.parametrize("b,heads,kv_heads,max_len,cache_dtype,hd", [
     (4, 8, 8, 1100, torch.float32, 128), (8, 8, 4, 2100, torch.bfloat16, 128), (16, 8, 2, 1500, torch.float32, 128),
     (6, 16, 4, 1400, torch.bfloat16, 128), (32, 8, 8, 300, torch.float32, 128), (64, 16, 4, 520, torch.bfloat16, 128),
