@@ -214,12 +214,13 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
             "quant_linear_share_of_step": t_linear / step,
             "quant_linear_GB/s": packed / t_linear / 1e9,
             "packed_weight_bytes": packed,
-            "launches_per_layer": 6 if (dec.fuse_norm and dec.fuse_gate) else 7 if dec.fuse_norm else 9,
+            "launches_per_step": dec.launches_per_step(),
             "loop": "one-token step replayed from a HIP graph, token fed back on the device; the step is this "
-                    "library's kernels only (fused q|k|v and w1|w3 GEMVs with the residual add + RMSNorm formed on "
-                    "their way in at small batch, RoPE + cache write + single-query attention in one kernel, merge "
-                    "of its row chunks, output projection, w2 with the SwiGLU gate on its way in at batch 1, greedy "
-                    "pick + embedding row) plus one counter increment",
+                    "library's kernels only (fused q|k|v and w1|w3 GEMVs, the residual adds and the SwiGLU gate in "
+                    "the matmuls' epilogues, the RMSNorms formed on the consumers' way in up to batch 4 and as "
+                    "launches of their own above, RoPE + cache write + single-query attention in one kernel, its "
+                    "row chunks merged by the output projection at batch 1 and by a launch above, greedy pick + "
+                    "embedding row + step counters in one launch)",
         }
         log("decode", r)
         results.append(r)
