@@ -272,12 +272,19 @@ int ajq_unrepack_w8(const uint32_t* wq, int N, int K, int8_t* q, void* stream) {
 // --------------------------------------------------------------- GEMV -----
 namespace {
 
+constexpr int kGemvFragWorkgroups = 256;  // one per CU
+
 template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
 int launch_gemv_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                     const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   constexpr size_t lds = gemv_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4, kSingle>;
+  // at most one workgroup per CU: the A fragments of every k-step wait in registers for the weights (measured:
+  // 3.87 -> 3.57 us on 4096 x 4096 at one row; on launches of several rounds the registers cost more in
+  // occupancy than the early fragments save, 7.16 -> 7.49 us on 14336 x 4096)
+  constexpr bool kCanHoldFrags = kSingle && TPW <= 4;
+  auto kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4, kSingle, false>;
+  if (kCanHoldFrags && N / kTileN <= kGemvFragWorkgroups) kernel = dequant_gemv_kernel<kWaves, TPW, MROWS, kW4, kSingle, kCanHoldFrags>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream,
                      reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M | (out_f32 << 8), N, y, scales8);
@@ -457,7 +464,8 @@ int launch_gemv_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, con
                         int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
   constexpr size_t lds = gemv_epi_lds_bytes(kWaves, TPW, MROWS);
   static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_gemv_epi_kernel<kWaves, TPW, MROWS, kW4, true, kEpi>;
+  auto kernel = dequant_gemv_epi_kernel<kWaves, TPW, MROWS, kW4, true, kEpi, false>;
+  if (TPW <= 4 && N / kTileN <= kGemvFragWorkgroups) kernel = dequant_gemv_epi_kernel<kWaves, TPW, MROWS, kW4, true, kEpi, TPW <= 4>;
   if (int s = allow_big_lds(kernel, lds)) return s;
   hipLaunchKernelGGL(kernel, dim3(N / kTileN), dim3(kWaves * 64), lds, stream, reinterpret_cast<const u32x4_t*>(wq),
                      meta, x, K, M | (out_f32 << 8), N, y, scales8, ep);

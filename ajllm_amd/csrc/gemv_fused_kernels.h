@@ -304,7 +304,21 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-  if (kW4) {
+  if constexpr (gemv_valu_group_sums(kW4, MROWS)) {  // the same arithmetic as dequant_gemv_body, bit for bit
+    float gs[MROWS][TPW];
+    gemv_group_sums<TPW, MROWS>(xs, kStride, gs);
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      f32x4_t part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+        part = mfma16(a, w4_unpack(w[p][0][j], w4c), part);
+      }
+#pragma unroll
+      for (int i = 0; i < MROWS; ++i) acc[i] += sc[p] * (part[i] - zc[p] * gs[i][p]);
+    }
+  } else if (kW4) {
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};

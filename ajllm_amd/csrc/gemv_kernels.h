@@ -65,7 +65,35 @@ struct GemvEpilogue {
   float* ssq_out;       // residual: [16][N / 16]
 };
 
-template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi>
+// W4 with at most four rows: the zero-point term's group sums, sum_k x over each 128-k group of the wave's
+// LDS slice, by the VALU instead of a second MFMA per k-step against an all-ones operand.  With one live row
+// an MFMA does sixteen rows' work for one, and the matrix pipe's time per tile (8 MFMAs of 32 cycles) is of
+// the order of the tile's share of the memory stream; this halves it.  Team t of the wave (16 lanes) sums
+// group t, t + 4, ...: one 16-byte LDS read per lane, seven adds, four row rotates; the result is wave-uniform.
+// Rows >= M hold copies of row M - 1 (the staging clamps), so every row is read as it is.
+template <int TPW, int MROWS>
+__device__ __forceinline__ void gemv_group_sums(const uint16_t* xs, int stride, float (&gs)[MROWS][TPW]) {
+  const int lane = threadIdx.x & 63, t = lane >> 4, c = lane & 15;
+#pragma unroll
+  for (int m = 0; m < MROWS; ++m) {
+#pragma unroll
+    for (int p0 = 0; p0 < TPW; p0 += 4) {
+      const int p = min(p0 + t, TPW - 1);  // teams past the last group repeat it; their sums are not read
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(xs + m * stride + p * kGroup + 8 * c);
+      auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
+      auto hi = [](uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); };
+      float sum = ((lo(v.x) + hi(v.x)) + (lo(v.y) + hi(v.y))) + ((lo(v.z) + hi(v.z)) + (lo(v.w) + hi(v.w)));
+      sum = team_sum16(sum);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (p0 + q < TPW) gs[m][p0 + q] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sum), 16 * q));
+    }
+  }
+}
+// whether a GEMV configuration takes its W4 group sums from gemv_group_sums
+constexpr bool gemv_valu_group_sums(bool w4, int mrows) { return w4 && mrows <= 4; }
+
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi, bool kFrags = false>
 __device__ __forceinline__ void dequant_gemv_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -104,21 +132,24 @@ __device__ __forceinline__ void dequant_gemv_body(
   // Every load below is unconditional (addresses are clamped into the wave's own
   // range instead), so the number of loads in flight is static and the compiler
   // can wait for exactly the operand it is about to use.
+  // Issue order: the activation slice (an L2 hit: one or two instructions, back long before the first weight
+  // tile, so the wave stages it and forms what depends on it alone while the weights travel; vector loads
+  // return in issue order), the weights, the meta words.
   auto load = [&](Batch& b, int g0) {
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      const int g = kSingle ? g0 + p : min(g0 + p, g_end - 1);
-#pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h)
-        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
-    }
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = min(lane + 64 * i, kVecs - 1);
       const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
       const int k = kSingle ? g0 * kGroup + 8 * c : min(g0 * kGroup + 8 * c, K - 8);
       b.x[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + k);
+    }
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) {
+      const int g = kSingle ? g0 + p : min(g0 + p, g_end - 1);
+#pragma unroll
+      for (int h = 0; h < kLoadsPerGroup; ++h)
+        b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
     }
     if (kW4) {
 #pragma unroll
@@ -137,6 +168,25 @@ __device__ __forceinline__ void dequant_gemv_body(
   const uint16_t* xrow = xs + row * kStride + 8 * kc;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 
+  // slice of a batch -> wave-private LDS.  LDS operations of one wave execute in order, so the reads of the
+  // previous batch are already done.
+  auto stage = [&](const Batch& b) {
+#pragma unroll
+    for (int i = 0; i < kXLoads; ++i) {
+      const int v = lane + 64 * i;
+      if ((i + 1) * 64 <= kVecs || v < kVecs)
+        *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = b.x[i];
+    }
+  };
+  // kSingle: formed from the activations alone, before the weights have landed (see the kSingle branch below)
+  static_assert(!kFrags || (kSingle && TPW <= 4), "A fragments are held in registers for single-batch waves of up to four tiles");
+  constexpr bool kValuSums = gemv_valu_group_sums(kW4, MROWS);
+  u32x4_t afr[kFrags ? TPW : 1][4];
+  float gs[kValuSums ? MROWS : 1][TPW];
+  auto fragment = [&](int p, int j) {
+    if constexpr (kFrags) return afr[p][j];
+    else return *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+  };
   auto compute = [&](Batch& b, int g0) {
     // The meta words are the last loads of the batch and their conversion is its
     // first use: a wave's tiles arrive together, so waiting for all of the batch
@@ -151,15 +201,24 @@ __device__ __forceinline__ void dequant_gemv_body(
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    // slice of this batch -> wave-private LDS.  LDS operations of one wave execute
-    // in order, so the reads of the previous batch are already done.
-#pragma unroll
-    for (int i = 0; i < kXLoads; ++i) {
-      const int v = lane + 64 * i;
-      if ((i + 1) * 64 <= kVecs || v < kVecs)
-        *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = b.x[i];
+    if (!kSingle) {
+      stage(b);
+      if constexpr (kValuSums) gemv_group_sums<TPW, MROWS>(xs, kStride, gs);
     }
-    if (kW4) {
+    if constexpr (kValuSums) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) {
+        if (kSingle || g0 + p < g_end) {
+          f32x4_t part = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) part = mfma16(fragment(p, j), w4_unpack(b.w[p][0][j], w4c), part);
+          // (128+q) and (128+z) cancel in fp32 before the scale is applied; only the lane quarter kc = 0
+          // holds live rows (row i in component i)
+#pragma unroll
+          for (int i = 0; i < MROWS; ++i) acc[i] += sc[p] * (part[i] - zc[p] * gs[i][p]);
+        }
+      }
+    } else if (kW4) {
 #pragma unroll
       for (int p = 0; p < TPW; ++p) {
         if (kSingle || g0 + p < g_end) {
@@ -168,7 +227,7 @@ __device__ __forceinline__ void dequant_gemv_body(
           f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+            const u32x4_t a = fragment(p, j);
             part = mfma16(a, w4_unpack(b.w[p][0][j], w4c), part);
             asum = mfma16(a, ones, asum);
           }
@@ -183,7 +242,7 @@ __device__ __forceinline__ void dequant_gemv_body(
         if (kSingle || g0 + p < g_end) {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+            const u32x4_t a = fragment(p, j);
             const u32x2_t lo = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1)]);
             const u32x2_t hi = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1) + 1]);
             acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);
@@ -224,6 +283,18 @@ __device__ __forceinline__ void dequant_gemv_body(
     Batch b0;
     load(b0, g_begin);
     epilogue_loads();
+    // what needs the activations only, while the weights are on their way: the LDS image, the W4 group sums,
+    // and (kFrags: launches of at most one workgroup per CU, where the registers cost no occupancy that
+    // matters) the A fragments of every k-step
+    stage(b0);
+    if constexpr (kFrags) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) afr[p][j] = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+    }
+    if constexpr (kValuSums) gemv_group_sums<TPW, MROWS>(xs, kStride, gs);
+    __builtin_amdgcn_sched_barrier(0);
     compute(b0, g_begin);
   } else if (g_begin < g_end) {
     Batch b0, b1;
@@ -324,19 +395,19 @@ __device__ __forceinline__ void dequant_gemv_body(
   }
 }
 
-template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle>
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, bool kFrags = false>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K,
     int m_flags, int N, void* __restrict__ y, const uint16_t* __restrict__ scales8) {
-  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, 0>(wq, meta, x, K, m_flags, N, y, scales8, GemvEpilogue{});
+  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, 0, kFrags>(wq, meta, x, K, m_flags, N, y, scales8, GemvEpilogue{});
 }
 
 // the same kernel with work around the matmul (see kEpi above)
-template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi>
+template <int kWaves, int TPW, int MROWS, bool kW4, bool kSingle, int kEpi, bool kFrags = false>
 __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_epi_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K,
     int m_flags, int N, void* __restrict__ y, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
-  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, kEpi>(wq, meta, x, K, m_flags, N, y, scales8, ep);
+  dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, kEpi, kFrags>(wq, meta, x, K, m_flags, N, y, scales8, ep);
 }
 
 // ---------------------------------------------------------------------------
