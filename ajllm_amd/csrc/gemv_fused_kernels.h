@@ -144,6 +144,11 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       sums[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
     }
   }
+  if (kW4) {  // before the weights: scales and zero-points are there when the first tile lands
+    const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
+#pragma unroll
+    for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
+  }
   {
     const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
 #pragma unroll
@@ -151,11 +156,6 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
 #pragma unroll
       for (int h = 0; h < kLoadsPerGroup; ++h)
         w[p][h] = __builtin_nontemporal_load(wtile + (p * kLoadsPerGroup + h) * 64);
-  }
-  if (kW4) {
-    const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
-#pragma unroll
-    for (int p = 0; p < TPW; ++p) mw[p] = mtile[p * 16];
   }
   constexpr bool kResid = kOut == kOutResid;
   constexpr int kLiveRows = MROWS < 4 ? MROWS : 4;
@@ -291,7 +291,15 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = pk;
   }
 
-  // ---- the matmul, as in dequant_gemv_kernel
+  // ---- the matmul, as in dequant_gemv_kernel.  What depends on the activations alone comes first, while the
+  // weights travel: the W4 group sums.  (Holding the A fragments in registers as well, as the plain GEMV does on
+  // small launches, bought under 1 % of a decode step here and is not built.)
+  constexpr bool kValuSums = gemv_valu_group_sums(kW4, MROWS);
+  const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
+  float gs[kValuSums ? MROWS : 1][TPW];
+  if constexpr (kValuSums) gemv_group_sums<TPW, MROWS>(xs, kStride, gs);
+  __builtin_amdgcn_sched_barrier(0);
+  auto fragment = [&](int p, int j) { return *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j); };
   float sc[TPW], zc[TPW];
   if (kW4) {
 #pragma unroll
@@ -302,19 +310,13 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
   }
   const W4Consts w4c = w4_consts();
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-  const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-  if constexpr (gemv_valu_group_sums(kW4, MROWS)) {  // the same arithmetic as dequant_gemv_body, bit for bit
-    float gs[MROWS][TPW];
-    gemv_group_sums<TPW, MROWS>(xs, kStride, gs);
+  if constexpr (kValuSums) {  // the same arithmetic as dequant_gemv_body, bit for bit
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       f32x4_t part = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-        part = mfma16(a, w4_unpack(w[p][0][j], w4c), part);
-      }
+      for (int j = 0; j < 4; ++j) part = mfma16(fragment(p, j), w4_unpack(w[p][0][j], w4c), part);
 #pragma unroll
       for (int i = 0; i < MROWS; ++i) acc[i] += sc[p] * (part[i] - zc[p] * gs[i][p]);
     }
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       f32x4_t part = {0.f, 0.f, 0.f, 0.f}, asum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+        const u32x4_t a = fragment(p, j);
         part = mfma16(a, w4_unpack(w[p][0][j], w4c), part);
         asum = mfma16(a, ones, asum);
       }
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     for (int p = 0; p < TPW; ++p)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
+        const u32x4_t a = fragment(p, j);
         const u32x2_t lo = w8_to_bf16(w[p][j >> 1][2 * (j & 1)]);
         const u32x2_t hi = w8_to_bf16(w[p][j >> 1][2 * (j & 1) + 1]);
         acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);

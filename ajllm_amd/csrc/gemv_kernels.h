@@ -134,7 +134,7 @@ __device__ __forceinline__ void dequant_gemv_body(
   // can wait for exactly the operand it is about to use.
   // Issue order: the activation slice (an L2 hit: one or two instructions, back long before the first weight
   // tile, so the wave stages it and forms what depends on it alone while the weights travel; vector loads
-  // return in issue order), the weights, the meta words.
+  // return in issue order), the meta words, the weights.
   auto load = [&](Batch& b, int g0) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -144,17 +144,17 @@ __device__ __forceinline__ void dequant_gemv_body(
       const int k = kSingle ? g0 * kGroup + 8 * c : min(g0 * kGroup + 8 * c, K - 8);
       b.x[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + k);
     }
+    if (kW4) {
+#pragma unroll
+      for (int p = 0; p < TPW; ++p)
+        b.m[p] = mtile[(size_t)(kSingle ? g0 + p : min(g0 + p, g_end - 1)) * 16];
+    }
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       const int g = kSingle ? g0 + p : min(g0 + p, g_end - 1);
 #pragma unroll
       for (int h = 0; h < kLoadsPerGroup; ++h)
         b.w[p][h] = __builtin_nontemporal_load(wtile + ((size_t)g * kLoadsPerGroup + h) * 64);
-    }
-    if (kW4) {
-#pragma unroll
-      for (int p = 0; p < TPW; ++p)
-        b.m[p] = mtile[(size_t)(kSingle ? g0 + p : min(g0 + p, g_end - 1)) * 16];
     }
     // the whole batch is in flight before anything else happens: left alone, the
     // instruction scheduler sinks loads towards their first use and turns one
@@ -188,10 +188,8 @@ __device__ __forceinline__ void dequant_gemv_body(
     else return *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
   };
   auto compute = [&](Batch& b, int g0) {
-    // The meta words are the last loads of the batch and their conversion is its
-    // first use: a wave's tiles arrive together, so waiting for all of the batch
-    // here costs nothing, and it keeps the scheduler from sinking those loads
-    // below an earlier wait (a second memory round trip).
+    // the meta words arrive before the weights (issued before them): scales and zero-points are ready when the
+    // first tile lands
     float sc[TPW], zc[TPW];
     if (kW4) {
 #pragma unroll
@@ -199,7 +197,6 @@ __device__ __forceinline__ void dequant_gemv_body(
         sc[p] = f16_bits_to_f32(b.m[p] & 0xFFFFu);
         zc[p] = f16_bits_to_f32(b.m[p] >> 16);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
     if (!kSingle) {
       stage(b);

@@ -536,7 +536,7 @@ def main() -> int:
             # HBM bytes per launch from separate rocprofv3 --pmc runs of this command
             # (FETCH_SIZE, WRITE_SIZE, each scaled by what a 64 MiB copy reads on the same counter)
             "traffic": GEMV_W4_4096_M1_HBM_BYTES,
-            "kernel": "ajq::dequant_gemv_kernel<8, 4, 1, true, true>",
+            "kernel": "ajq::dequant_gemv_kernel<8, 4, 1, true, true, true>",
             "algorithmic_bytes_per_launch": head["bytes_per_launch"],
             "avg_launch_us": head["us_per_launch"],
         },
