@@ -33,7 +33,7 @@ struct SkinnyBatch {
 // kEpi: the epilogue forms of dequant_gemv_epi_kernel (row scale of an RMSNorm applied to the outputs,
 // residual add with the next norm's preparation, SwiGLU gate on interleaved rows) for more rows than a GEMV
 // takes; ssq_in is [M][parts], ssq_out [M][N / 16].
-template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi>
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0>
 __device__ __forceinline__ void dequant_skinny_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
@@ -86,17 +86,10 @@ __device__ __forceinline__ void dequant_skinny_body(
   }
 
   // unconditional loads with clamped addresses: the number in flight is static
+  // Issue order: the activations (from L2: back first, vector loads return in issue order), the meta words,
+  // the weights.
   auto load = [&](Batch& b, int g0) {
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int p = 0; p < TPW; ++p) {
-        const int g = min(g0 + p, g_end - 1);
-#pragma unroll
-        for (int h = 0; h < kLoadsPerGroup; ++h)
-          b.w[t][p][h] = __builtin_nontemporal_load(wtile[t] + ((size_t)g * kLoadsPerGroup + h) * 64);
-      }
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const int v = lane + 64 * i;
@@ -110,6 +103,15 @@ __device__ __forceinline__ void dequant_skinny_body(
 #pragma unroll
         for (int p = 0; p < TPW; ++p) b.m[t][p] = mtile[t][(size_t)min(g0 + p, g_end - 1) * 16];
     }
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int p = 0; p < TPW; ++p) {
+        const int g = min(g0 + p, g_end - 1);
+#pragma unroll
+        for (int h = 0; h < kLoadsPerGroup; ++h)
+          b.w[t][p][h] = __builtin_nontemporal_load(wtile[t] + ((size_t)g * kLoadsPerGroup + h) * 64);
+      }
     __builtin_amdgcn_sched_barrier(0);
   };
 
@@ -132,7 +134,6 @@ __device__ __forceinline__ void dequant_skinny_body(
           sc[t][p] = f16_bits_to_f32(b.m[t][p] & 0xFFFFu);
           zc[t][p] = f16_bits_to_f32(b.m[t][p] >> 16);
         }
-      __builtin_amdgcn_sched_barrier(0);
     }
     // LDS operations of one wave execute in order: the previous batch's reads are done
 #pragma unroll
@@ -211,8 +212,20 @@ __device__ __forceinline__ void dequant_skinny_body(
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  if (g_begin >= g_end) epilogue_loads();
-  if (g_begin < g_end) {
+  if constexpr (kBatches > 0) {
+    // K == kWaves * TPW * kBatches * 128: every wave runs exactly kBatches full batches, the loop is straight-line
+    // code and the number of loads in flight is known at every wait (a batch is computed while the next travels)
+    Batch b[2];
+    load(b[0], g_begin);
+    epilogue_loads();
+#pragma unroll
+    for (int i = 0; i < kBatches; ++i) {
+      if (i + 1 < kBatches) load(b[(i + 1) & 1], g_begin + (i + 1) * TPW);
+      compute(b[i & 1], g_begin + i * TPW);
+    }
+  } else if (g_begin >= g_end) {
+    epilogue_loads();
+  } else {
     Batch b0, b1;
     load(b0, g_begin);
     epilogue_loads();
@@ -309,18 +322,18 @@ __device__ __forceinline__ void dequant_skinny_body(
   }
 }
 
-template <int kWaves, int TPW, int MROWS, int NT, bool kW4>
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kBatches = 0>
 __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8) {
-  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, 0>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, 0, kBatches>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
 }
 
-template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi>
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0>
 __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_epi_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
-  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, kEpi>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, kEpi, kBatches>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
 }
 
 // LDS bytes of one workgroup of dequant_skinny_kernel<kWaves, TPW, MROWS, *>
