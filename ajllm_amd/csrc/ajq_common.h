@@ -102,6 +102,20 @@ template <int kRor>
 __device__ __forceinline__ float row_ror(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + kRor, 0xF, 0xF, false));
 }
+// a / b, correctly rounded, for many a over one b: with y the correctly rounded 1 / b (one IEEE division per b),
+// q0 = a * y is within an ulp of the quotient, the FMA r = a - q0 * b is exact, and q0 + r * y rounds to the correctly
+// rounded a / b (Markstein's theorem).  Three instructions per quotient instead of the ten of the division expansion;
+// bit for bit a / b on normal operands (checked on 10^9 random pairs on the GPU; a zero numerator may come out with
+// the other sign).
+struct Divisor {
+  float b, y;
+  __device__ __forceinline__ explicit Divisor(float b_) : b(b_), y(1.0f / b_) {}
+  __device__ __forceinline__ float divide(float a) const {
+    const float q0 = a * y;
+    const float r = __builtin_fmaf(-q0, b, a);
+    return __builtin_fmaf(r, y, q0);
+  }
+};
 __device__ __forceinline__ float team_sum16(float v) {
   v += row_ror<8>(v);
   v += row_ror<4>(v);

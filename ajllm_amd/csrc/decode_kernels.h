@@ -59,11 +59,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ hi
   if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
   __syncthreads();
   ss = (part[0] + part[1]) + (part[2] + part[3]);
-  const float rms = sqrtf(ss / (float)D + eps);
+  const Divisor by_rms(sqrtf(ss / (float)D + eps));  // (h / rms) * gain, the division as the model code has it
   uint2* o2 = reinterpret_cast<uint2*>(out + (size_t)b * D);
   auto put = [&](int i, const float4& v, const float4& gg) {
-    const uint32_t lo = pack2_bf16((v.x / rms) * gg.x, (v.y / rms) * gg.y);
-    const uint32_t hi = pack2_bf16((v.z / rms) * gg.z, (v.w / rms) * gg.w);
+    const uint32_t lo = pack2_bf16(by_rms.divide(v.x) * gg.x, by_rms.divide(v.y) * gg.y);
+    const uint32_t hi = pack2_bf16(by_rms.divide(v.z) * gg.z, by_rms.divide(v.w) * gg.w);
     o2[i] = uint2{lo, hi};
   };
 #pragma unroll

@@ -197,12 +197,12 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
       float total = 0.f;
 #pragma unroll
       for (int u = 0; u < kWaves; ++u) total += part[u];
-      const float rms = sqrtf(total / (float)K + eps);
+      const Divisor by_rms(sqrtf(total / (float)K + eps));
       const float4 g0v = a2[i][0], g1v = a2[i][1];
-      xv[i][0] = (xv[i][0] / rms) * g0v.x; xv[i][1] = (xv[i][1] / rms) * g0v.y;
-      xv[i][2] = (xv[i][2] / rms) * g0v.z; xv[i][3] = (xv[i][3] / rms) * g0v.w;
-      xv[i][4] = (xv[i][4] / rms) * g1v.x; xv[i][5] = (xv[i][5] / rms) * g1v.y;
-      xv[i][6] = (xv[i][6] / rms) * g1v.z; xv[i][7] = (xv[i][7] / rms) * g1v.w;
+      xv[i][0] = by_rms.divide(xv[i][0]) * g0v.x; xv[i][1] = by_rms.divide(xv[i][1]) * g0v.y;
+      xv[i][2] = by_rms.divide(xv[i][2]) * g0v.z; xv[i][3] = by_rms.divide(xv[i][3]) * g0v.w;
+      xv[i][4] = by_rms.divide(xv[i][4]) * g1v.x; xv[i][5] = by_rms.divide(xv[i][5]) * g1v.y;
+      xv[i][6] = by_rms.divide(xv[i][6]) * g1v.z; xv[i][7] = by_rms.divide(xv[i][7]) * g1v.w;
     }
   } else if (kPro == kProNormSums) {
     // a row's total in its first lane, then through the wave's own LDS words to whoever holds a piece of the row
@@ -222,12 +222,12 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_pro_kernel(
     for (int i = 0; i < kXLoads; ++i) {
       const int v = min(lane + 64 * i, kVecs - 1);
       // one row: every lane already holds its total
-      const float rms = sqrtf((MROWS > 1 ? ssq[(v / kVecPerRow) * kWaves + wave] : total) / (float)K + eps);
+      const Divisor by_rms(sqrtf((MROWS > 1 ? ssq[(v / kVecPerRow) * kWaves + wave] : total) / (float)K + eps));
       const float4 h0 = a0[i][0], h1 = a0[i][1], g0v = a2[i][0], g1v = a2[i][1];
-      xv[i][0] = (h0.x / rms) * g0v.x; xv[i][1] = (h0.y / rms) * g0v.y;
-      xv[i][2] = (h0.z / rms) * g0v.z; xv[i][3] = (h0.w / rms) * g0v.w;
-      xv[i][4] = (h1.x / rms) * g1v.x; xv[i][5] = (h1.y / rms) * g1v.y;
-      xv[i][6] = (h1.z / rms) * g1v.z; xv[i][7] = (h1.w / rms) * g1v.w;
+      xv[i][0] = by_rms.divide(h0.x) * g0v.x; xv[i][1] = by_rms.divide(h0.y) * g0v.y;
+      xv[i][2] = by_rms.divide(h0.z) * g0v.z; xv[i][3] = by_rms.divide(h0.w) * g0v.w;
+      xv[i][4] = by_rms.divide(h1.x) * g1v.x; xv[i][5] = by_rms.divide(h1.y) * g1v.y;
+      xv[i][6] = by_rms.divide(h1.z) * g1v.z; xv[i][7] = by_rms.divide(h1.w) * g1v.w;
     }
   } else if (kPro == kProGate) {
 #pragma unroll
