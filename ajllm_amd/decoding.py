@@ -323,10 +323,11 @@ class FusedDecoder(GraphDecoder):
     """GraphDecoder whose step runs on this library's kernels only: fused q|k|v and w1|w3
     matmuls, residual add + RMSNorm, RoPE + cache write + single-query attention in one launch
     and the SwiGLU gate (``ajq_add_rmsnorm`` / ``ajq_attn_step`` / ``ajq_swiglu``), the greedy pick
-    with the embedding lookup and the step counters (``ajq_greedy_pick``).  Five launches per layer
-    at batch 1 (q|k|v with the norm, attention, output projection with the merge of the attention's
-    row chunks, w1|w3 with the gate, w2: ``launches_per_step``); six above batch 4, where the attention's merge is a
-    launch of its own.  The norm's row scale, the residual add and the gate ride in the matmuls' epilogues (GEMV kernel
+    with the embedding lookup and the step counters (``ajq_greedy_pick``).  Six launches per layer
+    (q|k|v with the norm, attention, the merge of the attention's row chunks, output projection, w1|w3 with the
+    gate, w2: ``launches_per_step``); five where the attention has one chunk per head or where ``fuse_merge`` is set
+    and the output projection merges the chunks on its way in (an option: measured slower than the launch at every
+    batch).  The norm's row scale, the residual add and the gate ride in the matmuls' epilogues (GEMV kernel
     up to 16 rows, weight-streaming kernel up to 255); nine launches per layer where those forms are not built.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
@@ -398,11 +399,15 @@ class FusedDecoder(GraphDecoder):
         self.fuse_norm = batch <= 4 and self.head.fusable(batch)
         self.fuse_gate = (batch == 1 and self.layers[0]["w2"].fusable(batch)
                           and self.layers[0]["w13"].rows16 == 2 * self.d_ff)
-        # the output projection merges the attention's row chunks on its way in where that is built
-        # (small batches; one launch less per layer)
+        # The output projection can merge the attention's row chunks on its way in where that is built (small
+        # batches; one launch less per layer): ``fuse_merge``, off by default.  Every workgroup of that GEMV re-reads
+        # every chunk of every head, and a dependent launch costs little more than its kernel in a replayed graph:
+        # measured on the 12-layer model, the merge as a launch of its own is faster at every batch (0.309 against
+        # 0.314 ms per step at batch 1, 0.364 against 0.398 at batch 2, 0.386 against 0.469 at batch 3).  Set it to
+        # True (where ``merge_splits`` > 0) before the first ``generate`` to have the merging projection.
         self.merge_splits = (self.layers[0]["o"].merge_splits(batch)
                              if self.layers[0]["o"].in_features == d and self.head_dim == 128 else 0)
-        self.fuse_merge = self.merge_splits > 0
+        self.fuse_merge = False
         # Larger batches (every workgroup would re-read the fp32 sources of all rows): the norm's row scale
         # is applied to the OUTPUTS of q|k|v, w1|w3 and the head instead, the output projection and w2 add
         # the residual and prepare the next norm on their way out, and w1|w3 (rows interleaved in blocks
@@ -434,10 +439,6 @@ class FusedDecoder(GraphDecoder):
             # the step's very first norm rides in layer 0's q|k|v where built
             self.first_norm_fused = self.fuse_norm and not self.norm_launch
             self.fuse_norm = self.fuse_gate = False
-            # the merge prologue re-reads every chunk of every head in every workgroup: with the cheaper epilogue
-            # kernels around it, it only pays at batch 1 (measured: 0.41 / 0.50 / 0.52 ms per step with it at
-            # batch 2 / 3 / 4 against 0.41 / 0.45 / 0.48 with the merge as a launch of its own)
-            self.fuse_merge = self.fuse_merge and batch == 1
             for w, layer in zip(self.layers, model.layers):
                 w["w13i"] = _FusedLinear.interleaved_gate(layer.feed_forward.w1, layer.feed_forward.w3)
             self.xt = torch.zeros((batch, d), dtype=torch.bfloat16, device=dev)

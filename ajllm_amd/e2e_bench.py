@@ -219,8 +219,8 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
                     "library's kernels only (fused q|k|v and w1|w3 GEMVs, the residual adds and the SwiGLU gate in "
                     "the matmuls' epilogues, the RMSNorms formed on the consumers' way in up to batch 4 and as "
                     "launches of their own above, RoPE + cache write + single-query attention in one kernel, its "
-                    "row chunks merged by the output projection at batch 1 and by a launch above, greedy pick + "
-                    "embedding row + step counters in one launch)",
+                    "row chunks merged by a launch of its own, greedy pick + embedding row + step counters in one "
+                    "launch)",
         }
         log("decode", r)
         results.append(r)

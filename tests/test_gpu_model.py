@@ -841,11 +841,13 @@ def test_fused_decoder_with_gemv_epilogues_matches_the_oracle_model(cuda, scheme
         assert dec.exact_norm == (rounding == "reference")
         # reference rounding above batch 4: the norms are launches of their own again (eight per layer)
         assert dec.norm_launch == (rounding == "reference" and batch > 4)
-        assert dec.fuse_merge == (batch == 1) and dec.first_norm_fused == (batch <= 4)
+        assert not dec.fuse_merge and dec.first_norm_fused == (batch <= 4)
+        if batch == 1 and rounding == "before_scale":
+            dec.fuse_merge = True   # the output projection that merges the attention's row chunks (an option)
         if dec.norm_launch:
             assert dec.launches_per_step() == 8 * 2 + 3
         else:
-            assert dec.launches_per_step() == (5 if batch == 1 else 6) * 2 + (2 if batch <= 4 else 3)
+            assert dec.launches_per_step() == (5 if dec.fuse_merge else 6) * 2 + (2 if batch <= 4 else 3)
 
     _fused_decoder_against_the_oracle_model(cuda, scheme, batch, model, configure, rounding)
 
