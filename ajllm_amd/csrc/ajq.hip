@@ -1286,7 +1286,8 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H, int Hkv,
                      int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream) {
   if (!q || !kcache || !vcache || !out) return fail(AJQ_ERR_NULL, "ajq_attn_prefill: null pointer argument");
-  if (head_dim != 128) return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (only 128 is built)", head_dim);
+  if (head_dim != 128 && head_dim != 64)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (128 and 64 are built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || T < 1 || start < 0 || (long long)start + T > max_len ||
       (long long)B * H > 65535)
     return fail(AJQ_ERR_SHAPE, "ajq_attn_prefill: unsupported shape (B=%d H=%d Hkv=%d T=%d start=%d max_len=%d)", B, H,
@@ -1299,14 +1300,19 @@ int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int
   if (!aligned16(q) || !aligned16(kcache) || !aligned16(vcache) || !aligned16(out))
     return fail(AJQ_ERR_ALIGN, "ajq_attn_prefill: q, the caches and out must be 16-byte aligned");
   const dim3 grid((unsigned)(((T + kPfBQ - 1) / kPfBQ) * B * H));  // (the kernel orders the work by cost)
-  if (cache_dtype == AJQ_KV_F32)
-    hipLaunchKernelGGL(attn_prefill_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, q,
-                       reinterpret_cast<const float*>(kcache), reinterpret_cast<const float*>(vcache), H, Hkv, T, start,
-                       max_len, out, out_bf16);
-  else
-    hipLaunchKernelGGL(attn_prefill_kernel<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, q,
-                       reinterpret_cast<const uint16_t*>(kcache), reinterpret_cast<const uint16_t*>(vcache), H, Hkv, T,
-                       start, max_len, out, out_bf16);
+  const bool f32 = cache_dtype == AJQ_KV_F32;
+  auto launch = [&](auto kernel, auto* cache_element) {
+    using CacheT = std::remove_pointer_t<decltype(cache_element)>;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), 0, (hipStream_t)stream, q, reinterpret_cast<const CacheT*>(kcache),
+                       reinterpret_cast<const CacheT*>(vcache), H, Hkv, T, start, max_len, out, out_bf16);
+  };
+  if (head_dim == 128) {
+    if (f32) launch(attn_prefill_kernel<float, 128>, (float*)nullptr);
+    else launch(attn_prefill_kernel<uint16_t, 128>, (uint16_t*)nullptr);
+  } else {
+    if (f32) launch(attn_prefill_kernel<float, 64>, (float*)nullptr);
+    else launch(attn_prefill_kernel<uint16_t, 64>, (uint16_t*)nullptr);
+  }
   return check_launch("ajq_attn_prefill");
 }
 

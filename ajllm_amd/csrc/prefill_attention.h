@@ -1,18 +1,19 @@
-// Causal self-attention for a block of T new positions (prefill), head_dim 128, on bf16 MFMA
+// Causal self-attention for a block of T new positions (prefill), head_dim HD = 128 or 64, on bf16 MFMA
 // with an online softmax: the T x (start + T) score matrix is never materialised.
 //
-//   out[b, t, h, :] = softmax_j( q[b, h, t, :] . k[b, hk, j, :] / sqrt(128) ) v[b, hk, j, :],
+//   out[b, t, h, :] = softmax_j( q[b, h, t, :] . k[b, hk, j, :] / sqrt(HD) ) v[b, hk, j, :],
 //   j <= start + t,   hk = h / (H / Hkv)
 //
-// q is fp32 [B, H, T, 128] (already rotated); keys and values are read where the model keeps
-// them, in the caches [B, Hkv, max_len, 128] (fp32 or bf16), rows 0 .. start + T - 1; out is
-// fp32 or bf16 [B, T, H * 128], the layout the output projection takes.
+// q is fp32 [B, H, T, HD] (already rotated); keys and values are read where the model keeps
+// them, in the caches [B, Hkv, max_len, HD] (fp32 or bf16), rows 0 .. start + T - 1; out is
+// fp32 or bf16 [B, T, H * HD], the layout the output projection takes.  (The layouts below are
+// written out for HD = 128; with 64 a row is 128 B = 8 chunks = 4 segments and there are two k-steps.)
 //
 // A workgroup of 4 waves owns 128 query rows of one (b, h), a wave two groups of 16 of them
 // (every key and value fragment read from LDS meets both), and walks the keys in blocks of 64.
 // Both products run transposed so that no operand changes layout between them:
 //   S^T = K Q^T :  A = 16 keys x 32 dims from the row-major key tile in LDS, B = the wave's Q
-//                  fragments (registers, bf16, pre-scaled by log2(e) / sqrt(128)); lane
+//                  fragments (registers, bf16, pre-scaled by log2(e) / sqrt(HD)); lane
 //                  (g = l / 16, r = l % 16) receives keys 4g..4g+3 of query row r.  The
 //                  accumulator starts at minus the row's reference point, so the MFMA result is
 //                  the exponent itself.
@@ -39,8 +40,7 @@ namespace ajq {
 
 constexpr float kPfSlack = 8.0f;          // log2 of how far a row's exponents may exceed its reference point
 constexpr float kPfTrigger = 4096.0f;     // lane sum of 16 probabilities above which the reference point is revisited
-constexpr int kPfBQ = 128, kPfBK = 64, kPfHD = 128;
-constexpr int kPfTileBytes = kPfBK * kPfHD * 2;  // 16 KiB: one block of keys (or values) as bf16
+constexpr int kPfBQ = 128, kPfBK = 64;
 
 __device__ __forceinline__ u32x4_t pack8_bf16(const float* v) {
   return u32x4_t{pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]), pack2_bf16(v[4], v[5]), pack2_bf16(v[6], v[7])};
@@ -96,10 +96,17 @@ __device__ __forceinline__ u32x2_t pf_read_tr(uint32_t address) {
 __device__ __forceinline__ u32x4_t pf_read128(uint32_t address) { return *(pf_lds_u32x4_t*)address; }
 #pragma clang diagnostic pop
 
-template <typename CacheT>
+template <typename CacheT, int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
                                                            const CacheT* __restrict__ vcache, int H, int Hkv, int T,
                                                            int start, int max_len, void* __restrict__ out, int out_bf16) {
+  static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+  constexpr int kPfHD = HD;
+  constexpr int RB = 2 * HD;          // bytes of a key (value) row as bf16
+  constexpr int C = HD / 8;           // 16-byte chunks per row
+  constexpr int KS = HD / 32;         // k-steps of the first product; also the parts a block's DMA is issued in
+  constexpr int TT = HD / 16;         // 32-byte segments per row = 16-dim output tiles
+  constexpr int kPfTileBytes = kPfBK * RB;  // one block of keys (or values) as bf16: 16 KiB at HD = 128
   // LDS map (byte addresses relative to lds0, the array's LDS address, which is 0 because the kernel
   // declares no other LDS; naming it also keeps the array allocated when nothing else refers to
   // it): two stages of a key tile and a value tile, 16 KiB each.
@@ -129,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   }
   const int b = bh / H, h = bh % H, hk = h / (H / Hkv);
   const int q0 = qb * kPfBQ;
-  const float qscale = 1.4426950408889634f * 0.08838834764831845f;  // log2(e) / sqrt(128)
+  const float qscale = 1.4426950408889634f * (HD == 128 ? 0.08838834764831845f : 0.125f);  // log2(e) / sqrt(HD)
 
   const CacheT* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
   const CacheT* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
@@ -140,82 +147,85 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
 
   float m_run[2], l_run[2];
   f32x4_t negm[2];
-  f32x4_t o[2][8];
+  f32x4_t o[2][TT];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     m_run[u] = 0.f;
     l_run[u] = 0.f;
     negm[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 8; ++t) o[u][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < TT; ++t) o[u][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
   // ---- Keys and values on their way into LDS.
   // bf16 caches: global -> LDS directly, one block ahead.  A wave-wide request fills 1 KiB = 4 key
-  // rows; wave w takes rows 4 w .. 4 w + 3 of every group of 16, so (row & 15) = 4 w + lane / 16 is
+  // rows (8 rows at HD = 64); wave w takes rows 4 w .. 4 w + 3 of every group of 16, so (row & 15) = 4 w + lane / 16 is
   // fixed per lane and the chunk it must fetch for its slot is too.
   // fp32 caches: through registers (converted on the way), one block in registers while the
   // previous one is being read: chunk ci = tid + 256 i (i < 4) is (key ci / 16, dims 8 (ci % 16) ..).
   // Rows past the filled part of the cache repeat its last row (finite values; those keys are masked).
   constexpr bool kDma = sizeof(CacheT) == 2;
-  const int krow = 4 * wave + (lane >> 4), slot = lane & 15;
-  const uint32_t k_chunk = (uint32_t)(slot ^ krow);
-  const uint32_t v_chunk = (uint32_t)((((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1));
-  // part i (0 .. 3) of block jblk: this wave's 4 key rows and 4 value rows of the i-th group of 16
+  constexpr int kReqRows = 1024 / RB;  // key rows of one wave-wide request: 4 (HD = 128) or 8
+  const int krow = kReqRows * wave + lane / C, slot = lane % C;
+  const uint32_t k_chunk = (uint32_t)(slot ^ (krow & (C - 1)));
+  const uint32_t v_chunk = (uint32_t)((((slot >> 1) ^ (krow & (TT - 1))) << 1) | (slot & 1));
+  // part i (0 .. KS - 1) of block jblk: this wave's kReqRows key rows and value rows of the i-th group of 4 * kReqRows
   auto issue_dma = [&](int jblk, int i) {
     const int kb0 = jblk * kPfBK;
     const uint32_t stage = lds0 + (uint32_t)((jblk & 1) * 2 * kPfTileBytes);
     const uint32_t k_to = stage + (uint32_t)((wave + 4 * i) * 1024), v_to = k_to + (uint32_t)kPfTileBytes;
     if (kb0 + kPfBK <= kv_len) {
-      const size_t row0 = (size_t)(kb0 + 16 * i) * 256;
-      dma16(reinterpret_cast<const char*>(kbase) + row0, (uint32_t)(krow * 256) + k_chunk * 16u, k_to);
-      dma16(reinterpret_cast<const char*>(vbase) + row0, (uint32_t)(krow * 256) + v_chunk * 16u, v_to);
+      const size_t row0 = (size_t)(kb0 + 4 * kReqRows * i) * RB;
+      dma16(reinterpret_cast<const char*>(kbase) + row0, (uint32_t)(krow * RB) + k_chunk * 16u, k_to);
+      dma16(reinterpret_cast<const char*>(vbase) + row0, (uint32_t)(krow * RB) + v_chunk * 16u, v_to);
     } else {
-      const uint32_t row = (uint32_t)min(kb0 + 16 * i + krow, kv_len - 1) * 256u;
+      const uint32_t row = (uint32_t)min(kb0 + 4 * kReqRows * i + krow, kv_len - 1) * (uint32_t)RB;
       dma16(kbase, row + k_chunk * 16u, k_to);
       dma16(vbase, row + v_chunk * 16u, v_to);
     }
   };
   typedef decltype(load8_raw(kbase)) raw8_t;
-  raw8_t kraw[kDma ? 1 : 4], vraw[kDma ? 1 : 4];
-  uint32_t k_st[kDma ? 1 : 4], v_st[kDma ? 1 : 4];
+  constexpr int kRegParts = kDma ? 0 : kPfBK * C / 256;  // 16-byte chunks of a block per thread: 4 (HD = 128) or 2
+  raw8_t kraw[kDma ? 1 : kRegParts], vraw[kDma ? 1 : kRegParts];
+  uint32_t k_st[kDma ? 1 : kRegParts], v_st[kDma ? 1 : kRegParts];
   auto fetch = [&](int kb0) {
 #pragma unroll
-    for (int i = 0; i < (kDma ? 0 : 4); ++i) {
+    for (int i = 0; i < kRegParts; ++i) {
       const int ci = threadIdx.x + 256 * i;
-      const size_t at = (size_t)min(kb0 + (ci >> 4), kv_len - 1) * kPfHD + 8 * (ci & 15);
+      const size_t at = (size_t)min(kb0 + ci / C, kv_len - 1) * kPfHD + 8 * (ci % C);
       kraw[i] = load8_raw(kbase + at);
       vraw[i] = load8_raw(vbase + at);
     }
   };
 #pragma unroll
-  for (int i = 0; i < (kDma ? 0 : 4); ++i) {
-    const int ci = threadIdx.x + 256 * i, k = ci >> 4, c = ci & 15;
-    k_st[i] = (uint32_t)(k * 256 + 16 * (c ^ (k & 15)));
-    v_st[i] = (uint32_t)(kPfTileBytes + k * 256 + 16 * ((((c >> 1) ^ (k & 7)) << 1) | (c & 1)));
+  for (int i = 0; i < kRegParts; ++i) {
+    const int ci = threadIdx.x + 256 * i, k = ci / C, c = ci % C;
+    k_st[i] = (uint32_t)(k * RB + 16 * (c ^ (k & (C - 1))));
+    v_st[i] = (uint32_t)(kPfTileBytes + k * RB + 16 * ((((c >> 1) ^ (k & (TT - 1))) << 1) | (c & 1)));
   }
   auto lay_down = [&](int stage) {
 #pragma unroll
-    for (int i = 0; i < (kDma ? 0 : 4); ++i) {
+    for (int i = 0; i < kRegParts; ++i) {
       *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + k_st[i]) = to_bf16x8(kraw[i]);
       *reinterpret_cast<u32x4_t*>(lds + stage * 2 * kPfTileBytes + v_st[i]) = to_bf16x8(vraw[i]);
     }
   };
   // ---- LDS read addresses (of the stage being read; flipped to the other stage after every block).
   // key fragment (tile jb, k-step s): row 16 jb + r, chunk 4 s + g  ->  (16 jb + r) * 256 + 16 * ((4 s + g) ^ r)
-  uint32_t k_rd[4];
+  uint32_t k_rd[KS];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) k_rd[s] = lds0 + (uint32_t)(r * 256 + 16 * ((4 * s + g) ^ r));
+  for (int s = 0; s < KS; ++s) k_rd[s] = lds0 + (uint32_t)(r * RB + 16 * ((4 * s + g) ^ (r & (C - 1))));
   // value fragment (half hf, slots 4 w2 .. 4 w2 + 3, dims 16 t ..): this lane addresses 8 bytes of key
   // 32 hf + 16 w2 + 4 g + (r >> 2): piece (r & 3) of the 32-byte segment t, which sits in slot t ^ (key & 7)
   const int vkey = 4 * g + (r >> 2);  // (16 w2 and 32 hf do not change key & 7)
-  uint32_t v_rd[8];
+  uint32_t v_rd[TT];
 #pragma unroll
-  for (int t = 0; t < 8; ++t) v_rd[t] = lds0 + (uint32_t)(kPfTileBytes + vkey * 256 + 32 * (t ^ (vkey & 7)) + 8 * (r & 3));
+  for (int t = 0; t < TT; ++t)
+    v_rd[t] = lds0 + (uint32_t)(kPfTileBytes + vkey * RB + 32 * (t ^ (vkey & (TT - 1))) + 8 * (r & 3));
 
   if (kDma) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) issue_dma(0, i);
+    for (int i = 0; i < KS; ++i) issue_dma(0, i);
   } else {
     fetch(0);
     lay_down(0);
@@ -225,14 +235,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   // Q fragments of the wave's two groups of 16 rows: Q[qrow][32 s + 8 g .. + 8), scaled, bf16.
   // Group u of wave w holds rows q0 + 32 w + 16 u .. + 15; this lane's row of it is qrow[u].
   int qrow[2], q_pos[2];
-  u32x4_t qf[2][4];
+  u32x4_t qf[2][KS];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     qrow[u] = q0 + 32 * wave + 16 * u + r;
     q_pos[u] = start + qrow[u];
     const float* qp = q + ((size_t)bh * T + min(qrow[u], T - 1)) * kPfHD + 8 * g;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < KS; ++s) {
       const float4 a = reinterpret_cast<const float4*>(qp + 32 * s)[0], c = reinterpret_cast<const float4*>(qp + 32 * s)[1];
       const float v[8] = {a.x * qscale, a.y * qscale, a.z * qscale, a.w * qscale,
                           c.x * qscale, c.y * qscale, c.z * qscale, c.w * qscale};
@@ -253,7 +263,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
       if (kDma) {
         if (kb0 > wave_last_pos) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) issue_dma(j + 1, i);
+          for (int i = 0; i < KS; ++i) issue_dma(j + 1, i);
         }
       } else {
         lay_down((j + 1) & 1);
@@ -268,22 +278,22 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
       f32x4_t sc[2][4];
       u32x4_t ka[4];
 #pragma unroll
-      for (int jb = 0; jb < 4; ++jb) ka[jb] = pf_read128(k_rd[0] + (uint32_t)(jb * 16 * 256));
+      for (int jb = 0; jb < 4; ++jb) ka[jb] = pf_read128(k_rd[0] + (uint32_t)(jb * 16 * RB));
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+      for (int s = 0; s < KS; ++s) {
         u32x4_t kn[4];
-        if (kDma && s < 3) {  // (the fp32 path has no registers to spare for a second set)
+        if (kDma && s < KS - 1) {  // (the fp32 path has no registers to spare for a second set)
 #pragma unroll
-          for (int jb = 0; jb < 4; ++jb) kn[jb] = pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
+          for (int jb = 0; jb < 4; ++jb) kn[jb] = pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * RB));
         }
 #pragma unroll
         for (int jb = 0; jb < 4; ++jb)
 #pragma unroll
           for (int u = 0; u < 2; ++u) sc[u][jb] = mfma16(ka[jb], qf[u][s], s == 0 ? negm[u] : sc[u][jb]);
         if (kDma && more) issue_dma(j + 1, s);
-        if (s < 3) {
+        if (s < KS - 1) {
 #pragma unroll
-          for (int jb = 0; jb < 4; ++jb) ka[jb] = kDma ? kn[jb] : pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * 256));
+          for (int jb = 0; jb < 4; ++jb) ka[jb] = kDma ? kn[jb] : pf_read128(k_rd[s + 1] + (uint32_t)(jb * 16 * RB));
         }
       }
       // only blocks that reach past the wave's first query position need the causal mask
@@ -327,7 +337,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
           negm[u] = f32x4_t{-m_run[u], -m_run[u], -m_run[u], -m_run[u]};
           l_run[u] *= corr;
 #pragma unroll
-          for (int t = 0; t < 8; ++t) o[u][t] *= corr;
+          for (int t = 0; t < TT; ++t) o[u][t] *= corr;
         }
         l_run[u] += psum;
         pf[u][0] = pack8_bf16(&p[0]);
@@ -336,9 +346,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
       // ---- O^T[hd 16 t + 4 g + i][qrow] += sum over the keys of each 32-key half; a value fragment
       // (two transposing reads: the half's first and second 16-key tile) meets both query groups.
       // The second half's fragments are requested as the first half's are consumed.
-      constexpr int kRing = kDma ? 8 : 4;  // fragments in flight (the fp32 path has fewer registers to spare)
-      auto v_lo = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256)); };
-      auto v_hi = [&](int i) { return pf_read_tr(v_rd[i & 7] + (uint32_t)((i >> 3) * 32 * 256 + 16 * 256)); };
+      constexpr int kRing = kDma ? (TT < 8 ? TT : 8) : 4;  // fragments in flight (the fp32 path has fewer registers to spare)
+      auto v_lo = [&](int i) { return pf_read_tr(v_rd[i % TT] + (uint32_t)((i / TT) * 32 * RB)); };
+      auto v_hi = [&](int i) { return pf_read_tr(v_rd[i % TT] + (uint32_t)((i / TT) * 32 * RB + 16 * RB)); };
       u32x2_t vlo[kRing], vhi[kRing];
 #pragma unroll
       for (int i = 0; i < kRing; ++i) {
@@ -346,11 +356,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
         vhi[i] = v_hi(i);
       }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {  // i = 8 hf + t
+      for (int i = 0; i < 2 * TT; ++i) {  // i = TT hf + t
         const u32x4_t vf = {vlo[i % kRing].x, vlo[i % kRing].y, vhi[i % kRing].x, vhi[i % kRing].y};
 #pragma unroll
-        for (int u = 0; u < 2; ++u) o[u][i & 7] = mfma16(vf, pf[u][i >> 3], o[u][i & 7]);
-        if (i + kRing < 16) {
+        for (int u = 0; u < 2; ++u) o[u][i % TT] = mfma16(vf, pf[u][i / TT], o[u][i % TT]);
+        if (i + kRing < 2 * TT) {
           vlo[i % kRing] = v_lo(i + kRing);
           vhi[i % kRing] = v_hi(i + kRing);
         }
@@ -358,9 +368,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
     }
     // flip every read address to the other stage
 #pragma unroll
-    for (int s = 0; s < 4; ++s) k_rd[s] ^= (uint32_t)(2 * kPfTileBytes);
+    for (int s = 0; s < KS; ++s) k_rd[s] ^= (uint32_t)(2 * kPfTileBytes);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) v_rd[t] ^= (uint32_t)(2 * kPfTileBytes);
+    for (int t = 0; t < TT; ++t) v_rd[t] ^= (uint32_t)(2 * kPfTileBytes);
     // the next block must have landed and every wave must be done with this one
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -373,13 +383,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
     if (out_bf16) {
       uint16_t* dst = reinterpret_cast<uint16_t*>(out) + at;
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
+      for (int t = 0; t < TT; ++t)
         *reinterpret_cast<u32x2_t*>(dst + 16 * t) =
             u32x2_t{pack2_bf16(o[u][t][0] * inv, o[u][t][1] * inv), pack2_bf16(o[u][t][2] * inv, o[u][t][3] * inv)};
     } else {
       float* dst = reinterpret_cast<float*>(out) + at;
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
+      for (int t = 0; t < TT; ++t)
         *reinterpret_cast<float4*>(dst + 16 * t) =
             float4{o[u][t][0] * inv, o[u][t][1] * inv, o[u][t][2] * inv, o[u][t][3] * inv};
     }

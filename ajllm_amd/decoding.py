@@ -332,7 +332,7 @@ class FusedDecoder(GraphDecoder):
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
     head_dim 128 or 64 (64: the geometry of the reference's configs/models/transformer_medium.yaml; the attention's
-    merge is then always a launch of its own and ``prefill(fused=True)`` is refused), 1, 2 or 4 query heads per
+    merge is then always a launch of its own), 1, 2 or 4 query heads per
     cache head, a quantized ``lm_head`` of its own (``quantize_model_(..., untie_head=True)`` for tied embeddings),
     every linear a QuantLinear.  ``kv_dtype``: torch.float32 (default, the model's own dtype) or
     torch.bfloat16 (keys and values rounded to nearest even on write, half the cache traffic)."""
@@ -458,8 +458,6 @@ class FusedDecoder(GraphDecoder):
         if not fused:
             super().prefill(prompt, rows_per_pass)
         else:
-            if self.head_dim != 128:
-                raise ValueError("the library's prefill attention is built for head_dim 128; use fused=False")
             if prompt.shape[0] != self.batch or prompt.shape[1] >= self.max_len:
                 raise ValueError("prompt must be [batch, T] with T < max_len")
             prompt = prompt.to(self.device)
@@ -485,7 +483,7 @@ class FusedDecoder(GraphDecoder):
         d, m = self.model.d_model, rows * seq
         hidden = self.embedding[prompt.reshape(-1)]  # [rows * seq, d] fp32, row b * seq + t
         normed = torch.empty((m, d), dtype=torch.bfloat16, device=self.device)
-        q_rot = torch.empty((rows, self.heads, seq, 128), dtype=torch.float32, device=self.device)
+        q_rot = torch.empty((rows, self.heads, seq, self.head_dim), dtype=torch.float32, device=self.device)
         w13 = self.layers[0]["w13"]
         gate_in_gemm = w13.rows16 == 2 * self.d_ff and w13.gate_fusable(m)
         gated = None if gate_in_gemm else torch.empty((m, self.d_ff), dtype=torch.bfloat16, device=self.device)
@@ -497,11 +495,11 @@ class FusedDecoder(GraphDecoder):
             keys, values = self.cache.keys[index][first:first + rows], self.cache.values[index][first:first + rows]
             _lib.check(lib.ajq_rope_prefill(qkv.data_ptr(), w["cos"].data_ptr(), w["sin"].data_ptr(), q_rot.data_ptr(),
                                             keys.data_ptr(), values.data_ptr(), self.kv_flag, rows, seq, self.heads,
-                                            self.kv_heads, 128, 0, self.max_len, st), "rope_prefill")
+                                            self.kv_heads, self.head_dim, 0, self.max_len, st), "rope_prefill")
             del qkv
             attended = torch.empty((m, d), dtype=torch.bfloat16, device=self.device)
             _lib.check(lib.ajq_attn_prefill(q_rot.data_ptr(), keys.data_ptr(), values.data_ptr(), self.kv_flag, rows,
-                                            self.heads, self.kv_heads, seq, 0, self.max_len, 128, attended.data_ptr(),
+                                            self.heads, self.kv_heads, seq, 0, self.max_len, self.head_dim, attended.data_ptr(),
                                             _lib.AJQ_OUT_BF16, st), "attn_prefill")
             delta = w["o"](attended)
             del attended

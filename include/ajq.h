@@ -294,7 +294,7 @@ int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
  * rounding of the fp32 result).  Flash-attention arithmetic: bf16 MFMA products,
  * fp32 online softmax, no T x T matrix (scaled_dot_product_attention under a causal mask,
  * src/ajllm/modeling/attention.py:20-33,106-117; the reference's own tiled and Triton variants,
- * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128 only. */
+ * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128 or 64. */
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H,
                      int Hkv, int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream);
 
