@@ -215,7 +215,7 @@ def bench_decode(device, log=print, batches=(1, 8), scheme: str = "w4a16_g128") 
             "quant_linear_GB/s": packed / t_linear / 1e9,
             "packed_weight_bytes": packed,
             "launches_per_step": dec.launches_per_step(),
-            "loop": "one-token step replayed from a HIP graph, token fed back on the device; the step is this "
+            "loop": "one-token step replayed from a HIP graph (eight steps per graph launch), token fed back on the device; the step is this "
                     "library's kernels only (fused q|k|v and w1|w3 GEMVs, the residual adds and the SwiGLU gate in "
                     "the matmuls' epilogues, the RMSNorms formed on the consumers' way in up to batch 4 and as "
                     "launches of their own above, RoPE + cache write + single-query attention in one kernel, its "

@@ -376,6 +376,38 @@ def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads
         assert (got2.float() - got.float()).abs().max() <= 2 ** -6
 
 
+@pytest.mark.parametrize("batch", [1, 5])
+def test_several_steps_per_graph_give_the_tokens_of_one_step_per_graph(cuda, batch):
+    """FusedDecoder replays a graph of eight consecutive steps while eight tokens are still wanted and the
+    one-step graph for the rest: the same kernels in the same order, so the tokens equal those of a decoder
+    that replays one step at a time bit for bit, across calls, with eager work between the replays, and with
+    an end-of-sequence stop."""
+    torch.manual_seed(14)
+    model = modeling.TransformerLM(vocab_size=512, context_length=128, d_model=256, num_layers=2, num_heads=2,
+                                   d_ff=640).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w4a16_g128")
+    prompt = torch.randint(0, 512, (batch, 20), generator=torch.Generator().manual_seed(12)).to(cuda)
+    one = decoding.FusedDecoder(fast, batch, 100)
+    one.steps_per_graph = 1
+    many = decoding.FusedDecoder(fast, batch, 100)
+    assert many.steps_per_graph == 8
+    for dec in (one, many):
+        dec.prefill(prompt)
+    a1, b1 = one.generate(5), many.generate(5)          # eager step, both captures, a few single replays
+    assert one.graph_many is None and many.graph_many is not None
+    torch.cuda.synchronize()
+    _ = fast(prompt)                                       # unrelated eager work between replays
+    a2, b2 = one.generate(31), many.generate(31)        # 26 more: three graphs of eight and two single steps
+    a3, b3 = one.generate(70), many.generate(70)
+    assert torch.equal(a1, b1) and torch.equal(a2, b2) and torch.equal(a3, b3) and torch.equal(a3[:, :31], a2)
+    assert int(many.cache.position) == int(one.cache.position) == 20 + 70 - 1
+    eos = int(a3[0, 40])
+    for dec in (one, many):
+        dec.prefill(prompt)
+    assert torch.equal(one.generate(70, eos_token_id=eos, eos_check_every=5),
+                       many.generate(70, eos_token_id=eos, eos_check_every=5))
+
+
 @pytest.mark.parametrize("scheme,batch,kv_heads,kv_dtype,folded", [
     ("w4a16_g128", 1, 2, None, True), ("w4a16_g128", 5, 2, None, True), ("w8a16", 2, 2, None, True),
     ("w8a16", 32, 1, None, True), ("w4a16_g128", 20, 1, None, True), ("w4a16_g128", 3, 2, torch.bfloat16, True),
