@@ -38,8 +38,9 @@ class GraphDecoder:
         # a second graph of ``steps_per_graph`` consecutive steps, replayed while that many tokens are still
         # wanted (1: none; the step's state lives on the device, so steps chain inside one graph as they do
         # across replays)
-        self.steps_per_graph = 1
+        self.steps_per_graph = 1   # read when the graphs are captured (the first ``generate``)
         self.graph_many: torch.cuda.CUDAGraph | None = None
+        self.graph_many_steps = 0
         self.stream = torch.cuda.Stream(device=device)
 
     def _logits(self) -> torch.Tensor:
@@ -134,11 +135,11 @@ class GraphDecoder:
                         with torch.cuda.graph(many, stream=self.stream):
                             for _ in range(self.steps_per_graph):
                                 self._step()
-                        self.graph_many = many
+                        self.graph_many, self.graph_many_steps = many, self.steps_per_graph
             while self.produced < new_tokens:
-                if self.graph_many is not None and new_tokens - self.produced >= self.steps_per_graph:
+                if self.graph_many is not None and new_tokens - self.produced >= self.graph_many_steps:
                     self.graph_many.replay()
-                    self.produced += self.steps_per_graph
+                    self.produced += self.graph_many_steps
                 else:
                     self.graph.replay()
                     self.produced += 1
