@@ -17,15 +17,15 @@ def flash_prefill(q: torch.Tensor, keys: torch.Tensor, values: torch.Tensor, sta
                   out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
     """Causal attention of the ``T`` new positions ``start .. start + T - 1``.
 
-    ``q`` fp32 ``[B, H, T, hd]`` (rotated; hd 128 or 64); ``keys`` / ``values`` ``[B, Hkv, max_len, hd]`` fp32 or
+    ``q`` fp32 ``[B, H, T, hd]`` (rotated; hd 128, 64 or 32); ``keys`` / ``values`` ``[B, Hkv, max_len, hd]`` fp32 or
     bf16 whose rows ``0 .. start + T - 1`` are filled (a KV cache, or the keys and values themselves
     with ``start == 0``).  Returns ``[B, T, H * hd]`` in ``out_dtype`` (fp32, or bf16 = its rounding)."""
     if not q.is_cuda:
         raise ValueError("flash_prefill needs tensors on a ROCm device (there is no CPU path)")
     batch, heads, seq, hd = q.shape
     kv_heads, max_len = keys.shape[1], keys.shape[2]
-    if hd not in (128, 64) or keys.shape != values.shape or keys.shape[0] != batch or keys.shape[3] != hd:
-        raise ValueError("flash_prefill: q [B, H, T, hd] and caches [B, Hkv, max_len, hd] with hd 128 or 64 expected")
+    if hd not in (128, 64, 32) or keys.shape != values.shape or keys.shape[0] != batch or keys.shape[3] != hd:
+        raise ValueError("flash_prefill: q [B, H, T, hd] and caches [B, Hkv, max_len, hd] with hd 128, 64 or 32 expected")
     if keys.dtype not in (torch.float32, torch.bfloat16) or values.dtype != keys.dtype:
         raise ValueError("flash_prefill: the caches must be float32 or bfloat16")
     if not (keys.is_contiguous() and values.is_contiguous()):

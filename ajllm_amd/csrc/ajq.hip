@@ -1109,7 +1109,8 @@ auto pick_attn_hd(int R, int cache_dtype) {
 }
 template <bool kStep>
 auto pick_attn(int R, int cache_dtype, int head_dim) {
-  return head_dim == 64 ? pick_attn_hd<kStep, 64>(R, cache_dtype) : pick_attn_hd<kStep, 128>(R, cache_dtype);
+  return head_dim == 32 ? pick_attn_hd<kStep, 32>(R, cache_dtype)
+                        : head_dim == 64 ? pick_attn_hd<kStep, 64>(R, cache_dtype) : pick_attn_hd<kStep, 128>(R, cache_dtype);
 }
 }  // namespace
 
@@ -1189,8 +1190,8 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
                     int H, int Hkv, int head_dim, int max_len, uint16_t* out, void* workspace, size_t workspace_bytes,
                     void* stream) {
   if (!q || !kcache || !vcache || !pos || !out) return fail(AJQ_ERR_NULL, "ajq_attn_decode: null pointer argument");
-  if (head_dim != 128 && head_dim != 64)
-    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (128 and 64 are built)", head_dim);
+  if (head_dim != 128 && head_dim != 64 && head_dim != 32)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_decode: head_dim %d (128, 64 and 32 are built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "ajq_attn_decode: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", B, H, Hkv, max_len);
   const int R = H / Hkv;
@@ -1223,9 +1224,9 @@ int attn_step_impl(const char* name, const float* qkv, const float* cosine, cons
                    void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim, int max_len,
                    uint16_t* out, int max_splits, int* splits, void* workspace, size_t workspace_bytes, void* stream) {
   if (!qkv || !cosine || !sine || !pos || !kcache || !vcache) return fail(AJQ_ERR_NULL, "%s: null pointer argument", name);
-  if (head_dim != 128 && !(head_dim == 64 && out))
+  if (head_dim != 128 && !((head_dim == 64 || head_dim == 32) && out))
     return fail(AJQ_ERR_UNSUPPORTED, "%s: head_dim %d (128 is built%s)", name, head_dim,
-                out ? ", and 64" : "; unmerged partial results are read by ajq_w*a16_gemv_merge, which assumes it");
+                out ? ", 64 and 32 too" : "; unmerged partial results are read by ajq_w*a16_gemv_merge, which assumes it");
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || max_len < 1)
     return fail(AJQ_ERR_SHAPE, "%s: unsupported shape (B=%d H=%d Hkv=%d max_len=%d)", name, B, H, Hkv, max_len);
   const int R = H / Hkv;
@@ -1286,8 +1287,8 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H, int Hkv,
                      int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream) {
   if (!q || !kcache || !vcache || !out) return fail(AJQ_ERR_NULL, "ajq_attn_prefill: null pointer argument");
-  if (head_dim != 128 && head_dim != 64)
-    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (128 and 64 are built)", head_dim);
+  if (head_dim != 128 && head_dim != 64 && head_dim != 32)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_attn_prefill: head_dim %d (128, 64 and 32 are built)", head_dim);
   if (B < 1 || H < 1 || Hkv < 1 || H % Hkv != 0 || T < 1 || start < 0 || (long long)start + T > max_len ||
       (long long)B * H > 65535)
     return fail(AJQ_ERR_SHAPE, "ajq_attn_prefill: unsupported shape (B=%d H=%d Hkv=%d T=%d start=%d max_len=%d)", B, H,
@@ -1309,9 +1310,12 @@ int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int
   if (head_dim == 128) {
     if (f32) launch(attn_prefill_kernel<float, 128>, (float*)nullptr);
     else launch(attn_prefill_kernel<uint16_t, 128>, (uint16_t*)nullptr);
-  } else {
+  } else if (head_dim == 64) {
     if (f32) launch(attn_prefill_kernel<float, 64>, (float*)nullptr);
     else launch(attn_prefill_kernel<uint16_t, 64>, (uint16_t*)nullptr);
+  } else {
+    if (f32) launch(attn_prefill_kernel<float, 32>, (float*)nullptr);
+    else launch(attn_prefill_kernel<uint16_t, 32>, (uint16_t*)nullptr);
   }
   return check_launch("ajq_attn_prefill");
 }

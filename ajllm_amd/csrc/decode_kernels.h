@@ -168,12 +168,12 @@ __global__ __launch_bounds__(256) void rope_prefill_kernel(const float* __restri
 // sums start on a 16-byte boundary so that a GEMV prologue can fetch them with 128-bit loads.
 constexpr int attn_partial_stride(int hd) { return 4 + hd; }
 constexpr int kAttnPartialStride = attn_partial_stride(128);
-// Which HD / 16 of a row's dimensions lane c of a team holds (DPL of them, 8 or 4), and how it fetches them.
+// Which HD / 16 of a row's dimensions lane c of a team holds (DPL of them: 8, 4 or 2), and how it fetches them.
 // 8 per lane, bf16 rows (256 B): 8c .. 8c+7, one 128-bit load.  8 per lane, fp32 rows (512 B): 4c .. 4c+3
 // and 64+4c .. 64+4c+3, so each of a team's two 128-bit loads covers 256 contiguous bytes.  4 per lane:
-// 4c .. 4c+3, one 128-bit (fp32) or 64-bit (bf16) load.
+// 4c .. 4c+3, one 128-bit (fp32) or 64-bit (bf16) load.  2 per lane: 2c, 2c+1, one 64-bit or 32-bit load.
 template <typename CacheT, int HD> struct LaneDims {
-  static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+  static_assert(HD == 128 || HD == 64 || HD == 32, "head_dim 128, 64 or 32");
   static constexpr int DPL = HD / 16;
   static constexpr bool split = sizeof(CacheT) == 4 && DPL == 8;
   static constexpr int per_lane = split ? 4 : DPL;   // the lane's first dimension = per_lane * c
@@ -197,11 +197,16 @@ template <bool kStream, int HD>
 __device__ __forceinline__ KvRow<HD / 16> load_row(const float* p) {
   using LD = LaneDims<float, HD>;
   KvRow<HD / 16> r;
-  const u32x4_t a = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p));
-  r.v[0] = __uint_as_float(a.x); r.v[1] = __uint_as_float(a.y); r.v[2] = __uint_as_float(a.z); r.v[3] = __uint_as_float(a.w);
-  if constexpr (LD::DPL == 8) {
-    const u32x4_t b = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p + LD::second));
-    r.v[4] = __uint_as_float(b.x); r.v[5] = __uint_as_float(b.y); r.v[6] = __uint_as_float(b.z); r.v[7] = __uint_as_float(b.w);
+  if constexpr (LD::DPL == 2) {
+    const u32x2_t a = load_kv<kStream>(reinterpret_cast<const u32x2_t*>(p));
+    r.v[0] = __uint_as_float(a.x); r.v[1] = __uint_as_float(a.y);
+  } else {
+    const u32x4_t a = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p));
+    r.v[0] = __uint_as_float(a.x); r.v[1] = __uint_as_float(a.y); r.v[2] = __uint_as_float(a.z); r.v[3] = __uint_as_float(a.w);
+    if constexpr (LD::DPL == 8) {
+      const u32x4_t b = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p + LD::second));
+      r.v[4] = __uint_as_float(b.x); r.v[5] = __uint_as_float(b.y); r.v[6] = __uint_as_float(b.z); r.v[7] = __uint_as_float(b.w);
+    }
   }
   return r;
 }
@@ -211,9 +216,11 @@ __device__ __forceinline__ KvRow<HD / 16> load_row(const uint16_t* p) {
   if constexpr (HD / 16 == 8) {
     const u32x4_t v = load_kv<kStream>(reinterpret_cast<const u32x4_t*>(p));
     widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]); widen2(v.z, r.v[4], r.v[5]); widen2(v.w, r.v[6], r.v[7]);
-  } else {
+  } else if constexpr (HD / 16 == 4) {
     const u32x2_t v = load_kv<kStream>(reinterpret_cast<const u32x2_t*>(p));
     widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]);
+  } else {
+    widen2(load_kv<kStream>(reinterpret_cast<const uint32_t*>(p)), r.v[0], r.v[1]);
   }
   return r;
 }
@@ -222,8 +229,12 @@ __device__ __forceinline__ KvRow<HD / 16> load_row(const uint16_t* p) {
 template <int HD>
 __device__ __forceinline__ void store_row(float* p, KvRow<HD / 16>& r) {
   using LD = LaneDims<float, HD>;
-  *reinterpret_cast<float4*>(p) = float4{r.v[0], r.v[1], r.v[2], r.v[3]};
-  if constexpr (LD::DPL == 8) *reinterpret_cast<float4*>(p + LD::second) = float4{r.v[4], r.v[5], r.v[6], r.v[7]};
+  if constexpr (LD::DPL == 2) {
+    *reinterpret_cast<float2*>(p) = float2{r.v[0], r.v[1]};
+  } else {
+    *reinterpret_cast<float4*>(p) = float4{r.v[0], r.v[1], r.v[2], r.v[3]};
+    if constexpr (LD::DPL == 8) *reinterpret_cast<float4*>(p + LD::second) = float4{r.v[4], r.v[5], r.v[6], r.v[7]};
+  }
 }
 template <int HD>
 __device__ __forceinline__ void store_row(uint16_t* p, KvRow<HD / 16>& r) {
@@ -233,11 +244,15 @@ __device__ __forceinline__ void store_row(uint16_t* p, KvRow<HD / 16>& r) {
     v.z = pack2_bf16(r.v[4], r.v[5]); v.w = pack2_bf16(r.v[6], r.v[7]);
     *reinterpret_cast<u32x4_t*>(p) = v;
     widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]); widen2(v.z, r.v[4], r.v[5]); widen2(v.w, r.v[6], r.v[7]);
-  } else {
+  } else if constexpr (HD / 16 == 4) {
     u32x2_t v;
     v.x = pack2_bf16(r.v[0], r.v[1]); v.y = pack2_bf16(r.v[2], r.v[3]);
     *reinterpret_cast<u32x2_t*>(p) = v;
     widen2(v.x, r.v[0], r.v[1]); widen2(v.y, r.v[2], r.v[3]);
+  } else {
+    const uint32_t v = pack2_bf16(r.v[0], r.v[1]);
+    *reinterpret_cast<uint32_t*>(p) = v;
+    widen2(v, r.v[0], r.v[1]);
   }
 }
 
@@ -280,7 +295,10 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
   // kStep: cosines / sines of the lane's DPL / 2 pairs (interleaved pairs never straddle a lane's four)
   float cs[DPL / 2], sn[DPL / 2];
   const float* qkv_row = q + (size_t)b * (H + 2 * Hkv) * hd + d0;  // kStep only
-  if (kStep) {
+  if (kStep && DPL == 2) {  // one pair per lane
+    cs[0] = cosine[p * (hd / 2) + d0 / 2];
+    sn[0] = sine[p * (hd / 2) + d0 / 2];
+  } else if (kStep) {
 #pragma unroll
     for (int h2 = 0; h2 < DPL / 4; ++h2) {
       const int pair0 = (d0 + h2 * LD::second) / 2;
@@ -301,11 +319,16 @@ __global__ __launch_bounds__(64 * kWaves) void attn_decode_kernel(const float* _
   // a row of fp32 activations (queries, the step's own key and value) in the lane's dimensions
   auto load_act = [&](const float* src) {
     Row r;
-    const float4 a = *reinterpret_cast<const float4*>(src);
-    r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
-    if constexpr (DPL == 8) {
-      const float4 b4 = *reinterpret_cast<const float4*>(src + LD::second);
-      r.v[4] = b4.x; r.v[5] = b4.y; r.v[6] = b4.z; r.v[7] = b4.w;
+    if constexpr (DPL == 2) {
+      const float2 a = *reinterpret_cast<const float2*>(src);
+      r.v[0] = a.x; r.v[1] = a.y;
+    } else {
+      const float4 a = *reinterpret_cast<const float4*>(src);
+      r.v[0] = a.x; r.v[1] = a.y; r.v[2] = a.z; r.v[3] = a.w;
+      if constexpr (DPL == 8) {
+        const float4 b4 = *reinterpret_cast<const float4*>(src + LD::second);
+        r.v[4] = b4.x; r.v[5] = b4.y; r.v[6] = b4.z; r.v[7] = b4.w;
+      }
     }
     return r;
   };

@@ -1,4 +1,4 @@
-// Causal self-attention for a block of T new positions (prefill), head_dim HD = 128 or 64, on bf16 MFMA
+// Causal self-attention for a block of T new positions (prefill), head_dim HD = 128, 64 or 32, on bf16 MFMA
 // with an online softmax: the T x (start + T) score matrix is never materialised.
 //
 //   out[b, t, h, :] = softmax_j( q[b, h, t, :] . k[b, hk, j, :] / sqrt(HD) ) v[b, hk, j, :],
@@ -7,7 +7,8 @@
 // q is fp32 [B, H, T, HD] (already rotated); keys and values are read where the model keeps
 // them, in the caches [B, Hkv, max_len, HD] (fp32 or bf16), rows 0 .. start + T - 1; out is
 // fp32 or bf16 [B, T, H * HD], the layout the output projection takes.  (The layouts below are
-// written out for HD = 128; with 64 a row is 128 B = 8 chunks = 4 segments and there are two k-steps.)
+// written out for HD = 128; with 64 a row is 128 B = 8 chunks = 4 segments and there are two k-steps, with 32 a row is
+// 64 B = 4 chunks = 2 segments and there is one.)
 //
 // A workgroup of 4 waves owns 128 query rows of one (b, h), a wave two groups of 16 of them
 // (every key and value fragment read from LDS meets both), and walks the keys in blocks of 64.
@@ -100,7 +101,7 @@ template <typename CacheT, int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __restrict__ q, const CacheT* __restrict__ kcache,
                                                            const CacheT* __restrict__ vcache, int H, int Hkv, int T,
                                                            int start, int max_len, void* __restrict__ out, int out_bf16) {
-  static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+  static_assert(HD == 128 || HD == 64 || HD == 32, "head_dim 128, 64 or 32");
   constexpr int kPfHD = HD;
   constexpr int RB = 2 * HD;          // bytes of a key (value) row as bf16
   constexpr int C = HD / 8;           // 16-byte chunks per row
@@ -136,7 +137,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const float* __res
   }
   const int b = bh / H, h = bh % H, hk = h / (H / Hkv);
   const int q0 = qb * kPfBQ;
-  const float qscale = 1.4426950408889634f * (HD == 128 ? 0.08838834764831845f : 0.125f);  // log2(e) / sqrt(HD)
+  const float qscale =  // log2(e) / sqrt(HD)
+      1.4426950408889634f * (HD == 128 ? 0.08838834764831845f : HD == 64 ? 0.125f : 0.17677669529663687f);
 
   const CacheT* kbase = kcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;
   const CacheT* vbase = vcache + ((size_t)b * Hkv + hk) * max_len * kPfHD;

@@ -348,7 +348,7 @@ class FusedDecoder(GraphDecoder):
     up to 16 rows, weight-streaming kernel up to 255); nine launches per layer where those forms are not built.
 
     Needs the architecture the benchmark model has: pre-norm RMSNorm blocks, RoPE, SwiGLU,
-    head_dim 128 or 64 (64: the geometry of the reference's configs/models/transformer_medium.yaml; the attention's
+    head_dim 128, 64 or 32 (64: the geometry of the reference's configs/models/transformer_medium.yaml; the attention's
     merge is then always a launch of its own), 1, 2 or 4 query heads per
     cache head, a quantized ``lm_head`` of its own (``quantize_model_(..., untie_head=True)`` for tied embeddings),
     every linear a QuantLinear.  ``kv_dtype``: torch.float32 (default, the model's own dtype) or
@@ -371,14 +371,14 @@ class FusedDecoder(GraphDecoder):
             model.position_encoding == "rope" and first.norm_placement == "pre"
             and isinstance(first.norm1, modeling.RMSNorm) and isinstance(first.feed_forward, modeling.SwiGLU)
             and isinstance(model.final_norm, modeling.RMSNorm) and isinstance(model.lm_head, QuantLinear)
-            and model.d_model // model.num_heads in (128, 64) and model.num_heads // model.num_kv_heads in (1, 2, 4)
+            and model.d_model // model.num_heads in (128, 64, 32) and model.num_heads // model.num_kv_heads in (1, 2, 4)
             and all(isinstance(m, QuantLinear) for layer in model.layers
                     for m in (layer.attention.q_proj, layer.attention.k_proj, layer.attention.v_proj,
                               layer.attention.output_proj, layer.feed_forward.w1, layer.feed_forward.w2,
                               layer.feed_forward.w3))
         )
         if not ok:
-            raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128 or 64 and "
+            raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128, 64 or 32 and "
                              "quantized linears everywhere (an lm_head of its own included: quantize_model_(..., "
                              "untie_head=True) gives a model with tied embeddings one)")
         dev, d = self.device, model.d_model

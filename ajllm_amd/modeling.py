@@ -209,7 +209,7 @@ class MultiHeadSelfAttention(nn.Module):
         self.rope = (RotaryPositionalEmbedding(rope_theta, self.head_dimension, context_length)
                      if position_encoding == "rope" else None)
         # as the reference's flag (attention.py:106-117): on a GPU, multi-token calls go to the
-        # library's flash-attention kernel instead of the masked softmax below (head_dim 128 or 64)
+        # library's flash-attention kernel instead of the masked softmax below (head_dim 128, 64 or 32)
         self.use_flash_attention = False
 
     def forward(self, inputs: torch.Tensor, positions: torch.Tensor, cache: KVCache | None = None,
@@ -243,7 +243,7 @@ class MultiHeadSelfAttention(nn.Module):
             start = cache.length
             cache.keys[layer_index][:, :, start:start + seq] = k
             cache.values[layer_index][:, :, start:start + seq] = v
-        if self.use_flash_attention and inputs.is_cuda and hd in (128, 64) and seq > 1:
+        if self.use_flash_attention and inputs.is_cuda and hd in (128, 64, 32) and seq > 1:
             from .attention import flash_prefill  # the library binding; model code stays importable without it
             if cache is not None and cache.keys[layer_index].is_contiguous():
                 joined = flash_prefill(q, cache.keys[layer_index], cache.values[layer_index], start)

@@ -255,7 +255,8 @@ int ajq_rope_prefill(const float* qkv, const float* cosine, const float* sine, f
 /* single-query softmax attention over cache rows 0 .. *pos, out bf16 [B, H * head_dim]
  * (scaled_dot_product_attention, src/ajllm/modeling/attention.py:20-33, for one query row;
  * H / Hkv = 1, 2 or 4 query heads share a cache head, whose rows are read once for all of
- * them).  head_dim 128 or 64 (the reference's configs/models/transformer_medium.yaml: 768 / 12 heads).
+ * them).  head_dim 128, 64 (the reference's configs/models/transformer_medium.yaml: 768 / 12 heads) or 32
+ * (transformer_baseline.yaml: 512 / 16 heads).
  * The workspace holds the partial results of up to 16 row chunks. */
 size_t ajq_attn_decode_workspace_bytes(int B, int H);
 /* Row chunks per cache head that ajq_attn_decode and ajq_attn_step use for this shape (0: bad shape).  With 1
@@ -267,7 +268,7 @@ int ajq_attn_decode(const float* q, const void* kcache, const void* vcache, int 
                     void* workspace, size_t workspace_bytes, void* stream);
 
 /* The two operators above in one kernel: qkv as for ajq_rope_cache; the step's key and value
- * rows are written to row *pos of the caches and attended to from registers.  head_dim 128 or 64. */
+ * rows are written to row *pos of the caches and attended to from registers.  head_dim 128, 64 or 32. */
 size_t ajq_attn_step_workspace_bytes(int B, int H);
 int ajq_attn_step(const float* qkv, const float* cosine, const float* sine, const int64_t* pos,
                   void* kcache, void* vcache, int cache_dtype, int B, int H, int Hkv, int head_dim,
@@ -294,7 +295,8 @@ int ajq_swiglu(const float* ab, uint16_t* out, int B, int F, void* stream);
  * rounding of the fp32 result).  Flash-attention arithmetic: bf16 MFMA products,
  * fp32 online softmax, no T x T matrix (scaled_dot_product_attention under a causal mask,
  * src/ajllm/modeling/attention.py:20-33,106-117; the reference's own tiled and Triton variants,
- * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128 or 64. */
+ * src/ajllm/modeling/flash_attention.py:44-108,194-298, are CUDA-gated).  head_dim 128, 64 or 32 (the head sizes of
+ * the benchmark models and of the reference's configs/models/transformer_medium.yaml and transformer_baseline.yaml). */
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H,
                      int Hkv, int T, int start, int max_len, int head_dim, void* out, int out_dtype, void* stream);
 

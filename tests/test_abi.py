@@ -80,7 +80,7 @@ def test_shape_alignment_and_option_errors():
     assert lib.ajq_w4a16_gemv(odd, 1, 128, p, p, 16, p, 0, None) == -3      # misaligned x
     assert lib.ajq_w8a16_gemm(p, 1, 192, p, p, 16, p, 0, None) == -2
     assert lib.ajq_add_rmsnorm(p, None, p, 1e-5, p, 1, 6, None) == -2            # D not a multiple of 4
-    assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 32, 8, p, p, 1 << 20, None) == -4  # head_dim 32 is not built
+    assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 48, 8, p, p, 1 << 20, None) == -4  # head_dim 48 is not built
     assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 16, 128, 1024, p, None, 0, None) == -6  # split attention needs its workspace
     assert lib.ajq_attn_decode(p, p, p, 5, p, 1, 16, 16, 128, 8, p, p, 1 << 20, None) == -4  # unknown cache dtype
     assert lib.ajq_swiglu(p, p, 1, 3, None) == -2

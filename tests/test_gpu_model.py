@@ -186,6 +186,37 @@ def test_reference_medium_geometry_decodes_through_the_fused_decoder(cuda, schem
     assert errors(dec._logits(), logits_eager.cpu())[1] <= 2e-2
 
 
+@pytest.mark.parametrize("scheme,batch,kv_dtype", [("w8a16", 2, None), ("w4a16_g128", 5, torch.bfloat16)])
+def test_head_dim_32_model_decodes_through_the_fused_decoder(cuda, scheme, batch, kv_dtype):
+    """The head size of the reference's configs/models/transformer_baseline.yaml (d_model 512, 16 heads of 32;
+    its d_ff 1344 is no multiple of 128 and cannot be quantized in groups, so 1408 here): decode attention, its
+    merge and the prefill attention at head_dim 32 inside the all-kernel decoder, against the eager loop."""
+    torch.manual_seed(23)
+    model = modeling.TransformerLM(vocab_size=1024, context_length=128, d_model=512, num_layers=2, num_heads=16,
+                                   d_ff=1408).eval()
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), scheme)
+    prompt = torch.randint(0, 1024, (batch, 24), generator=torch.Generator().manual_seed(7)).to(cuda)
+    eager, margins = modeling.greedy_decode(fast, prompt, 40, return_margins=True, kv_dtype=kv_dtype)
+    dec = decoding.FusedDecoder(fast, batch, 80, kv_dtype=kv_dtype)
+    assert dec.head_dim == 32
+    dec.prefill(prompt)
+    got = dec.generate(40)
+    report = compare_greedy(torch.cat((prompt, got), 1).cpu(), eager.cpu(), margins.cpu(), 24, noise=2e-3)
+    assert not report["unexplained"], report
+    dec.prefill(prompt)
+    with torch.no_grad():
+        logits_fused = dec._logits()
+        cache = fast.new_cache(batch, 80, dtype=kv_dtype)
+        fast(prompt, cache)
+        logits_eager = fast(dec.token, cache)[:, -1, :]
+    assert errors(logits_fused, logits_eager.cpu())[1] <= 3e-3
+    keys_model = [k.clone() for k in dec.cache.keys]
+    dec.prefill(prompt, fused=True)    # flash-attention arithmetic at head_dim 32
+    for mine, theirs in zip(dec.cache.keys, keys_model):
+        assert errors(mine[:, :, :24].float(), theirs[:, :, :24].float().cpu())[1] <= 1e-2
+    assert errors(dec._logits(), logits_eager.cpu())[1] <= 2e-2
+
+
 @pytest.mark.parametrize("batch", [1, 3])
 def test_graph_replayed_decoding_matches_eager_decoding(cuda, batch):
     """The decode step recorded into a HIP graph and replayed per token (with the program's own
@@ -328,17 +359,19 @@ def test_add_rmsnorm_over_widths(cuda, d):
     (4, 8, 8, 1100, torch.float32, 128), (8, 8, 4, 2100, torch.bfloat16, 128), (16, 8, 2, 1500, torch.float32, 128),
     (6, 16, 4, 1400, torch.bfloat16, 128), (32, 8, 8, 300, torch.float32, 128), (64, 16, 4, 520, torch.bfloat16, 128),
     (128, 4, 2, 200, torch.float32, 128), (16, 8, 8, 1100, torch.float32, 64), (64, 16, 4, 600, torch.bfloat16, 64),
-    (12, 12, 12, 900, torch.bfloat16, 64)])
+    (12, 12, 12, 900, torch.bfloat16, 64), (32, 16, 16, 1100, torch.float32, 32), (16, 16, 8, 2100, torch.bfloat16, 32),
+    (1, 16, 16, 256, torch.float32, 32), (3, 16, 4, 200, torch.bfloat16, 32), (2, 12, 12, 512, torch.float32, 64)])
 def test_decode_attention_over_caches_that_are_streamed(cuda, b, heads, kv_heads, max_len, cache_dtype, hd):
     """Caches above 16 MB per launch take the kernel's streaming form (non-temporal loads, rows dealt to the row
     chunks in blocks of 32), and from 256 (sequence, cache head) pairs on one 1024-thread workgroup reads a whole
-    head (256 pairs and more); head_dim 128 and 64: ajq_attn_decode and ajq_attn_step against the model code's attention, at positions
+    head (256 pairs and more); head_dim 128, 64 and 32 (the last three cases: the small caches of the reference's own
+    configurations, read with ordinary loads): ajq_attn_decode and ajq_attn_step against the model code's attention, at positions
     on both sides of block and chunk boundaries, with scores spread widely enough that the running reference
     exponent of the grouped-head form has to move many times."""
     from ajllm_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
-    assert 2 * b * kv_heads * max_len * hd * (4 if cache_dtype == torch.float32 else 2) > 16 << 20
+    assert 2 * b * kv_heads * max_len * hd * (4 if cache_dtype == torch.float32 else 2) > 16 << 20 or max_len <= 512
     g = torch.Generator().manual_seed(b * 1000 + max_len)
     att = modeling.MultiHeadSelfAttention(heads * hd, heads, max_len, "rope", 10000.0, num_kv_heads=kv_heads).to(cuda)
     kv_flag = _lib.AJQ_KV_BF16 if cache_dtype == torch.bfloat16 else _lib.AJQ_KV_F32
@@ -499,7 +532,7 @@ def test_graph_decoders_stop_at_eos(cuda, batch):
         assert stop < 40  # (one row always has a common token: the stop is exercised)
 
 
-@pytest.mark.parametrize("hd", [128, 64])
+@pytest.mark.parametrize("hd", [128, 64, 32])
 @pytest.mark.parametrize("b,heads,kv_heads,t,start,cache_dtype", [
     (2, 4, 2, 100, 0, torch.float32), (1, 2, 2, 64, 0, torch.float32), (1, 4, 1, 130, 37, torch.float32),
     (3, 2, 1, 257, 5, torch.bfloat16), (1, 1, 1, 1, 9, torch.float32), (1, 8, 2, 512, 0, torch.bfloat16),
@@ -509,8 +542,8 @@ def test_flash_prefill_attention(cuda, b, heads, kv_heads, t, start, cache_dtype
     """ajq_attn_prefill against the model code's masked softmax attention.  The kernel rounds q, k, v
     and the probabilities to bf16 (flash-attention arithmetic): compared with the fp32 statement on the
     same bf16-rounded inputs within 4e-3 relative Frobenius, and with the unrounded one within 1e-2.
-    head_dim 128 (the benchmark models) and 64 (the reference's configs/models/transformer_medium.yaml, whose
-    shape 12 heads x 511 positions is the last case)."""
+    head_dim 128 (the benchmark models), 64 (the reference's configs/models/transformer_medium.yaml, whose
+    shape 12 heads x 511 positions is the last case) and 32 (transformer_baseline.yaml)."""
     from ajllm_amd.attention import flash_prefill
     g = torch.Generator().manual_seed(b * 1000 + t)
     max_len = start + t + 3
