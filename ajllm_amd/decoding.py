@@ -372,15 +372,15 @@ class FusedDecoder(GraphDecoder):
             and isinstance(first.norm1, modeling.RMSNorm) and isinstance(first.feed_forward, modeling.SwiGLU)
             and isinstance(model.final_norm, modeling.RMSNorm) and isinstance(model.lm_head, QuantLinear)
             and model.d_model // model.num_heads in (128, 64, 32) and model.num_heads // model.num_kv_heads in (1, 2, 4)
-            and all(isinstance(m, QuantLinear) for layer in model.layers
+            and all(isinstance(m, QuantLinear) and m.padded_in_features == m.in_features for layer in model.layers
                     for m in (layer.attention.q_proj, layer.attention.k_proj, layer.attention.v_proj,
                               layer.attention.output_proj, layer.feed_forward.w1, layer.feed_forward.w2,
                               layer.feed_forward.w3))
         )
         if not ok:
             raise ValueError("FusedDecoder needs pre-norm RMSNorm + RoPE + SwiGLU blocks with head_dim 128, 64 or 32 and "
-                             "quantized linears everywhere (an lm_head of its own included: quantize_model_(..., "
-                             "untie_head=True) gives a model with tied embeddings one)")
+                             "quantized linears everywhere with input widths that are multiples of 128 (an lm_head of its "
+                             "own included: quantize_model_(..., untie_head=True) gives a model with tied embeddings one)")
         dev, d = self.device, model.d_model
         self.heads, self.kv_heads, self.head_dim = model.num_heads, model.num_kv_heads, d // model.num_heads
         self.d_ff = first.feed_forward.w1.out_features

@@ -113,11 +113,14 @@ def unrepack_w4(wq: torch.Tensor, meta: torch.Tensor) -> tuple[torch.Tensor, tor
 
 
 def repack_w8(q: torch.Tensor) -> torch.Tensor:
-    """int8 [N, K] -> wq int32 [N16/16, K/64, 64, 4] (rows zero-padded to a multiple of 16)."""
+    """int8 [N, K] -> wq int32 [N16/16, K128/64, 64, 4] (rows zero-padded to a multiple of 16, columns to a
+    multiple of 128: per-channel scales put no condition on K, and zero codes add exact zeros to a product whose
+    activations are padded with zeros alike)."""
     _require_cuda(q)
     n, k = q.shape
     if k % GROUP != 0:
-        raise ValueError(f"K={k} must be a multiple of {GROUP} for w8a16")
+        q = torch.nn.functional.pad(q, (0, GROUP - k % GROUP))
+        k = q.shape[1]
     n16 = (n + TILE_N - 1) // TILE_N * TILE_N
     q = _pad_rows(q, n16)
     wq = torch.empty((n16 // TILE_N, k // 64, 64, 4), dtype=torch.int32, device=q.device)
@@ -248,6 +251,12 @@ class QuantLinear(nn.Module):
             raise ValueError("the reference Linear is bias-free; a biased layer cannot be swapped")
         return cls.from_weight(linear.weight.data, scheme)
 
+    @property
+    def padded_in_features(self) -> int:
+        """Columns of the kernel-private weight tensor: ``in_features`` rounded up to a multiple of 128 (W8 only;
+        W4 groups need ``in_features`` itself on that grid)."""
+        return (self.in_features + GROUP - 1) // GROUP * GROUP
+
     def prepare(self) -> None:
         """(Re)build the kernel-private tensors from the canonical ones."""
         if self.scheme == "w8a16":
@@ -298,6 +307,8 @@ class QuantLinear(nn.Module):
         want = out_dtype or inputs.dtype
         if x.dtype != torch.bfloat16:
             x = x.to(torch.bfloat16)
+        if self.padded_in_features != self.in_features:  # W8 with in_features off the kernels' 128-column grid
+            x = torch.nn.functional.pad(x, (0, self.padded_in_features - self.in_features))
         kernel_out = torch.float32 if want == torch.float32 else torch.bfloat16
         if self.scheme == "w8a16":
             y = w8a16_matmul(x, self.wq, self.meta, kernel_out)

@@ -59,6 +59,61 @@ def test_quant_linear_rejects_bias_and_bad_k(cuda):
         QuantLinear.from_weight(torch.zeros(16, 100, device=cuda))
 
 
+def test_w8_layer_with_an_input_width_off_the_128_grid(cuda):
+    """Per-channel W8 puts no condition on K (the reference's configs/models/transformer_baseline.yaml has d_ff
+    1344 = 10.5 groups of 128): the canonical tensors are the oracle's, the kernel-private copy is padded with zero
+    codes to 1408 columns and the activations with zeros, which adds exact zeros to every product."""
+    torch.manual_seed(5)
+    dense = modeling.Linear(1344, 520)
+    ref = qspec.QuantLinearRef.from_linear(dense, "w8a16")
+    layer = QuantLinear.from_linear(dense.to(cuda), "w8a16")
+    assert (layer.in_features, layer.padded_in_features, layer.out_features) == (1344, 1408, 520)
+    state = layer.state_dict()
+    assert tuple(state["qweight"].shape) == (520, 1344) and torch.equal(state["qweight"].cpu(), ref.qweight)
+    assert torch.equal(state["scales"].cpu().view(torch.int16), ref.scales.view(torch.int16))
+    for m in (1, 15, 40, 300):   # GEMV, weight-streaming and tile kernels
+        x = make_activations(m, 1344, m)
+        assert errors(layer(x.to(cuda)), ref(x))[1] <= REL_FRO_TOL, m
+    fresh = QuantLinear(1344, 520, "w8a16")
+    fresh.load_state_dict({k: v.clone() for k, v in state.items()})
+    x = make_activations(7, 1344, 9)
+    assert torch.equal(fresh(x.to(cuda)), layer(x.to(cuda)))
+    with pytest.raises(ValueError):
+        QuantLinear.from_linear(dense.to(cuda), "w4a16_g128")   # groups of 128 input channels need K on that grid
+
+
+def test_reference_baseline_geometry_decodes_with_w8(cuda):
+    """configs/models/transformer_baseline.yaml (d_model 512, 16 heads of 32, d_ff 1344, 4 layers, context 256)
+    under W8A16: every linear is swapped, the greedy tokens follow the oracle model's up to its own margin noise,
+    and the graph-replayed loop with the library's prefill attention (head_dim 32) gives the eager loop's tokens.
+    The all-kernel decoder does not take the model (w2's input width is off the 128-column grid)."""
+    torch.manual_seed(24)
+    model = modeling.TransformerLM(vocab_size=1024, context_length=256, d_model=512, num_layers=4, num_heads=16,
+                                   d_ff=1344).eval()
+    ref = _oracle_model(model, "w8a16")
+    fast = quantize_model_(copy.deepcopy(model).to(cuda), "w8a16")
+    assert len([m for m in fast.modules() if isinstance(m, QuantLinear)]) == 4 * 7 + 1
+    prompt = torch.randint(0, 1024, (2, 24), generator=torch.Generator().manual_seed(8))
+    ref_tokens, margins = modeling.greedy_decode(ref, prompt, 32, return_margins=True)
+    noise = errors(fast(ref_tokens.to(cuda)), ref(ref_tokens))[0]
+    assert noise <= 5e-2
+    eager = modeling.greedy_decode(fast, prompt.to(cuda), 32)
+    report = compare_greedy(eager.cpu(), ref_tokens, margins, 24, noise=noise)
+    assert not report["unexplained"], report
+    for layer in fast.layers:
+        layer.attention.use_flash_attention = True
+    flash, flash_margins = modeling.greedy_decode(fast, prompt.to(cuda), 32, return_margins=True)
+    report = compare_greedy(flash.cpu(), eager.cpu(), flash_margins.cpu(), 24, noise=2e-2)   # flash-attention arithmetic
+    assert not report["unexplained"], report
+    dec = decoding.GraphDecoder(fast, 2, 64)
+    dec.prefill(prompt.to(cuda))
+    got = dec.generate(32)
+    report = compare_greedy(torch.cat((prompt.to(cuda), got), 1).cpu(), flash.cpu(), flash_margins.cpu(), 24, noise=1e-3)
+    assert not report["unexplained"], report
+    with pytest.raises(ValueError, match="multiples of 128"):
+        decoding.FusedDecoder(fast, 2, 64)
+
+
 def test_quantize_model_swaps_every_linear(cuda):
     torch.manual_seed(1)
     model = modeling.TransformerLM(vocab_size=512, context_length=64, d_model=256, num_layers=2, num_heads=2,
