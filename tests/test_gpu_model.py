@@ -82,36 +82,45 @@ def test_w8_layer_with_an_input_width_off_the_128_grid(cuda):
         QuantLinear.from_linear(dense.to(cuda), "w4a16_g128")   # groups of 128 input channels need K on that grid
 
 
-def test_reference_baseline_geometry_decodes_with_w8(cuda):
-    """configs/models/transformer_baseline.yaml (d_model 512, 16 heads of 32, d_ff 1344, 4 layers, context 256)
-    under W8A16: every linear is swapped, the greedy tokens follow the oracle model's up to its own margin noise,
-    and the graph-replayed loop with the library's prefill attention (head_dim 32) gives the eager loop's tokens.
-    The all-kernel decoder does not take the model (w2's input width is off the 128-column grid)."""
+@pytest.mark.parametrize("geometry", ["baseline", "tiny"])
+def test_reference_baseline_and_tiny_geometries_decode_with_w8(cuda, geometry):
+    """configs/models/transformer_baseline.yaml (d_model 512, 16 heads of 32, d_ff 1344, 4 layers, context 256) and
+    transformer_tiny.yaml (d_model 64, 4 heads of 16, d_ff 128, 2 layers, vocabulary 300, context 32) under W8A16:
+    every linear is swapped (input widths 1344 and 64 are padded to the kernels' 128-column grid), the greedy
+    tokens follow the oracle model's up to its own margin noise, and the graph-replayed loop (with the library's
+    prefill attention where the head size is built: 32) gives the eager loop's tokens.  The all-kernel decoder
+    does not take such a model."""
     torch.manual_seed(24)
-    model = modeling.TransformerLM(vocab_size=1024, context_length=256, d_model=512, num_layers=4, num_heads=16,
-                                   d_ff=1344).eval()
+    if geometry == "baseline":
+        model = modeling.TransformerLM(vocab_size=1024, context_length=256, d_model=512, num_layers=4, num_heads=16,
+                                       d_ff=1344).eval()
+        layers, new, vocab = 4, 32, 1024
+    else:
+        model = modeling.TransformerLM(vocab_size=300, context_length=32, d_model=64, num_layers=2, num_heads=4,
+                                       d_ff=128).eval()
+        layers, new, vocab = 2, 8, 300
     ref = _oracle_model(model, "w8a16")
     fast = quantize_model_(copy.deepcopy(model).to(cuda), "w8a16")
-    assert len([m for m in fast.modules() if isinstance(m, QuantLinear)]) == 4 * 7 + 1
-    prompt = torch.randint(0, 1024, (2, 24), generator=torch.Generator().manual_seed(8))
-    ref_tokens, margins = modeling.greedy_decode(ref, prompt, 32, return_margins=True)
+    assert len([m for m in fast.modules() if isinstance(m, QuantLinear)]) == layers * 7 + 1
+    prompt = torch.randint(0, vocab, (2, 24), generator=torch.Generator().manual_seed(8))
+    ref_tokens, margins = modeling.greedy_decode(ref, prompt, new, return_margins=True)
     noise = errors(fast(ref_tokens.to(cuda)), ref(ref_tokens))[0]
     assert noise <= 5e-2
-    eager = modeling.greedy_decode(fast, prompt.to(cuda), 32)
+    eager = modeling.greedy_decode(fast, prompt.to(cuda), new)
     report = compare_greedy(eager.cpu(), ref_tokens, margins, 24, noise=noise)
     assert not report["unexplained"], report
     for layer in fast.layers:
-        layer.attention.use_flash_attention = True
-    flash, flash_margins = modeling.greedy_decode(fast, prompt.to(cuda), 32, return_margins=True)
+        layer.attention.use_flash_attention = True   # (head_dim 16 of the tiny model: the model's own attention)
+    flash, flash_margins = modeling.greedy_decode(fast, prompt.to(cuda), new, return_margins=True)
     report = compare_greedy(flash.cpu(), eager.cpu(), flash_margins.cpu(), 24, noise=2e-2)   # flash-attention arithmetic
     assert not report["unexplained"], report
-    dec = decoding.GraphDecoder(fast, 2, 64)
+    dec = decoding.GraphDecoder(fast, 2, 24 + new)
     dec.prefill(prompt.to(cuda))
-    got = dec.generate(32)
+    got = dec.generate(new)
     report = compare_greedy(torch.cat((prompt.to(cuda), got), 1).cpu(), flash.cpu(), flash_margins.cpu(), 24, noise=1e-3)
     assert not report["unexplained"], report
     with pytest.raises(ValueError, match="multiples of 128"):
-        decoding.FusedDecoder(fast, 2, 64)
+        decoding.FusedDecoder(fast, 2, 24 + new)
 
 
 def test_quantize_model_swaps_every_linear(cuda):
