@@ -182,15 +182,16 @@ def bench_dense_library_gemm(m: int, n: int, k: int, steps: int, warmup: int, de
             "frac_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS}
 
 
-def bench_flash_prefill(batch: int, heads: int, kv_heads: int, seq: int, cache_dtype, device, reps: int = 10) -> dict:
-    """Causal prefill attention (``ajq_attn_prefill``) on config 5's prefill shape: head_dim 128,
-    fp32 queries, bf16 output; flops counted for the causal half only."""
+def bench_flash_prefill(batch: int, heads: int, kv_heads: int, seq: int, cache_dtype, device, reps: int = 10,
+                        head_dim: int = 128) -> dict:
+    """Causal prefill attention (``ajq_attn_prefill``) on config 5's prefill shape (head_dim 128; 64 and 32 for
+    the head-size sweep), fp32 queries, bf16 output; flops counted for the causal half only."""
     from ajllm_amd.attention import flash_prefill
 
     g = torch.Generator(device="cpu").manual_seed(11)
-    q = torch.randn((batch, heads, seq, 128), generator=g).to(device)
-    keys = torch.randn((batch, kv_heads, seq, 128), generator=g).to(device).to(cache_dtype)
-    values = torch.randn((batch, kv_heads, seq, 128), generator=g).to(device).to(cache_dtype)
+    q = torch.randn((batch, heads, seq, head_dim), generator=g).to(device)
+    keys = torch.randn((batch, kv_heads, seq, head_dim), generator=g).to(device).to(cache_dtype)
+    values = torch.randn((batch, kv_heads, seq, head_dim), generator=g).to(device).to(cache_dtype)
     for _ in range(3):
         flash_prefill(q, keys, values, 0, out_dtype=torch.bfloat16)
     torch.cuda.synchronize()
@@ -201,8 +202,9 @@ def bench_flash_prefill(batch: int, heads: int, kv_heads: int, seq: int, cache_d
     end.record()
     end.synchronize()
     us = start.elapsed_time(end) * 1e3 / reps
-    flops = 4.0 * batch * heads * seq * seq * 0.5 * 128
-    return {"B": batch, "H": heads, "Hkv": kv_heads, "T": seq, "kv_cache": str(cache_dtype).replace("torch.", ""),
+    flops = 4.0 * batch * heads * seq * seq * 0.5 * head_dim
+    return {"B": batch, "H": heads, "Hkv": kv_heads, "T": seq, "head_dim": head_dim,
+            "kv_cache": str(cache_dtype).replace("torch.", ""),
             "us_per_call": us, "causal_TFLOP/s": flops / us * 1e-6, "frac_mfma_peak": flops / us * 1e-6 / MFMA_BF16_PEAK_TFLOPS}
 
 
@@ -456,6 +458,12 @@ def main() -> int:
 
         extras["decode"] = bench_decode_short(device, log)
     if args.sweep:
+        heads_sweep = [bench_flash_prefill(b, 32, 8, t, dt, device, head_dim=hd)
+                       for hd in (128, 64, 32) for (b, t) in ((4, 2048), (1, 8192))
+                       for dt in (torch.bfloat16, torch.float32)]
+        for r in heads_sweep:
+            log("prefill attention by head size", json.dumps(r))
+        extras["prefill_attention_head_sizes"] = heads_sweep
         sweep = []
         for scheme in ("w4", "w8"):
             for (sn, sk) in ((4096, 4096), (14336, 4096), (4096, 14336)):
