@@ -89,6 +89,7 @@ SIGNATURES: dict[str, tuple] = {
          c_void_p],
     ),
     "ajq_gemv_epilogue_supported": (c_int, [c_int, c_int]),
+    "ajq_gemv_rowscale_supported": (c_int, [c_int, c_int]),
     "ajq_w4a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p]),
     "ajq_w8a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,

@@ -506,6 +506,10 @@ bool gemv_epi_straight(int M, int K) {
   return M <= kMaxGemvM && (K == 2048 || K == 4096 || (K == 5632 && M <= 8));
 }
 bool gemv_epi_supported(int M, int K) { return M >= 1 && M <= kMaxEpiM && K >= kGroup && K % kGroup == 0; }
+// the row-scale consumer adds the K / 16 per-tile sums of squares with 32 per wave: eight waves cover 256 of them
+// (K <= 4096), the eleven of the straight-line K = 5632 configuration 352
+int gemv_rowscale_max_parts(int M, int K) { return (gemv_epi_straight(M, K) && K == 5632) ? 11 * 32 : 8 * 32; }
+bool gemv_rowscale_supported(int M, int K) { return gemv_epi_supported(M, K) && K / 16 <= gemv_rowscale_max_parts(M, K); }
 
 template <bool kW4, int kEpi>
 int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
@@ -541,10 +545,11 @@ int gemv_rowscale(const char* name, const uint16_t* xt, const float* ssq, int pa
                          const uint32_t* wq, const void* aux, int N, void* y, int out_dtype, int gate, void* stream) {
   if (int s = check_matmul_args(name, xt, M, K, wq, aux, N, y, out_dtype, kGroup)) return s;
   if (int s = check_epi(name, M, K)) return s;
+  if (!gemv_rowscale_supported(M, K))
+    return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d has more than %d tile sums per row (ajq_gemv_rowscale_supported)", name,
+                M, K, gemv_rowscale_max_parts(M, K));
   if (!ssq || !aligned16(ssq)) return fail(ssq ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq must be non-null and 16-byte aligned", name);
-  const int waves = (gemv_epi_straight(M, K) && K == 5632) ? 11 : 8;
-  if (parts < 4 || parts % 4 != 0 || parts > waves * 32)
-    return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, %d]", name, parts, waves * 32);
+  if (parts != K / 16) return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be K / 16 = %d", name, parts, K / 16);
   if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);
   GemvEpilogue ep{};
   ep.ssq_in = ssq;
@@ -726,8 +731,8 @@ int gemv_norm_sums(const char* name, const float* h, const float* ssq, int parts
     return fail(AJQ_ERR_UNSUPPORTED, "%s: M=%d, K=%d is not built (ajq_gemv_fused_supported)", name, M, K);
   if (!ssq || !gain || !aligned16(ssq) || !aligned16(gain))
     return fail(ssq && gain ? AJQ_ERR_ALIGN : AJQ_ERR_NULL, "%s: ssq and gain must be non-null and 16-byte aligned", name);
-  if (parts < 4 || parts % 4 != 0 || parts > 256)
-    return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be a multiple of 4 in [4, 256]", name, parts);
+  if (parts != K / 16 || parts > 256)
+    return fail(AJQ_ERR_SHAPE, "%s: parts=%d must be K / 16 = %d and at most 256", name, parts, K / 16);
   if (gate && out_dtype != AJQ_OUT_BF16) return fail(AJQ_ERR_UNSUPPORTED, "%s: the gated output is bf16", name);
   const uint32_t* meta = kW4 ? static_cast<const uint32_t*>(aux) : nullptr;
   const uint16_t* scales = kW4 ? nullptr : static_cast<const uint16_t*>(aux);
@@ -800,6 +805,8 @@ int ajq_w8a16_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1 : 0; }
 
 int ajq_gemv_epilogue_supported(int M, int K) { return gemv_epi_supported(M, K) ? 1 : 0; }
+
+int ajq_gemv_rowscale_supported(int M, int K) { return gemv_rowscale_supported(M, K) ? 1 : 0; }
 
 int ajq_w4a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
                          void* stream) {

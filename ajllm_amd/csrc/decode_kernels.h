@@ -528,8 +528,8 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
                                                            const float* __restrict__ embedding, int D,
                                                            float* __restrict__ hidden, long long* __restrict__ token,
                                                            long long* __restrict__ out, int out_ld,
-                                                           const long long* __restrict__ step,
-                                                           long long* advance, unsigned* ticket) {
+                                                           const long long* step, long long* advance,
+                                                           unsigned* ticket) {
   const int b = blockIdx.x, t = threadIdx.x;
   const float* row = logits + (size_t)b * ld;
   float best = -INFINITY;
@@ -578,11 +578,15 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
     if (bi == 0x7FFFFFFF) bi = 0;  // a row of NaNs: torch picks the NaN; here index 0
     chosen = bi;
     token[b] = bi;
-    out[(size_t)b * out_ld + min(max(*step, 0LL), (long long)out_ld - 1)] = bi;  // device data: held inside the row
+    // `step` may alias advance[0..1] (hence no __restrict__ on either): read it once, through a volatile
+    // access so the load stays in front of the fence below
+    const long long at = *reinterpret_cast<const volatile long long*>(step);
+    out[(size_t)b * out_ld + min(max(at, 0LL), (long long)out_ld - 1)] = bi;  // device data: held inside the row
     if (advance) {
-      // the step's two counters (cache row, output column) advance here, once every workgroup has
-      // read them: this thread's read of *step above has returned (its value addressed the store)
-      // before its ticket is drawn, so the workgroup that draws the last ticket writes after all reads
+      // the step's two counters (cache row, output column) advance here, once every workgroup has read them:
+      // the fence orders this thread's read of *step in front of its ticket, so the workgroup that draws the
+      // last ticket writes after every read
+      __threadfence();
       if (atomicAdd(ticket, 1u) == gridDim.x - 1) {
         advance[0] += 1;
         advance[1] += 1;

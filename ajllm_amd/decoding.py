@@ -234,6 +234,10 @@ class _FusedLinear:
         input width."""
         return bool(_lib.load().ajq_gemv_epilogue_supported(batch, self.in_features))
 
+    def rowscale_fusable(self, batch: int) -> bool:
+        """Whether ``rowscaled`` is built for this batch and input width (it adds ``in_features / 16`` tile sums)."""
+        return bool(_lib.load().ajq_gemv_rowscale_supported(batch, self.in_features))
+
     def residual(self, x_bf16: torch.Tensor, h_in: torch.Tensor, gain: torch.Tensor, h_out: torch.Tensor,
                  xt: torch.Tensor | None, ssq: torch.Tensor) -> None:
         """``h_out = h_in + self(x)``, ``xt = bf16(h_out * gain)`` (skipped if None) and the per-tile sums of squares
@@ -450,10 +454,11 @@ class FusedDecoder(GraphDecoder):
         # launches per layer instead of nine
         self.norm_launch = self.exact_norm and not (batch <= 4 and self.head.fusable(batch))
         self.fuse_epilogue = (
-            self.d_ff % 8 == 0 and d // 16 <= 256
+            self.d_ff % 8 == 0 and d // 16 <= 256  # the norm-from-sums consumer takes at most 256 tile sums
             and self.layers[0]["o"].in_features == d
             and all(self.layers[0][name].epilogue_fusable(batch) for name in ("qkv", "o", "w13", "w2"))
-            and self.head.epilogue_fusable(batch)
+            and all(self.layers[0][name].rowscale_fusable(batch) for name in ("qkv", "w13"))
+            and self.head.epilogue_fusable(batch) and self.head.rowscale_fusable(batch)
         )
         if self.fuse_epilogue:
             # the step's very first norm rides in layer 0's q|k|v where built

@@ -288,10 +288,24 @@ class QuantLinear(nn.Module):
             return  # leave the layer as it was: a partial load must not leave mixed tensors behind
         expect_q = ((self.out_features, self.in_features) if self.scheme == "w8a16"
                     else (self.out_features, self.in_features // 8))
-        if tuple(found["qweight"].shape) != expect_q:
-            error_msgs.append(f"size mismatch for {prefix}qweight: checkpoint {tuple(found['qweight'].shape)}, "
-                              f"layer ({self.scheme}) expects {expect_q}")
-            return
+        w8 = self.scheme == "w8a16"
+        groups = (self.out_features,) if w8 else (self.out_features, self.in_features // GROUP)
+        expect = {"qweight": (expect_q, torch.int8 if w8 else torch.int32), "scales": (groups, torch.float16)}
+        if not w8:
+            expect["zeros"] = (groups, torch.uint8)
+        bad = False
+        for name, (shape, dtype) in expect.items():
+            got = found[name]
+            if tuple(got.shape) != shape:
+                error_msgs.append(f"size mismatch for {prefix}{name}: checkpoint {tuple(got.shape)}, "
+                                  f"layer ({self.scheme}) expects {shape}")
+                bad = True
+            elif got.dtype != dtype:
+                error_msgs.append(f"dtype mismatch for {prefix}{name}: checkpoint {got.dtype}, "
+                                  f"layer ({self.scheme}) expects {dtype}")
+                bad = True
+        if bad:
+            return  # nothing of the layer has been touched
         for name, value in found.items():
             setattr(self, name, value.clone())
         if self.scheme == "w8a16" and "zeros" not in found:

@@ -140,16 +140,20 @@ int ajq_w8a16_gemv_gate(const float* ab, int M, int K, const uint32_t* wq, const
  *              (gain[N]: of the norm that follows) and ssq_out[max(16, M)][N / 16]: per row, the sum of squares of
  *              h_out over each 16-column tile (rows >= M are not written);
  *   _rowscale: y = rstd[m] * (xt W^T) with rstd[m] = rsqrt(sum(ssq[m][0 .. parts)) / K + eps), ssq laid out
- *              [16][parts] as _residual leaves it (parts = K / 16; a multiple of 4, at most 256, 352 for
- *              K = 5632).  gate != 0: the rows of W are tiles of 8 gate-projection rows followed by the 8
+ *              [max(16, M)][parts] as _residual leaves it; parts must be K / 16 and at most 256 (K <= 4096), or 352
+ *              for K = 5632 with M <= 8: ajq_gemv_rowscale_supported reports whether (M, K) is taken.  gate != 0: the rows of W are tiles of 8 gate-projection rows followed by the 8
  *              matching up-projection rows (w1 and w3 interleaved in blocks of 8) and
  *              y[M, N / 2] = bf16(silu(a) * u), out_dtype AJQ_OUT_BF16.
  * xt is rounded to bf16 BEFORE the row scale is applied (the reference order rounds the normalised value);
  * both are one bf16 rounding of the same quantity up to the fp32 factor rstd.  Sums run in a fixed order:
  * results are run-to-run identical.  Built for the (M, K) that ajq_gemv_epilogue_supported reports: 1 <= M <= 255,
  * K % 128 == 0 (the GEMV kernel for M <= 16 with K = 2048 or 4096 and M <= 8 with K = 5632, the weight-streaming
- * kernel otherwise; ssq has max(16, M) rows); AJQ_ERR_UNSUPPORTED otherwise. */
+ * kernel otherwise; ssq has max(16, M) rows); AJQ_ERR_UNSUPPORTED otherwise.  _rowscale is built for the narrower
+ * set that ajq_gemv_rowscale_supported reports (its K is the width whose K / 16 tile sums it adds up): the
+ * _residual -> _rowscale pair needs both queries to say yes, the first for the producer's (M, K), the second
+ * for the consumer's. */
 int ajq_gemv_epilogue_supported(int M, int K);
+int ajq_gemv_rowscale_supported(int M, int K);
 int ajq_w4a16_gemv_residual(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                             const float* h_in, const float* gain, float* h_out, uint16_t* xt_out, float* ssq_out,
                             void* stream);

@@ -75,3 +75,57 @@ def compare_greedy(tokens_got: torch.Tensor, tokens_ref: torch.Tensor, margins_r
             unexplained.append((b, first, float(margins_ref[b, first])))
     return {"rows": rows, "identical_rows": identical_rows, "attributable": attributable,
             "unexplained": unexplained, "min_margin_on_compared_prefix": min_margin}
+
+
+# ---------------------------------------------------------------- quantizer corner cases
+# (fp16 scale, weight, code by IEEE division, code by multiplying with the rounded reciprocal):
+# found by search; W / d and W * (1 / d) land on different sides of a half.
+W8_DIVISION_CASES = [
+    (0.005665, "0x1.67a6p-4", 16, 15),
+    (0.003347, "-0x1.ed9802p-7", -5, -4),
+    (0.006348, "0x1.b6bffep-2", 67, 68),
+]
+W4_DIVISION_CASES = [  # groups spanning -5 d ... 10 d (zero-point 5); codes include the zero-point
+    (0.003347, "-0x1.ed9802p-7", 0, 1),
+    (0.009796, "0x1.692002p-5", 10, 9),
+    (0.005737, "0x1.a70002p-6", 10, 9),
+]
+W4_ZERO_DIVISION_CASES = [  # (fp16 scale, min, max, zero by division, zero by reciprocal)
+    (0.0008893, "-0x1.d24002p-12", "0x1.a68ap-7", 1, 0),
+    (0.006264, "-0x1.0d64p-4", "0x1.cddp-6", 10, 11),
+    (0.006393, "-0x1.7bb8p-4", "0x1.a3p-9", 14, 15),
+]
+
+
+def tie_and_division_rows(k: int = 512) -> np.ndarray:
+    """fp32 rows [*, k] (k >= 512, a multiple of 128) holding the quantizers' rounding corners:
+    W4 code ties under an odd zero-point, zero-points exactly on a half, and the committed
+    (scale, weight) pairs where IEEE division and a multiply by the rounded reciprocal round
+    to different integers (per-row absmax for W8, per-group range for W4)."""
+    rows = []
+    d = np.float32(2.0**-3)
+    row = np.zeros(k, np.float32)
+    row[0], row[1] = -5 * d, 10 * d
+    row[2:8] = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32) * d
+    rows.append(row)
+    d = np.float32(2.0**-4)
+    row = np.zeros(k, np.float32)
+    for g, below in enumerate((2.5, 3.5, 4.5, 14.5)):
+        row[128 * g], row[128 * g + 1] = -below * d, (15 - below) * d
+    rows.append(row)
+    for scale, weight, _, _ in W8_DIVISION_CASES:
+        dd = np.float32(np.float16(scale))
+        row = np.zeros(k, np.float32)
+        row[0], row[1] = np.float32(127.0) * dd, np.float32(float.fromhex(weight))
+        rows.append(row)
+    row = np.zeros(k, np.float32)
+    for g, (scale, weight, _, _) in enumerate(W4_DIVISION_CASES):
+        dd = np.float32(np.float16(scale))
+        row[128 * g], row[128 * g + 1] = np.float32(-5.0) * dd, np.float32(10.0) * dd
+        row[128 * g + 2] = np.float32(float.fromhex(weight))
+    rows.append(row)
+    row = np.zeros(k, np.float32)
+    for g, (_, mn, mx, _, _) in enumerate(W4_ZERO_DIVISION_CASES):
+        row[128 * g], row[128 * g + 1] = np.float32(float.fromhex(mn)), np.float32(float.fromhex(mx))
+    rows.append(row)
+    return np.stack(rows)

@@ -96,6 +96,14 @@ def test_shape_alignment_and_option_errors():
     assert lib.ajq_gemv_epilogue_supported(1, 2048) == 1 and lib.ajq_gemv_epilogue_supported(16, 4096) == 1
     assert lib.ajq_gemv_epilogue_supported(9, 5632) == 1 and lib.ajq_gemv_epilogue_supported(200, 14336) == 1   # streaming kernel
     assert lib.ajq_gemv_epilogue_supported(256, 2048) == 0 and lib.ajq_gemv_epilogue_supported(4, 1000) == 0
+    # the row-scale consumer adds K / 16 tile sums: K <= 4096, or K = 5632 on the eleven-wave GEMV (M <= 8)
+    assert lib.ajq_gemv_rowscale_supported(1, 2048) == 1 and lib.ajq_gemv_rowscale_supported(32, 4096) == 1
+    assert lib.ajq_gemv_rowscale_supported(8, 5632) == 1 and lib.ajq_gemv_rowscale_supported(12, 5632) == 0
+    assert lib.ajq_gemv_rowscale_supported(32, 8192) == 0 and lib.ajq_gemv_rowscale_supported(200, 14336) == 0
+    assert lib.ajq_w4a16_gemv_rowscale(p, p, 352, 1e-5, 12, 5632, p, p, 16, p, 0, 0, None) == -4
+    assert lib.ajq_w8a16_gemv_rowscale(p, p, 512, 1e-5, 32, 8192, p, p, 16, p, 0, 0, None) == -4
+    assert lib.ajq_w4a16_gemv_rowscale(p, p, 64, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2     # parts is not K / 16
+    assert lib.ajq_w4a16_gemv_norm_sums(p, p, 64, p, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 128, 1e-5, 300, 2048, p, p, 16, p, 0, 0, None) == -4   # more rows than built
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 130, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2   # parts not a multiple of 4
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 260, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2   # more parts than the waves cover
@@ -138,6 +146,36 @@ def test_python_layer_refuses_cpu_tensors():
     with pytest.raises(RuntimeError):
         QuantLinear(128, 16)(torch.zeros(1, 128))
     assert w4a16_matmul.__module__ == "ajllm_amd.quant"
+
+
+def test_state_dict_loading_checks_every_canonical_tensor():
+    """A checkpoint whose scales or zero-points have another shape or dtype is refused like a size mismatch of
+    the reference layer's weight (strict loading, training/checkpoint.py:35-45); the layer stays untouched."""
+    import torch
+
+    from ajllm_amd import QuantLinear
+
+    def w4_state(groups=2, scale_dtype=torch.float16):
+        return {"qweight": torch.zeros(16, 32, dtype=torch.int32), "scales": torch.ones(16, groups, dtype=scale_dtype),
+                "zeros": torch.zeros(16, groups, dtype=torch.uint8)}
+
+    layer = QuantLinear(256, 16)
+    layer.load_state_dict(w4_state())                      # the right shapes load (CPU tensors: nothing is repacked)
+    assert layer.scales.shape == (16, 2)
+    for bad in (w4_state(groups=4), w4_state(scale_dtype=torch.float32)):
+        fresh = QuantLinear(256, 16)
+        with pytest.raises(RuntimeError, match="mismatch for scales"):
+            fresh.load_state_dict(bad)
+        assert fresh.qweight is None and fresh.scales is None
+    state = w4_state()
+    state["zeros"] = torch.zeros(16, 2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="dtype mismatch for zeros"):
+        QuantLinear(256, 16).load_state_dict(state)
+    w8 = {"qweight": torch.zeros(16, 256, dtype=torch.int8), "scales": torch.ones(16, 2, dtype=torch.float16)}
+    with pytest.raises(RuntimeError, match="size mismatch for scales"):
+        QuantLinear(256, 16, scheme="w8a16").load_state_dict(w8)
+    w8["scales"] = torch.ones(16, dtype=torch.float16)
+    QuantLinear(256, 16, scheme="w8a16").load_state_dict(w8)
 
 
 def test_bench_refuses_more_than_one_gpu():

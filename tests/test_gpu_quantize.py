@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import qspec
-from tests.helpers import make_weight
+from tests.helpers import make_weight, tie_and_division_rows
 
 pytestmark = pytest.mark.gpu
 
@@ -25,7 +25,7 @@ def _special_rows(k: int) -> torch.Tensor:
         torch.randn(k, generator=g).abs() * 0.02,                    # one-signed group
         -torch.randn(k, generator=g).abs() * 0.02,
     ]
-    return torch.stack(rows).float()
+    return torch.cat([torch.stack(rows).float(), torch.from_numpy(tie_and_division_rows(k))])
 
 
 @pytest.mark.parametrize("n,k,seed", [(16, 128, 1), (64, 1024, 2), (4096, 4096, 3), (1000, 2048, 4)])

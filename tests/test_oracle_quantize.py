@@ -10,6 +10,7 @@ import pytest
 
 from oracle import qspec
 from tests import pyspec
+from tests.helpers import W4_DIVISION_CASES, W4_ZERO_DIVISION_CASES, W8_DIVISION_CASES
 
 
 # ------------------------------------------------------------------ W8 closed forms
@@ -86,6 +87,73 @@ def test_w4_ties_round_half_to_even_before_the_zero_point_is_added():
     assert float(s[0, 0]) == d and int(z[0, 0]) == 4
     # rint(0.5)=0, rint(1.5)=2, rint(2.5)=2, rint(-0.5)=-0, rint(-1.5)=-2, rint(-2.5)=-2, then +4
     assert list(q[0, :8]) == [0, 15, 4, 6, 6, 4, 2, 2]
+
+
+def test_w4_ties_with_an_odd_zero_point_round_before_the_zero_point_is_added():
+    """With an odd zero-point rint(x) + zero and rint(x + zero) differ at every tie."""
+    d = 2.0**-3
+    group = np.zeros(128, np.float32)
+    group[0], group[1] = -5 * d, 10 * d  # range 15 d -> scale d, zero 5
+    group[2:8] = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5], np.float32) * d
+    q, s, z = qspec.quantize_w4_g128(group[None, :])
+    assert float(s[0, 0]) == d and int(z[0, 0]) == 5
+    # rint: 0.5 -> 0, 1.5 -> 2, 2.5 -> 2, -0.5 -> -0, -1.5 -> -2, -2.5 -> -2, then + 5
+    # (rounding x + 5 instead would give 6, 6, 8, 4, 4, 2)
+    assert list(q[0, :8]) == [0, 15, 5, 7, 7, 5, 3, 3]
+    assert list(q[0, :8]) == pyspec.quantize_w4_group([float(v) for v in group])[0][:8]
+
+
+@pytest.mark.parametrize("below,zero", [(2.5, 2), (3.5, 4), (4.5, 4), (0.5, 0), (14.5, 14)])
+def test_w4_zero_point_ties_round_half_to_even(below, zero):
+    """-min/d exactly on a half: the zero-point is the even neighbour (half-up would give floor + 1)."""
+    d = 2.0**-4
+    group = np.zeros(128, np.float32)
+    group[0], group[1] = -below * d, (15 - below) * d  # max - min = 15 d -> scale d
+    q, s, z = qspec.quantize_w4_g128(group[None, :])
+    assert float(s[0, 0]) == d
+    assert int(z[0, 0]) == zero
+    assert int(z[0, 0]) == pyspec.quantize_w4_group([float(v) for v in group])[2]
+
+
+@pytest.mark.parametrize("scale,weight,by_division,by_reciprocal", W8_DIVISION_CASES)
+def test_w8_divides_rather_than_multiplying_by_a_reciprocal(scale, weight, by_division, by_reciprocal):
+    d = np.float32(np.float16(scale))
+    w = np.float32(float.fromhex(weight))
+    assert int(np.rint(w * (np.float32(1.0) / d))) == by_reciprocal != by_division  # the case does discriminate
+    row = np.zeros(16, np.float32)
+    row[0], row[1] = np.float32(127.0) * d, w  # 127 d is exact in binary32, so the scale is d
+    q, s = qspec.quantize_w8(row[None, :])
+    assert np.float32(s[0]) == d
+    assert int(q[0, 1]) == by_division
+    q_py, s_py = pyspec.quantize_w8_row([float(v) for v in row])
+    assert q_py[1] == by_division and s_py == float(d)
+
+
+@pytest.mark.parametrize("scale,weight,by_division,by_reciprocal", W4_DIVISION_CASES)
+def test_w4_codes_divide_rather_than_multiplying_by_a_reciprocal(scale, weight, by_division, by_reciprocal):
+    d = np.float32(np.float16(scale))
+    w = np.float32(float.fromhex(weight))
+    assert int(np.rint(w * (np.float32(1.0) / d))) + 5 == by_reciprocal != by_division
+    group = np.zeros(128, np.float32)
+    group[0], group[1], group[2] = np.float32(-5.0) * d, np.float32(10.0) * d, w
+    q, s, z = qspec.quantize_w4_g128(group[None, :])
+    assert np.float32(s[0, 0]) == d and int(z[0, 0]) == 5
+    assert int(q[0, 2]) == by_division
+    q_py, s_py, z_py = pyspec.quantize_w4_group([float(v) for v in group])
+    assert q_py[2] == by_division and s_py == float(d) and z_py == 5
+
+
+@pytest.mark.parametrize("scale,mn,mx,by_division,by_reciprocal", W4_ZERO_DIVISION_CASES)
+def test_w4_zero_point_divides_rather_than_multiplying_by_a_reciprocal(scale, mn, mx, by_division, by_reciprocal):
+    d = np.float32(np.float16(scale))
+    lo, hi = np.float32(float.fromhex(mn)), np.float32(float.fromhex(mx))
+    assert int(np.rint(-lo * (np.float32(1.0) / d))) == by_reciprocal != by_division
+    group = np.zeros(128, np.float32)
+    group[0], group[1] = lo, hi
+    _, s, z = qspec.quantize_w4_g128(group[None, :])
+    assert np.float32(s[0, 0]) == d
+    assert int(z[0, 0]) == by_division
+    assert pyspec.quantize_w4_group([float(v) for v in group])[2] == by_division
 
 
 def test_w4_constant_group_and_one_signed_group():
@@ -172,3 +240,20 @@ def test_argument_errors():
         qspec.pack_int4(np.full((1, 8), 16, np.uint8))
     with pytest.raises(ValueError):
         qspec.pack_int4(np.zeros((1, 7), np.uint8))
+
+
+def test_corner_rows_shared_with_the_gpu_tests_hold_the_expected_codes():
+    """The rows the HIP quantizers are given carry the same cases: check the oracle's answer on them."""
+    from tests.helpers import tie_and_division_rows
+
+    w = tie_and_division_rows(512)
+    q8, _ = qspec.quantize_w8(w)
+    q4, _, z4 = qspec.quantize_w4_g128(w)
+    assert list(q4[0, :8]) == [0, 15, 5, 7, 7, 5, 3, 3] and int(z4[0, 0]) == 5
+    assert list(z4[1]) == [2, 4, 4, 14]
+    for i, (_, _, by_division, _) in enumerate(W8_DIVISION_CASES):
+        assert int(q8[2 + i, 1]) == by_division
+    for g, (_, _, by_division, _) in enumerate(W4_DIVISION_CASES):
+        assert int(q4[5, 128 * g + 2]) == by_division and int(z4[5, g]) == 5
+    for g, (_, _, _, by_division, _) in enumerate(W4_ZERO_DIVISION_CASES):
+        assert int(z4[6, g]) == by_division
