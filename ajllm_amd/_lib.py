@@ -124,19 +124,13 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
 }
 
-# libajq_bench.so (include/ajq_bench.h): measurement probes for bench.py, not operators
+# libajq_bench.so (include/ajq_bench.h): the device yardstick for bench.py, not an operator
 BENCH_LIBRARY_PATH = Path(__file__).resolve().parent / "libajq_bench.so"
-
-
-class BenchResult(ctypes.Structure):
-    _fields_ = [("name", ctypes.c_char * 112), ("us_per_stage", ctypes.c_double), ("frac_hbm_peak", ctypes.c_double),
-                ("matches_reference", c_int), ("error_word", c_int)]
 
 
 BENCH_SIGNATURES: dict[str, tuple] = {
     "ajqb_last_error": (c_char_p, []),
     "ajqb_mfma_rate": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
-    "ajqb_launch_alternatives": (c_int, [c_int, c_int, ctypes.POINTER(BenchResult), c_int, ctypes.POINTER(c_int)]),
 }
 
 _lib: ctypes.CDLL | None = None

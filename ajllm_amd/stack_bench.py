@@ -64,7 +64,10 @@ def _eager_linear_seconds(model, rows: int, device) -> float:
 
 @torch.no_grad()
 def bench_stack(device, log=print, config: dict | None = None, batch: int = BATCH, context: int = CONTEXT,
-                decode_steps: int = 32, scheme: str = "w8a16", kv_dtype: torch.dtype | None = None) -> dict:
+                decode_steps: int = 32, scheme: str = "w8a16", kv_dtype: torch.dtype | None = None,
+                short: bool = False) -> dict:
+    """``short`` (the default bench line's leg) leaves out the pass through the model's own PyTorch code and the
+    two decoder options (bf16 cache, activations rounded before the norm's row scale)."""
     config = dict(config or CONFIG)
     t0 = time.perf_counter()
     model = build_quantized_model(device, scheme, seed=4321, config=config)
@@ -84,11 +87,13 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     torch.cuda.synchronize()
     # (a) the model's own PyTorch code around the library's GEMMs and flash attention, one pass
     dec.cache.static = False
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    eager_logits = model(prompt[:PREFILL_ROWS], dec.cache.rows(0, PREFILL_ROWS), last_token_only=True)[:, -1, :]
-    torch.cuda.synchronize()
-    t_pass_eager = time.perf_counter() - t0
+    eager_logits, t_pass_eager = None, None
+    if not short:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eager_logits = model(prompt[:PREFILL_ROWS], dec.cache.rows(0, PREFILL_ROWS), last_token_only=True)[:, -1, :]
+        torch.cuda.synchronize()
+        t_pass_eager = time.perf_counter() - t0
     # (b) library kernels only, every pass (this is what fills the cache the decode below starts from)
     pass_times = []
     logits = []
@@ -101,11 +106,13 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
     pass_times.sort()
     t_pass = pass_times[len(pass_times) // 2]
     t_pass_linear = _eager_linear_seconds(model, PREFILL_ROWS * context, device)
-    logits_rel = float((eager_logits.double() - logits[0].double()).norm() / eager_logits.double().norm())
-    top2 = torch.topk(eager_logits.float(), 2, dim=-1).values
-    first_match = {"rows_with_equal_argmax": int((torch.argmax(eager_logits, -1) == torch.argmax(logits[0], -1)).sum()),
-                   "rows": PREFILL_ROWS, "smallest_top2_margin": float((top2[:, 0] - top2[:, 1]).min()),
-                   "largest_logit_difference": float((eager_logits.float() - logits[0].float()).abs().max())}
+    logits_rel, first_match = None, None
+    if eager_logits is not None:
+        logits_rel = float((eager_logits.double() - logits[0].double()).norm() / eager_logits.double().norm())
+        top2 = torch.topk(eager_logits.float(), 2, dim=-1).values
+        first_match = {"rows_with_equal_argmax": int((torch.argmax(eager_logits, -1) == torch.argmax(logits[0], -1)).sum()),
+                       "rows": PREFILL_ROWS, "smallest_top2_margin": float((top2[:, 0] - top2[:, 1]).min()),
+                       "largest_logit_difference": float((eager_logits.float() - logits[0].float()).abs().max())}
     # hand the prefilled cache to the decoder (what FusedDecoder.prefill does after its passes)
     dec.cache.length = context
     dec.cache.static = True
@@ -175,7 +182,10 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
                    "kv_cache_dtype": str(dec.cache.keys[0].dtype).replace("torch.", ""),
                    "first_tokens_row0": tokens[0, :8].tolist()},
     }
-    if kv_dtype is None:
+    result["decode"]["launches_per_step"] = dec.launches_per_step()
+    if short:
+        result["prefill"] = {k: v for k, v in result["prefill"].items() if v is not None}
+    if kv_dtype is None and not short:
         # the same decode with a bf16 KV cache (keys and values rounded on write; arithmetic fp32):
         # the attention's bytes halve
         del dec

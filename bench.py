@@ -14,7 +14,8 @@ Default run (what the driver calls: ``python bench.py --gpus 1 --steps K --warmu
   linear timed on this box's host cores for the same GEMV shape.
 
 * also after it: the end-to-end greedy decode of the 12-layer W4A16 model (prompt 512 + 256 tokens,
-  batch 1 and 8) in tokens/s, short form.
+  batch 1 and 8) in tokens/s, short form, and the Llama-3-8B-shaped W8A16 stack (4 x 2048 prefill passes,
+  batch-32 decode at context 2048 with the quantized linears' share of the step), short form.
 
 ``--sweep`` adds the rest of the decode sweep (three shapes x M in {1, 4, 16}, W4 and W8)
 and all prefill shapes; ``--decode`` replaces the short decode leg by the long one (eager PyTorch loop
@@ -35,6 +36,8 @@ import torch
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, vendor peak
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, vendor peak
 GEMV_W4_4096_M1_HBM_BYTES = 9.03e6  # measured: 4407.6 KiB x 1.9993 fetched + 8 KiB x 1.0 written per launch
+GEMV_W4_4096_M1_HBM_BYTES_SOURCE = ("constant from profiles/gemv_w4_m1_4096_hbm_traffic.md (separate rocprofv3 --pmc "
+                                    "FETCH_SIZE and WRITE_SIZE runs of this command), not measured by this run")
 
 
 def log(*args) -> None:
@@ -240,32 +243,6 @@ def bench_mfma_rate(device, workgroups: int = 256, iters: int = 100_000, launche
     return out
 
 
-def bench_launch_alternatives(stages: int = 64, reps: int = 20) -> list[dict]:
-    """What a chain of 8.7 MB GEMVs costs per matrix under the alternatives to one launch per matrix
-    (``ajqb_launch_alternatives``: launches in a HIP graph, prefetch on a second graph branch or inside
-    the kernel, one launch for all stages with the activations exchanged through device memory)."""
-    from ajllm_amd import _lib
-
-    lib = _lib.load_bench()
-    results = (_lib.BenchResult * 32)()
-    count = ctypes.c_int(0)
-    status = lib.ajqb_launch_alternatives(stages, reps, results, 32, ctypes.byref(count))
-    if status:
-        raise RuntimeError(f"ajqb_launch_alternatives: {lib.ajqb_last_error().decode()}")
-    out = []
-    for r in results[: count.value]:
-        row = {"what": r.name.decode(), "us_per_matrix": r.us_per_stage}
-        if r.frac_hbm_peak > 0:
-            row["frac_hbm_peak"] = r.frac_hbm_peak
-        if r.matches_reference >= 0:
-            row["output_equals_reference_chain"] = bool(r.matches_reference)
-        if r.error_word:
-            row["error_word"] = r.error_word
-        out.append(row)
-    return out
-
-
-# ------------------------------------------------------------------ CPU baseline
 def cpu_baseline(m: int, n: int, k: int, budget_s: float = 15.0) -> dict:
     """The oracle's quantized linear (dequantize -> matmul, fp32) on the host cores, same shape
     and seeded inputs as the timed GEMV.  The reference project has no quantized CPU path (its
@@ -397,8 +374,6 @@ def main() -> int:
     ap.add_argument("--decode", action="store_true", help="also time end-to-end greedy decode")
     ap.add_argument("--stack", action="store_true",
                     help="also time the Llama-3-8B-shaped W8A16 stack (4 x 2048 prefill, batch-32 decode at context 2048)")
-    ap.add_argument("--probes", action="store_true",
-                    help="also time the alternatives to one launch per matrix for a chain of GEMVs (bench-only probes)")
     ap.add_argument("--forms", action="store_true",
                     help="also time the decode GEMV's prologue forms against its epilogue forms (norm, gate, residual)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -425,10 +400,11 @@ def main() -> int:
     extras: dict = {}
     if not args.no_extras:
         gemm = []
-        for scheme in ("w4", "w8"):
-            r = bench_gemm(scheme, 2048, 4096, 4096, steps=10, warmup=3, device=device)
-            log("gemm", json.dumps(r))
-            gemm.append(r)
+        for gn in (4096, 14336):  # the prefill configuration's two output widths at the target M = 2048
+            for scheme in ("w4", "w8"):
+                r = bench_gemm(scheme, 2048, gn, 4096, steps=10 if gn == 4096 else 5, warmup=3, device=device)
+                log("gemm", json.dumps(r))
+                gemm.append(r)
         extras["prefill_gemm"] = gemm
         # the headline kernel with 64 times the rows per launch: what it streams once the cost of
         # launching is spread over 559 MB instead of 8.7 MB
@@ -437,10 +413,12 @@ def main() -> int:
         extras["gemv_same_kernel_64x_rows_per_launch"] = tall
         dense = bench_dense_library_gemm(2048, 4096, 4096, steps=10, warmup=3, device=device)
         log("dense library gemm", json.dumps(dense))
+        dense_wide = bench_dense_library_gemm(2048, 14336, 4096, steps=5, warmup=3, device=device)
+        log("dense library gemm", json.dumps(dense_wide))
         rate = bench_mfma_rate(device)
         log("mfma rate", json.dumps(rate))
         extras["yardsticks"] = {
-            "dense_bf16_library_gemm": [dense],
+            "dense_bf16_library_gemm": [dense, dense_wide],
             "mfma_from_registers": rate,
             "note": "not part of the product path: the vendor library's plain bf16 GEMM on weights already "
                     "expanded to bf16, and the MFMA rate sustained with no memory traffic (random operands "
@@ -492,18 +470,19 @@ def main() -> int:
         from ajllm_amd.e2e_bench import bench_decode  # heavy import kept off the default path
 
         extras["decode"] = bench_decode(device, log)
-    if args.probes:
-        extras["gemv_chain_launch_alternatives"] = bench_launch_alternatives()
-        for row in extras["gemv_chain_launch_alternatives"]:
-            log("probe", json.dumps(row))
     if args.forms:
         extras["decode_gemv_forms"] = bench_gemv_forms(device)
         for row in extras["decode_gemv_forms"]:
             log("forms", json.dumps(row))
-    if args.stack:
+    if args.stack or not (args.no_extras or args.no_decode):
+        # the Llama-3-8B-shaped W8A16 stack: one 4 x 2048 prefill pass per four sequences, then batch-32 decode at
+        # context 2048 with the quantized linears' and the attention's share of the step; the default line carries
+        # the short form (fp32 cache, reference rounding only), --stack adds the decoder's two options
         from ajllm_amd.stack_bench import bench_stack
 
-        extras["stack_8b_w8a16"] = bench_stack(device, log)
+        torch.cuda.empty_cache()
+        extras["stack_8b_w8a16"] = bench_stack(device, log, short=not args.stack)
+        torch.cuda.empty_cache()
     # a plain device-to-device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     # counters of a profiling run are scaled by (64 MiB read + 64 MiB written per launch)
     calib_src = torch.empty(64 * 2**20, dtype=torch.uint8, device=device)
@@ -544,6 +523,7 @@ def main() -> int:
             # HBM bytes per launch from separate rocprofv3 --pmc runs of this command
             # (FETCH_SIZE, WRITE_SIZE, each scaled by what a 64 MiB copy reads on the same counter)
             "traffic": GEMV_W4_4096_M1_HBM_BYTES,
+            "traffic_source": GEMV_W4_4096_M1_HBM_BYTES_SOURCE,
             "kernel": "ajq::dequant_gemv_kernel<8, 4, 1, true, true, true>",
             "algorithmic_bytes_per_launch": head["bytes_per_launch"],
             "avg_launch_us": head["us_per_launch"],

@@ -225,7 +225,9 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
  * allocates and frees nothing; shapes whose ajq_w4a16_gemm_workspace_bytes(M, K) exceeds the
  * array return AJQ_ERR_WORKSPACE.  All calls on one GPU share the array: two calls that overlap
  * in time on one GPU (different streams, or threads) race on it; calls on one stream do not.
- * The first call on a device resolves the array's address and should not run under capture. */
+ * The first call on a device resolves the array's address and should not run under capture.  The array used is
+ * the CURRENT device's (hipGetDevice at the time of the call): that device must be the one `stream` and every
+ * pointer belong to. */
 size_t ajq_noalloc_scratch_bytes(void);
 int ajq_w4a16_gemm_noalloc(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                            void* y, int out_dtype, void* stream);

@@ -467,26 +467,3 @@ def test_gemv_residual_then_rowscale_against_the_oracle(cuda, scheme, m, k1, d, 
     assert lib.ajq_gemv_epilogue_supported(256, 2048) == 0 and lib.ajq_gemv_epilogue_supported(9, 5632) == 1
     assert row_fn(xt.data_ptr(), ssq.data_ptr(), 6, eps, m, d, wq2.data_ptr(), meta2.data_ptr(), n2, y.data_ptr(),
                   _lib.AJQ_OUT_F32, 0, st) != 0
-
-
-
-def test_launch_alternative_probes_reproduce_the_reference_chain(cuda):
-    """The bench-only probes of the alternatives to one launch per matrix (a chain of dependent GEMV
-    stages in ONE launch, activations exchanged through device memory behind flags or as stamped
-    records): a short run must finish without touching a spin limit and every dependent variant must
-    reproduce the per-stage-launch chain's last output bit for bit.  Timings are measurements, not
-    pass criteria."""
-    import ctypes
-
-    from ajllm_amd import _lib
-    lib = _lib.load_bench()
-    results = (_lib.BenchResult * 32)()
-    count = ctypes.c_int(0)
-    status = lib.ajqb_launch_alternatives(8, 2, results, 32, ctypes.byref(count))
-    assert status == 0, lib.ajqb_last_error().decode()
-    rows = results[: count.value]
-    assert len(rows) >= 12
-    compared = [r for r in rows if r.matches_reference >= 0]
-    assert len(compared) == 3 and all(r.matches_reference == 1 for r in compared)
-    assert all(r.error_word == 0 and r.us_per_stage > 0 for r in rows)
-    assert lib.ajqb_launch_alternatives(2, 2, results, 32, ctypes.byref(count)) == -2
