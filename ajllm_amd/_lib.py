@@ -40,6 +40,7 @@ SIGNATURES: dict[str, tuple] = {
     "ajq_w4a16_gemv": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_w8a16_gemv": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_w4a16_gemm_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "ajq_w4a16_gemm_workspace_bytes_for": (c_size_t, [c_int, c_int, c_int]),
     "ajq_w4a16_gemm": (
         c_int,
         [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_size_t, c_void_p],

@@ -10,6 +10,8 @@
 #include "gemv_fused_kernels.h"
 #include "gemm_kernels.h"
 #include "gemm_ring_kernels.h"
+#include "gemm_split_kernels.h"
+#include "gemm_wide_kernels.h"
 #include "gemm128_kernels.h"
 #include "skinny_kernels.h"
 #include "decode_kernels.h"
@@ -109,37 +111,42 @@ int check_matmul_args(const char* name, const void* x, int M, int K, const void*
   return AJQ_OK;
 }
 
-// 256 x 128 tiles on 32x32x16 MFMA; M >= 256 (the last row tile is shifted, not masked)
-template <int MT, bool kW4, bool kGate = false>
-int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
-                   const uint16_t* scales8, const void* gs3, int N, void* y, int out_f32, hipStream_t stream) {
-  const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
-#ifndef AJQ_G2_RING
-#define AJQ_G2_RING 1
+// 256-row tiles on 32x32x16 MFMA; M >= 256 (the last row tile is shifted, not masked).  Shapes with enough tiles
+// take 256 x 256 ones (gemm_wide_kernels.h); otherwise 256 x 128: W8 with K % 256 == 0
+// runs the ring kernel (four compute waves that unpack their own weights, a loader wave); W4, and W8 on any other
+// K % 128 == 0, the split-role kernel (four compute waves, four producers that dequantize once per workgroup; W4
+// needs no group sums there).
+#ifndef AJQ_GEMM_WIDE
+#define AJQ_GEMM_WIDE 1
 #endif
-  if (AJQ_G2_RING && !kW4 && K % 256 == 0) {
-    // W8: the same tiles with the operands in a ring of four 64-k stages, loaded by a wave of its own
+template <bool kW4, bool kGate = false>
+int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                   int N, void* y, int out_f32, hipStream_t stream) {
+  const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
+  if (!kGate) {
+    // 256 x 256 tiles move half the activation bytes per MFMA and measure 9-15 % faster per flop, but there are half
+    // as many of them: they run when that still fills the CUs' rounds better (a wide tile takes 2 / 1.12 narrow ones)
+    const long long wide = (long long)((M + kGWBM - 1) / kGWBM) * ((N + kGWBN - 1) / kGWBN);
+    const double cost_wide = (double)((wide + 255) / 256) * (2.0 / 1.12), cost_narrow = (double)((tiles + 255) / 256);
+    if (AJQ_GEMM_WIDE && cost_wide < cost_narrow) {
+      auto kernel = dequant_gemm256w_kernel<kW4>;
+      if (int s = allow_big_lds(kernel, kGWLdsBytes)) return s;
+      hipLaunchKernelGGL(kernel, dim3((unsigned)wide), dim3(kGWThreads), kGWLdsBytes, stream, x, M, K,
+                         reinterpret_cast<const u32x4_t*>(wq), meta, scales8, N, y, out_f32);
+      return AJQ_OK;
+    }
+  }
+  if (!kW4 && K % 256 == 0) {
     auto ring = dequant_gemm256r_w8_kernel<kGate>;
     if (int s = allow_big_lds(ring, kGRLdsBytes)) return s;
     hipLaunchKernelGGL(ring, dim3(tiles), dim3(kGRThreads), kGRLdsBytes, stream, x, M, K,
                        reinterpret_cast<const u32x4_t*>(wq), scales8, N, y, out_f32);
     return AJQ_OK;
   }
-#ifndef AJQ_G2_RING4
-#define AJQ_G2_RING4 1
-#endif
-  if (AJQ_G2_RING4 && kW4 && K % 256 == 0) {
-    auto ring = dequant_gemm256r_w4_kernel<kGate>;
-    if (int s = allow_big_lds(ring, kGR4LdsBytes)) return s;
-    hipLaunchKernelGGL(ring, dim3(tiles), dim3(kGRThreads), kGR4LdsBytes, stream, x, M, K,
-                       reinterpret_cast<const u32x4_t*>(wq), meta, reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
-    return AJQ_OK;
-  }
-  auto kernel = dequant_gemm256_kernel<MT, kW4, kGate>;
-  if (int s = allow_big_lds(kernel, kG2LdsBytes)) return s;
-  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(1024 / MT), kG2LdsBytes, stream, x, M, K,
-                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8,
-                     reinterpret_cast<const u32x4_t*>(gs3), N, y, out_f32);
+  auto split = dequant_gemm256s_kernel<kW4, kGate>;
+  if (int s = allow_big_lds(split, kGSLdsBytes)) return s;
+  hipLaunchKernelGGL(split, dim3(tiles), dim3(kGSThreads), kGSLdsBytes, stream, x, M, K,
+                     reinterpret_cast<const u32x4_t*>(wq), meta, scales8, N, y, out_f32);
   return AJQ_OK;
 }
 
@@ -164,12 +171,6 @@ int launch_gemm128(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 #define AJQ_GEMM256_MIN_M 256
 #endif
 constexpr int kGemm256MinM = AJQ_GEMM256_MIN_M;
-#ifndef AJQ_G2_MT_W4
-#define AJQ_G2_MT_W4 2
-#endif
-#ifndef AJQ_G2_MT_W8
-#define AJQ_G2_MT_W8 4
-#endif
 
 }  // namespace
 
@@ -942,8 +943,13 @@ int ajq_w8a16_gemv_merge_residual(const float* partial, int S, int M, int K, con
 
 // --------------------------------------------------------------- GEMM -----
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K) {
-  if (M < kG1BM || K < kGroup) return 0;  // only the tile kernels need the group sums
+  if (M < kG1BM || K < kGroup) return 0;  // only the 128 x 128 tile kernel needs the group sums
   return (size_t)(K / kGroup) * M * 16;
+}
+
+size_t ajq_w4a16_gemm_workspace_bytes_for(int M, int N, int K) {
+  if (M <= kMaxGemvM || N < 1 || K < kGroup || pick_matmul_kernel(M, N, K, true) != kTiles128) return 0;
+  return ajq_w4a16_gemm_workspace_bytes(M, K);
 }
 
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
@@ -956,20 +962,20 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
                                  : launch_skinny<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream);
     return s ? s : check_launch("ajq_w4a16_gemm");
   }
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  if (which == kTiles256) {  // zero-points are subtracted when the weights are unpacked: no group sums, one launch
+    if (int s = launch_gemm256<true>(x, M, K, wq, meta, nullptr, N, y, out_f32, (hipStream_t)stream)) return s;
+    return check_launch("ajq_w4a16_gemm");
+  }
   const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
   if (!workspace || workspace_bytes < need)
     return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm: workspace must be 16-byte aligned");
-  if ((long long)M * K * 2 >= (1LL << 32))
-    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
   const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
   hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
                      K, reinterpret_cast<u32x4_t*>(workspace));
-  if (int s = which == kTiles128
-                  ? launch_gemm128<true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32, (hipStream_t)stream)
-                  : launch_gemm256<AJQ_G2_MT_W4, true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32,
-                                                       (hipStream_t)stream))
-    return s;
+  if (int s = launch_gemm128<true>(x, M, K, wq, meta, nullptr, workspace, N, y, out_f32, (hipStream_t)stream)) return s;
   return check_launch("ajq_w4a16_gemm");
 }
 
@@ -978,7 +984,8 @@ size_t ajq_noalloc_scratch_bytes(void) { return kScratchBytes; }
 int ajq_w4a16_gemm_noalloc(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
                            int out_dtype, void* stream) {
   if (M < 1 || K < 1) return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_noalloc: M and K must be positive (got %d, %d)", M, K);
-  const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
+  if (N < 1) return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_noalloc: N must be positive (got %d)", N);
+  const size_t need = ajq_w4a16_gemm_workspace_bytes_for(M, N, K);
   if (need > kScratchBytes)
     return fail(AJQ_ERR_WORKSPACE,
                 "ajq_w4a16_gemm_noalloc: M=%d, K=%d needs %zu bytes of group sums, the built-in scratch holds %zu "
@@ -1002,8 +1009,7 @@ int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
     return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
   if (int s = which == kTiles128
                   ? launch_gemm128<false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32, (hipStream_t)stream)
-                  : launch_gemm256<AJQ_G2_MT_W8, false>(x, M, K, wq, nullptr, scales, nullptr, N, y, out_f32,
-                                                        (hipStream_t)stream))
+                  : launch_gemm256<false>(x, M, K, wq, nullptr, scales, N, y, out_f32, (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemm");
 }
@@ -1021,20 +1027,20 @@ int ajq_w4a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, con
   if (!ajq_gemm_gate_supported(M, N2, K, 1))
     return fail(AJQ_ERR_UNSUPPORTED, "ajq_w4a16_gemm_gate: M=%d, N=%d, K=%d is not a tile-kernel shape with N %% 128 == 0", M,
                 N2, K);
+  if ((long long)M * K * 2 >= (1LL << 32))
+    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_gate: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
+  if (pick_matmul_kernel(M, N2, K, true) == kTiles256) {  // no group sums, no workspace
+    if (int s = launch_gemm256<true, true>(x, M, K, wq, meta, nullptr, N2, y, 0, (hipStream_t)stream)) return s;
+    return check_launch("ajq_w4a16_gemm_gate");
+  }
   const size_t need = ajq_w4a16_gemm_workspace_bytes(M, K);
   if (!workspace || workspace_bytes < need)
     return fail(AJQ_ERR_WORKSPACE, "ajq_w4a16_gemm_gate: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_w4a16_gemm_gate: workspace must be 16-byte aligned");
-  if ((long long)M * K * 2 >= (1LL << 32))
-    return fail(AJQ_ERR_SHAPE, "ajq_w4a16_gemm_gate: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
   const long long teams4 = (long long)M * ((K / kGroup + 3) / 4);
   hipLaunchKernelGGL(group_sum3_kernel, dim3((unsigned)((teams4 + 15) / 16)), dim3(256), 0, (hipStream_t)stream, x, M,
                      K, reinterpret_cast<u32x4_t*>(workspace));
-  if (int s = pick_matmul_kernel(M, N2, K, true) == kTiles128
-                  ? launch_gemm128<true, true>(x, M, K, wq, meta, nullptr, workspace, N2, y, 0, (hipStream_t)stream)
-                  : launch_gemm256<AJQ_G2_MT_W4, true, true>(x, M, K, wq, meta, nullptr, workspace, N2, y, 0,
-                                                             (hipStream_t)stream))
-    return s;
+  if (int s = launch_gemm128<true, true>(x, M, K, wq, meta, nullptr, workspace, N2, y, 0, (hipStream_t)stream)) return s;
   return check_launch("ajq_w4a16_gemm_gate");
 }
 
@@ -1048,8 +1054,7 @@ int ajq_w8a16_gemm_gate(const uint16_t* x, int M, int K, const uint32_t* wq, con
     return fail(AJQ_ERR_SHAPE, "ajq_w8a16_gemm_gate: M * K = %lld exceeds the 32-bit activation offsets", (long long)M * K);
   if (int s = pick_matmul_kernel(M, N2, K, false) == kTiles128
                   ? launch_gemm128<false, true>(x, M, K, wq, nullptr, scales, nullptr, N2, y, 0, (hipStream_t)stream)
-                  : launch_gemm256<AJQ_G2_MT_W8, false, true>(x, M, K, wq, nullptr, scales, nullptr, N2, y, 0,
-                                                              (hipStream_t)stream))
+                  : launch_gemm256<false, true>(x, M, K, wq, nullptr, scales, N2, y, 0, (hipStream_t)stream))
     return s;
   return check_launch("ajq_w8a16_gemm_gate");
 }

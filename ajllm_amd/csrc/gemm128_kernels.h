@@ -2,9 +2,11 @@
 // short of workgroups (M between 128 and about 1500 on N = 4096: 32 ... 192 big tiles for 256
 // CUs).
 //
-// Same arithmetic and operand paths as dequant_gemm256_kernel (everything enters LDS by DMA;
-// exact integers in bf16 through v_mfma_f32_32x32x16_bf16, scales in fp32, the W4 zero-point as
-// a ninth k-step against the three bf16 pieces of the activations' group sums), eight waves as
+// Everything enters LDS by DMA (activations, the packed private weight tiles of the workgroup's columns, the W4
+// meta words); a wave unpacks the weights of its own columns just in time to exact integers in bf16 (128 + q for
+// int4, q for int8) for v_mfma_f32_32x32x16_bf16; scales stay fp32 (per group for W4: acc += s * part, once per
+// channel for W8).  The W4 zero-point is a ninth k-step per group: -(128 + z) against the three bf16 pieces of the
+// activations' per-row group sums (group_sum3_kernel, a launch of its own in front of this one).  Eight waves as
 // 2 x 4 with 64 x 32 wave tiles, K walked in blocks of 128.  What differs: a workgroup has a CU
 // to itself, and a k-block is 36 MFMAs per SIMD, about half a microsecond: less than a trip to
 // memory.  So the tiles travel in a ring of THREE buffers and
@@ -32,7 +34,7 @@ constexpr size_t kG1LdsBytesW8 = kG1WBase + kG1Ring * kG1W8Slot;       // 144 Ki
 // SIMD always has a second instruction stream to issue from).
 // kGate (kWN = 4 only): w1 | w3 weights of a SwiGLU feed-forward, output bf16( silu(a) * u ),
 // [M, N / 2]; the workgroup's four 32-column blocks alternate between the two halves as in
-// dequant_gemm256_kernel, here one block per wave, so the pairs meet in an fp32 staging tile.
+// the 256 x 128 kernels, here one block per wave, so the pairs meet in an fp32 staging tile.
 template <bool kW4, int kWN, bool kGate = false>
 __global__ __launch_bounds__(128 * kWN) void dequant_gemm128_kernel(
     const uint16_t* __restrict__ x, int M, int K, const u32x4_t* __restrict__ wq,

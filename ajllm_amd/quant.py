@@ -177,8 +177,8 @@ def w4a16_matmul(
                 x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n16, y.data_ptr(), flag, _stream()
             )
         else:
-            nbytes = lib.ajq_w4a16_gemm_workspace_bytes(m, k)
-            workspace = torch.empty((nbytes,), dtype=torch.uint8, device=x.device)
+            nbytes = lib.ajq_w4a16_gemm_workspace_bytes_for(m, n16, k)  # 0 unless the 128 x 128 tile kernel runs
+            workspace = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=x.device)
             status = lib.ajq_w4a16_gemm(
                 x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n16, y.data_ptr(), flag,
                 workspace.data_ptr(), nbytes, _stream(),

@@ -209,10 +209,13 @@ int ajq_w8a16_gemv_merge(const float* partial, int S, int M, int K, const uint32
  * together) a weight-streaming kernel with 32-row activation blocks, and from M = 128 on the
  * fastest by a measured cost model of that kernel, a 128 x 128 tile kernel (shapes with few
  * tiles) and a 256 x 128 tile kernel (M >= 256, prefill).
- * The W4 GEMM needs a workspace of ajq_w4a16_gemm_workspace_bytes(M, K) bytes (per-row,
- * per-group activation sums for the tile kernels; 0 bytes below M = 128, where workspace may
- * be NULL). */
+ * Of the W4 kernels only the 128 x 128 tile kernel needs a workspace (per-row, per-group activation sums): the
+ * 256 x 128 tile kernel subtracts the zero-points when it unpacks the weights and runs as one launch.
+ * ajq_w4a16_gemm_workspace_bytes_for(M, N, K) is what a call on that shape needs (0 unless the 128 x 128 kernel
+ * is chosen; workspace may then be NULL); ajq_w4a16_gemm_workspace_bytes(M, K) is its upper bound over all N
+ * (0 below M = 128). */
 size_t ajq_w4a16_gemm_workspace_bytes(int M, int K);
+size_t ajq_w4a16_gemm_workspace_bytes_for(int M, int N, int K);
 int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N,
                    void* y, int out_dtype, void* workspace, size_t workspace_bytes, void* stream);
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,

@@ -86,9 +86,13 @@ def test_shape_alignment_and_option_errors():
     assert need == 4 * 300 * 16                                             # G=4 groups x 300 rows x 16 bytes
     assert lib.ajq_w4a16_gemm_workspace_bytes(127, 512) == 0                 # below 128 rows no tile kernel runs: no workspace
     assert lib.ajq_attn_decode(p, p, p, 0, p, 1, 16, 2, 128, 8, p, p, 1 << 20, None) == -4  # 8 query heads per cache head
-    need = lib.ajq_w4a16_gemm_workspace_bytes(2048, 4096)                    # a shape the tile kernel takes
-    assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, None, 0, None) == -6
-    assert lib.ajq_w4a16_gemm(p, 2048, 4096, p, p, 4096, p, 0, p, need - 1, None) == -6
+    # only the 128 x 128 tile kernel takes group sums: M = 1024 on 4096 x 4096 runs it, M = 2048 the 256 x 128 kernel
+    need = lib.ajq_w4a16_gemm_workspace_bytes_for(1024, 4096, 4096)
+    assert need == 32 * 1024 * 16 == lib.ajq_w4a16_gemm_workspace_bytes(1024, 4096)
+    assert lib.ajq_w4a16_gemm_workspace_bytes_for(2048, 4096, 4096) == 0
+    assert lib.ajq_w4a16_gemm_workspace_bytes_for(40, 4096, 4096) == 0 == lib.ajq_w4a16_gemm_workspace_bytes_for(8, 4096, 4096)
+    assert lib.ajq_w4a16_gemm(p, 1024, 4096, p, p, 4096, p, 0, None, 0, None) == -6
+    assert lib.ajq_w4a16_gemm(p, 1024, 4096, p, p, 4096, p, 0, p, need - 1, None) == -6
     # matmuls with a residual / row-scale / gate epilogue: which (M, K) are built, and what is refused before any launch
     assert lib.ajq_gemv_epilogue_supported(1, 2048) == 1 and lib.ajq_gemv_epilogue_supported(16, 4096) == 1
     assert lib.ajq_gemv_epilogue_supported(9, 5632) == 1 and lib.ajq_gemv_epilogue_supported(200, 14336) == 1   # streaming kernel

@@ -23,7 +23,7 @@ def _both(lib, x, wq, meta, n, k, out_dtype):
     m = x.shape[0]
     flag = _lib.AJQ_OUT_F32 if out_dtype == torch.float32 else _lib.AJQ_OUT_BF16
     stream = torch.cuda.current_stream().cuda_stream
-    nbytes = lib.ajq_w4a16_gemm_workspace_bytes(m, k)
+    nbytes = lib.ajq_w4a16_gemm_workspace_bytes_for(m, n, k)
     workspace = torch.empty((max(nbytes, 16),), dtype=torch.uint8, device=x.device)
     want = torch.empty((m, n), dtype=out_dtype, device=x.device)
     _lib.check(lib.ajq_w4a16_gemm(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, want.data_ptr(), flag,
@@ -56,9 +56,9 @@ def test_noalloc_gemm_equals_workspace_gemm_twice(cuda):
     lib = _lib.load()
     n, k = 4096, 4096
     wq, meta = _private_w4(n, k, 31, cuda)
-    # first call: 256 x 128 tiles (M = 2048); second, smaller: 128 x 128 tiles (M = 384) and a
-    # third below the tile kernels (M = 40: no group sums at all)
-    for m, out_dtype in ((2048, torch.float32), (384, torch.bfloat16), (40, torch.float32), (2048, torch.bfloat16)):
+    # 128 x 128 tiles (M = 1024, then the smaller M = 384: the kernels that keep their group sums in the scratch),
+    # then shapes that need none: below the tile kernels (M = 40) and 256 x 128 tiles (M = 2048)
+    for m, out_dtype in ((1024, torch.float32), (384, torch.bfloat16), (40, torch.float32), (2048, torch.bfloat16)):
         x = make_activations(m, k, 500 + m, outliers=True).to(cuda)
         got, want = _both(lib, x, wq, meta, n, k, out_dtype)
         assert torch.equal(got, want), (m, out_dtype)
@@ -71,7 +71,7 @@ def test_noalloc_gemm_runs_under_graph_capture(cuda):
     from ajllm_amd import _lib
 
     lib = _lib.load()
-    n, k, m = 1024, 2048, 512
+    n, k, m = 4096, 4096, 1024  # 128 x 128 tiles: the kernels whose group sums live in the scratch
     wq, meta = _private_w4(n, k, 33, cuda)
     x = make_activations(m, k, 77, outliers=True).to(cuda)
     want = torch.empty((m, n), dtype=torch.float32, device=cuda)
@@ -104,11 +104,13 @@ def test_noalloc_gemm_rejects_what_does_not_fit(cuda):
     assert cap == 16 << 20
     k = 14336
     m = cap // (16 * (k // 128)) + 128        # one tile row past the array
-    assert lib.ajq_w4a16_gemm_workspace_bytes(m, k) > cap
-    wq, meta = _private_w4(128, k, 32, cuda)
+    n = 256                                   # few tiles: the 128 x 128 kernel, the one that keeps group sums
+    assert lib.ajq_w4a16_gemm_workspace_bytes_for(m, n, k) > cap
+    assert lib.ajq_w4a16_gemm_workspace_bytes_for(m, 4096, k) == 0   # 256 x 128 tiles: nothing to hold, any size fits
+    wq, meta = _private_w4(n, k, 32, cuda)
     x = torch.zeros((m, k), dtype=torch.bfloat16, device=cuda)
-    y = torch.empty((m, 128), dtype=torch.bfloat16, device=cuda)
-    status = lib.ajq_w4a16_gemm_noalloc(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), 128, y.data_ptr(),
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=cuda)
+    status = lib.ajq_w4a16_gemm_noalloc(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(),
                                         _lib.AJQ_OUT_BF16, torch.cuda.current_stream().cuda_stream)
     assert status == -6
     with pytest.raises(ValueError, match="built-in scratch"):
