@@ -123,13 +123,13 @@ template <bool kW4, bool kGate = false>
 int launch_gemm256(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                    int N, void* y, int out_f32, hipStream_t stream) {
   const int tiles = ((M + kG2BM - 1) / kG2BM) * ((N + kG2BN - 1) / kG2BN);
-  if (!kGate) {
+  if (!kGate || (N / 2) % (kGWBN / 2) == 0) {
     // 256 x 256 tiles move half the activation bytes per MFMA and measure 9-15 % faster per flop, but there are half
     // as many of them: they run when that still fills the CUs' rounds better (a wide tile takes 2 / 1.12 narrow ones)
     const long long wide = (long long)((M + kGWBM - 1) / kGWBM) * ((N + kGWBN - 1) / kGWBN);
     const double cost_wide = (double)((wide + 255) / 256) * (2.0 / 1.12), cost_narrow = (double)((tiles + 255) / 256);
     if (AJQ_GEMM_WIDE && cost_wide < cost_narrow) {
-      auto kernel = dequant_gemm256w_kernel<kW4>;
+      auto kernel = dequant_gemm256w_kernel<kW4, kGate>;
       if (int s = allow_big_lds(kernel, kGWLdsBytes)) return s;
       hipLaunchKernelGGL(kernel, dim3((unsigned)wide), dim3(kGWThreads), kGWLdsBytes, stream, x, M, K,
                          reinterpret_cast<const u32x4_t*>(wq), meta, scales8, N, y, out_f32);

@@ -38,7 +38,10 @@ constexpr size_t kGWLdsBytes = (size_t)kGWBM * kGWOutStride;  // 132 KiB (>= the
 constexpr int kGWThreads = 512;
 static_assert(kGWLdsBytes >= (size_t)kGWUnitBase + 2 * 1024, "the output staging covers ring and tables");
 
-template <bool kW4>
+// kGate: the weights are the w1 | w3 rows of a SwiGLU feed-forward (N = 2 F, F % 128 == 0).  A workgroup then takes
+// 128 gate-projection columns and the SAME 128 up-projection columns: its 32-column blocks alternate between the two
+// halves, so a wave's two accumulator blocks are a matching pair, and it writes bf16( silu(a) * u ), [M, F].
+template <bool kW4, bool kGate = false>
 __global__ __launch_bounds__(kGWThreads) void dequant_gemm256w_kernel(const uint16_t* __restrict__ x, int M, int K,
                                                                       const u32x4_t* __restrict__ wq,
                                                                       const uint32_t* __restrict__ meta,     // W4
@@ -56,7 +59,7 @@ __global__ __launch_bounds__(kGWThreads) void dequant_gemm256w_kernel(const uint
   const int tiles_m = (M + kGWBM - 1) / kGWBM;
   const int tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
   const int m0 = min(tile_m * kGWBM, M - kGWBM);
-  const int n0 = tile_n * kGWBN;
+  const int n0 = tile_n * (kGate ? kGWBN / 2 : kGWBN);  // kGate: first of the workgroup's 128 columns of each half
   const int NR = K >> 7;  // rounds of four stages
   const int ntiles16 = N / kTileN;
   const int nt16_0 = n0 / kTileN;
@@ -80,7 +83,9 @@ __global__ __launch_bounds__(kGWThreads) void dequant_gemm256w_kernel(const uint
   uint32_t meta_voff[2];
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int T = min(nt16_0 + 2 * wave + u, ntiles16 - 1);
+    // kGate: wave w's 32-column block is half w & 1 (gate / up), columns 32 (w >> 1) .. of the workgroup's 128
+    const int T = kGate ? (wave & 1) * (ntiles16 >> 1) + nt16_0 + (wave >> 1) * 2 + u
+                        : min(nt16_0 + 2 * wave + u, ntiles16 - 1);
     b_src[u] = wq + (size_t)T * tiles_k * 64;
     meta_voff[u] = (uint32_t)((T * NR * 16 + nl) * 4);
   }
@@ -308,8 +313,32 @@ __global__ __launch_bounds__(kGWThreads) void dequant_gemm256w_kernel(const uint
   float scale[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const int n = n0 + wn * 64 + t * 32 + col;
+    const int n = kGate ? t * (N >> 1) + n0 + wn * 32 + col : n0 + wn * 64 + t * 32 + col;
     scale[t] = kW4 ? cs[t] : f16_bits_to_f32(scales8[min(n, N - 1)]);
+  }
+  if (kGate) {
+    // block 0 holds the gate projection a, block 1 the up projection u of the same 32 columns: bf16( a sigmoid(a) u ),
+    // staged as 256-byte rows 272 bytes apart and stored four rows per wave-wide 128-bit store
+    constexpr int kGateStride = 272;
+    const int F = N >> 1;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = wm * 128 + i * 32 + (e & 3) + 8 * (e >> 2) + 4 * kh;
+        const float a = acc[i][0][e] * scale[0], u = acc[i][1][e] * scale[1];
+        *reinterpret_cast<uint16_t*>(lds + row * kGateStride + (wn * 32 + col) * 2) =
+            f32_to_bf16_rne(a * (1.0f / (1.0f + expf(-a))) * u);
+      }
+    __syncthreads();
+    const int piece = lane & 15, rsub = lane >> 4;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = wave * 32 + j * 4 + rsub;
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(lds + row * kGateStride + piece * 16);
+      *reinterpret_cast<u32x4_t*>(reinterpret_cast<uint16_t*>(y) + (size_t)(m0 + row) * F + n0 + piece * 8) = v;
+    }
+    return;
   }
   if (!out_f32) {
 #pragma unroll

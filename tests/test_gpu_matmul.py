@@ -155,14 +155,40 @@ def test_prefill_gemm_m8192(cuda, scheme, n):
     _check(scheme, "gemm", 8192, n, 4096, seed=32, cuda=cuda, outliers=True, max_rows=128)
 
 
-@pytest.mark.parametrize("m,n,k", [(2048, 4096, 512), (2048, 4096, 1280), (300, 512, 1024), (40, 512, 1024), (4, 512, 1024)])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+@pytest.mark.parametrize("m,n,k", [(4096, 4096, 14336), (2300, 7168, 640), (4096, 3856, 384)])
+def test_prefill_gemm_on_256x256_tiles(cuda, scheme, m, n, k):
+    """Shapes with enough tiles for the 256 x 256 kernel: the longest K of the benchmark models, ragged M (the last
+    row tile shifted up) with an odd number of 128-k rounds, and an N whose last column tile is mostly outside the
+    matrix; fp32 and bf16 outputs."""
+    _check(scheme, "gemm", m, n, k, seed=35, cuda=cuda, outliers=True, max_rows=96)
+
+
+def test_w4_gemm_on_256_row_tiles_takes_no_workspace(cuda):
+    """The 256-row tile kernels subtract the zero-points while unpacking: no group sums, a NULL workspace is fine."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    for m, n, k in ((2048, 4096, 1024), (4096, 4096, 512)):  # 256 x 128 and 256 x 256 tiles
+        assert lib.ajq_w4a16_gemm_workspace_bytes_for(m, n, k) == 0
+        w_hat, wq, meta = _quantized("w4", n, k, 41, cuda)
+        x = make_activations(m, k, 6, True).to(cuda)
+        y = torch.empty((m, n), dtype=torch.float32, device=cuda)
+        _lib.check(lib.ajq_w4a16_gemm(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, y.data_ptr(), _lib.AJQ_OUT_F32,
+                                      None, 0, torch.cuda.current_stream().cuda_stream), "w4 gemm without workspace")
+        torch.cuda.synchronize()
+        want = x.double() @ w_hat.to(cuda).double().t()
+        assert errors(y.double().cpu(), want.cpu())[1] <= 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(2048, 4096, 512), (2048, 4096, 1280), (4096, 4096, 640), (300, 512, 1024), (40, 512, 1024),
+                                   (4, 512, 1024)])
 def test_w4_group_scales_far_apart_and_zero(cuda, m, n, k):
     """W4 columns whose group scales differ by six orders of magnitude from one group to the next, with
     constant-zero groups (scale 0) and constant non-zero groups (scale 0 too: they dequantize to 0) in
     between, first and last.  The tile kernels carry their accumulators in units of the current group's
     scale, so a wrong rescale at a group boundary, or a zero scale, shows as an O(1) error here.  Shapes:
-    256 x 128 tiles on the four-stage ring (K % 256 == 0), the same tiles double-buffered (K = 1280),
-    128 x 128 tiles, the weight-streaming kernel and the GEMV."""
+    256 x 128 tiles (an even and an odd number of groups), 256 x 256 tiles (M = 4096), 128 x 128 tiles, the
+    weight-streaming kernel and the GEMV."""
     from ajllm_amd import repack_w4, w4a16_matmul
 
     gen = torch.Generator().manual_seed(m + n + k)
@@ -295,7 +321,8 @@ def test_matmul_random_shapes(cuda, scheme, m, n, k):
     assert torch.equal(y16, y32.to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("m,f,k", [(256, 7168, 1024), (2048, 2048, 2048), (1000, 3072, 4096), (200, 14336, 4096)])
+@pytest.mark.parametrize("m,f,k", [(256, 7168, 1024), (2048, 2048, 2048), (1000, 3072, 4096), (200, 14336, 4096),
+                                   (4096, 2048, 512), (2300, 3584, 640)])  # the last two: 256 x 256 tiles
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemm_with_gate_epilogue_equals_gemm_then_swiglu(cuda, scheme, m, f, k):
     """ajq_w*a16_gemm_gate on the (w1 | w3) rows: bit for bit the fp32 GEMM followed by ajq_swiglu
