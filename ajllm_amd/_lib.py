@@ -91,6 +91,8 @@ SIGNATURES: dict[str, tuple] = {
     ),
     "ajq_gemv_epilogue_supported": (c_int, [c_int, c_int]),
     "ajq_gemv_rowscale_supported": (c_int, [c_int, c_int]),
+    "ajq_matmul_workspace_bytes": (c_size_t, []),
+    "ajq_matmul_workspace_set": (c_int, [c_void_p, c_size_t]),
     "ajq_w4a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_void_p]),
     "ajq_w8a16_gemv_residual": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,

@@ -417,6 +417,64 @@ int launch_skinny_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, c
   return AJQ_OK;
 }
 
+// ---- split-K form of the weight-streaming kernel (see kSplitK in skinny_kernels.h): only with a buffer the caller
+// has lent to this host thread's calls (ajq_matmul_workspace_set), which holds the ticket words and the partial sums
+constexpr int kSplitTiles = 4, kSplitWays = 4;          // row tiles per workgroup, workgroups per row-tile group
+constexpr size_t kSplitTicketBytes = 4096;              // one word per (row-tile group, row block), zeroed
+constexpr int kSplitMaxCells = 64;                      // 256 workgroups: one round of the chip
+constexpr size_t kSplitCellBytes = (size_t)kSplitWays * kSplitTiles * 2 * 1024;
+constexpr size_t kSplitWorkspaceBytes = kSplitTicketBytes + kSplitMaxCells * kSplitCellBytes;
+struct SplitWorkspace {
+  void* base = nullptr;
+  size_t bytes = 0;
+};
+thread_local SplitWorkspace g_split_ws;
+
+// Whether the split-K form takes (M, N, K): a lent buffer, one round of workgroups, a K that four workgroups share
+// evenly, and enough of it that the activation traffic saved (each row-tile group of four reads the block once
+// instead of four times) outweighs the exchange of partial sums through memory (about 3 us: measured 22.1 -> 17.5 us
+// at N = 4096, K = 14336, M = 32 for int8 weights; no gain at K = 4096).
+bool skinny_split_applies(int M, int N, int K) {
+  if (!g_split_ws.base || g_split_ws.bytes < kSplitWorkspaceBytes) return false;
+  const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
+  const int cells = ((ntiles + kSplitTiles - 1) / kSplitTiles) * mblocks;
+  return K >= 8192 && (K / kGroup) % kSplitWays == 0 && cells <= kSplitMaxCells && ntiles >= kSplitTiles;
+}
+
+template <bool kW4, int kEpi, int kBatches>
+int launch_skinny_split_kernel(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                               const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep,
+                               hipStream_t stream) {
+  constexpr size_t lds = kEpi ? skinny_epi_lds_bytes(8, 1, 32) : skinny_lds_bytes(8, 1, 32);
+  const int ntiles = N / kTileN;
+  const int ngroups = (ntiles + kSplitTiles - 1) / kSplitTiles, mblocks = (M + 31) / 32;
+  const dim3 grid(8 * ((ngroups + 7) / 8) * mblocks * kSplitWays), block(8 * 64);
+  SkinnySplit sp{reinterpret_cast<float*>(static_cast<char*>(g_split_ws.base) + kSplitTicketBytes),
+                 static_cast<unsigned*>(g_split_ws.base), kSplitWays};
+  if constexpr (kEpi != 0) {
+    auto kernel = dequant_skinny_split_epi_kernel<8, 1, 32, kSplitTiles, kW4, kEpi, kBatches>;
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32,
+                       scales8, ep, sp);
+  } else {
+    auto kernel = dequant_skinny_split_kernel<8, 1, 32, kSplitTiles, kW4, kBatches>;
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32,
+                       scales8, sp);
+  }
+  return AJQ_OK;
+}
+
+template <bool kW4, int kEpi>
+int launch_skinny_split(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                        int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  // a workgroup's K / 4 as seven or eight waves' runs of four groups (K = 14336: 28 groups): straight-line code
+  const int count = K / kGroup / kSplitWays;
+  if (count == 28 || count == 32)
+    return launch_skinny_split_kernel<kW4, kEpi, 4>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  return launch_skinny_split_kernel<kW4, kEpi, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+}
+
 #ifndef AJQ_SKINNY_FORCE_NT
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
@@ -450,6 +508,7 @@ int skinny_row_tiles(int M, int N) {
 template <bool kW4, int kEpi>
 int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                       int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  if (skinny_split_applies(M, N, K)) return launch_skinny_split<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   const int nt = skinny_row_tiles<kW4>(M, N);
   const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
   if (nt == 1) return launch_skinny_epi_cfg<8, 2, 32, 1, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
@@ -462,6 +521,8 @@ int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const
 template <bool kW4>
 int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
+  if (skinny_split_applies(M, N, K))
+    return launch_skinny_split<kW4, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
   const int ntiles = N / kTileN;
   const int mblocks = (M + 31) / 32;
   int nt = 1;
@@ -808,6 +869,21 @@ int ajq_gemv_fused_supported(int M, int K) { return gemv_pro_supported(M, K) ? 1
 int ajq_gemv_epilogue_supported(int M, int K) { return gemv_epi_supported(M, K) ? 1 : 0; }
 
 int ajq_gemv_rowscale_supported(int M, int K) { return gemv_rowscale_supported(M, K) ? 1 : 0; }
+
+size_t ajq_matmul_workspace_bytes(void) { return kSplitWorkspaceBytes; }
+
+int ajq_matmul_workspace_set(void* workspace, size_t bytes) {
+  if (!workspace) {
+    g_split_ws = SplitWorkspace{};
+    return AJQ_OK;
+  }
+  if (!aligned16(workspace)) return fail(AJQ_ERR_ALIGN, "ajq_matmul_workspace_set: workspace must be 16-byte aligned");
+  if (bytes < kSplitWorkspaceBytes)
+    return fail(AJQ_ERR_WORKSPACE, "ajq_matmul_workspace_set: %zu bytes needed, %zu given", kSplitWorkspaceBytes, bytes);
+  g_split_ws.base = workspace;
+  g_split_ws.bytes = bytes;
+  return AJQ_OK;
+}
 
 int ajq_w4a16_gemv_gated(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, int N, void* y,
                          void* stream) {

@@ -16,8 +16,18 @@
 //  * the waves' partial sums meet once in LDS (each wave's own region, which it no
 //    longer needs) and are added in wave order: no atomics, run-to-run identical.
 // Every workgroup reads its whole activation block from L2 (MROWS * K * 2 bytes
-// against 16 * K weight bytes or half that), which is what bounds the kernel for
-// M above about 32: a CU's vector memory path moves 64 bytes per clock.
+// against 16 * K * NT weight bytes or half that).  With one row tile per workgroup that
+// is four times the int8 weight stream, and the L2s' delivery to the CUs (about 14 TB/s
+// over the chip, measured) bounds the kernel instead of HBM: 82 MB for a 16.8 MB matrix
+// at K = N = 4096, 293 MB for 58.7 MB at K = 14336.
+//
+// kSplitK: S workgroups share NT row tiles and take 1 / S of K each, so a row-tile group
+// still has S * 8 waves' worth of loads in flight but the activation block is read once
+// per group instead of once per tile (4 tiles x 4 splits: 33.6 MB and 117 MB for the two
+// shapes above).  A workgroup leaves its partial sums in a caller-lent buffer, draws a
+// ticket, and the one that draws the last ticket of its group adds the S partial results
+// in split order (whatever order they arrived in: run-to-run identical) and runs the
+// epilogue.  Nobody waits for anybody, so the kernel cannot hang on scheduling order.
 #pragma once
 #include "gemv_kernels.h"
 
@@ -33,13 +43,21 @@ struct SkinnyBatch {
 // kEpi: the epilogue forms of dequant_gemv_epi_kernel (row scale of an RMSNorm applied to the outputs,
 // residual add with the next norm's preparation, SwiGLU gate on interleaved rows) for more rows than a GEMV
 // takes; ssq_in is [M][parts], ssq_out [M][N / 16].
-template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0>
+// Cross-workgroup part of the split-K form: S splits; `partial` holds S x NT x MROWS / 16 KiB per (row-tile group,
+// row block), `tickets` one zeroed word each, which the kernel leaves zeroed.
+struct SkinnySplit {
+  float* partial;
+  unsigned* tickets;
+  int S;
+};
+
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0, bool kSplitK = false>
 __device__ __forceinline__ void dequant_skinny_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
-    const GemvEpilogue& ep) {
+    const GemvEpilogue& ep, const SkinnySplit& sp = SkinnySplit{}) {
   static_assert(MROWS % 16 == 0, "row block is a whole number of MFMA tiles");
   static_assert(kEpi == 0 || MROWS == 32, "the epilogue forms lay their row sums out for 32-row blocks");
   constexpr int MB = MROWS / 16;
@@ -63,17 +81,21 @@ __device__ __forceinline__ void dequant_skinny_body(
   const int ngroups = (ntiles + NT - 1) / NT;
   const int mblocks = (M + MROWS - 1) / MROWS;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int ng = xcd + 8 * (slot / mblocks);
+  const int S = kSplitK ? sp.S : 1;  // the splits of one (row-tile group, row block) sit in consecutive slots too
+  const int ng = xcd + 8 * (slot / (mblocks * S));
   if (ng >= ngroups) return;  // padding of the last round (whole workgroup: no barrier is left waiting)
   const int nt0 = ng * NT;
-  const int m0 = (slot % mblocks) * MROWS;
+  const int mblock = (slot / S) % mblocks, split = slot % S;
+  const int m0 = mblock * MROWS;
   const int G = K >> 7;
   constexpr int kRegion = MROWS * kStride;  // bf16 elements of one wave's region
   uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * kRegion;
 
-  const int per_wave = (G + kWaves - 1) / kWaves;
-  const int g_begin = wave * per_wave;
-  const int g_end = min(G, g_begin + per_wave);
+  // this workgroup's groups (all of K, or split `split` of S equal parts), a contiguous run per wave
+  const int g_count = G / S, g_first = split * g_count;
+  const int per_wave = kBatches > 0 ? TPW * kBatches : (g_count + kWaves - 1) / kWaves;
+  const int g_begin = g_first + wave * per_wave;
+  const int g_end = min(g_first + g_count, g_begin + per_wave);
 
   // row tiles past the matrix repeat the last one (their results are not stored)
   const u32x4_t* wtile[NT];
@@ -212,9 +234,12 @@ __device__ __forceinline__ void dequant_skinny_body(
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  if constexpr (kBatches > 0) {
-    // K == kWaves * TPW * kBatches * 128: every wave runs exactly kBatches full batches, the loop is straight-line
-    // code and the number of loads in flight is known at every wait (a batch is computed while the next travels)
+  if (kBatches > 0 && g_begin >= g_end) {
+    epilogue_loads();  // (more waves than runs of TPW * kBatches groups: the last waves have none)
+  } else if constexpr (kBatches > 0) {
+    // the workgroup's groups are a whole number of runs of TPW * kBatches: every wave that has any runs exactly
+    // kBatches full batches, the loop is straight-line code and the number of loads in flight is known at every
+    // wait (a batch is computed while the next travels)
     Batch b[2];
     load(b[0], g_begin);
     epilogue_loads();
@@ -258,9 +283,8 @@ __device__ __forceinline__ void dequant_skinny_body(
     if (lane < 32) red2[lane * kWaves + wave] = sh;
   }
   __syncthreads();
-  for (int u = wave; u < NT * MB; u += kWaves) {
-    const int t = u / MB, r = u % MB;
-    if (nt0 + t >= ntiles) break;
+  // the workgroup's sum of unit u: the waves' partial sums in wave order
+  auto unit_sum = [&](int u) -> f32x4_t {
     f32x4_t part[kWaves];
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
@@ -268,6 +292,51 @@ __device__ __forceinline__ void dequant_skinny_body(
     f32x4_t sum = part[0];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w) sum += part[w];
+    return sum;
+  };
+  f32x4_t* shared_partial = nullptr;  // split-K: [S][NT * MB][64] of this (row-tile group, row block)
+  if constexpr (kSplitK) {
+    __shared__ unsigned drawn;
+    const int cell = ng * mblocks + mblock;
+    shared_partial = reinterpret_cast<f32x4_t*>(sp.partial) + (size_t)cell * S * (NT * MB * 64);
+    // The partial sums travel as device-scope atomic stores and loads (written through and read past the L2 of
+    // the XCD, which is not coherent with the other seven): a device-scope release / acquire fence around plain
+    // accesses writes back and invalidates the whole L2 each time, measured at 55 us for 256 workgroups.  A wave's
+    // stores have completed when it arrives at the barrier (workgroup-scope release), the ticket is drawn after it.
+    unsigned long long* cell_partial = reinterpret_cast<unsigned long long*>(shared_partial);
+    for (int u = wave; u < NT * MB; u += kWaves) {
+      const f32x4_t v = unit_sum(u);
+      unsigned long long* dst = cell_partial + (((size_t)split * NT * MB + u) * 64 + lane) * 2;
+      __hip_atomic_store(dst, (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 1, (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) drawn = __hip_atomic_fetch_add(sp.tickets + cell, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (drawn != (unsigned)(S - 1)) return;
+    if (threadIdx.x == 0) __hip_atomic_store(sp.tickets + cell, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (int u = wave; u < NT * MB; u += kWaves) {
+    const int t = u / MB, r = u % MB;
+    if (nt0 + t >= ntiles) break;
+    f32x4_t sum;
+    if constexpr (kSplitK) {
+      const unsigned long long* src = reinterpret_cast<const unsigned long long*>(shared_partial) + ((size_t)u * 64 + lane) * 2;
+      auto fetch = [&](int q) -> f32x4_t {
+        const unsigned long long* at = src + (size_t)q * NT * MB * 128;
+        const unsigned long long lo = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi = __hip_atomic_load(at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return f32x4_t{__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
+                       __uint_as_float((uint32_t)(hi >> 32))};
+      };
+      sum = fetch(0);
+      for (int q = 1; q < S; ++q) sum += fetch(q);
+    } else {
+      sum = unit_sum(u);
+    }
     const int n = (nt0 + t) * kTileN + nl;
     float cs = 1.0f;
     if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
@@ -334,6 +403,22 @@ __global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skin
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
   dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, kEpi, kBatches>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
+}
+
+// the split-K forms (see kSplitK above)
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kBatches = 0>
+__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_split_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, SkinnySplit sp) {
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, 0, kBatches, true>(wq, meta, x, K, M, N, y, out_f32, scales8,
+                                                                       GemvEpilogue{}, sp);
+}
+
+template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0>
+__global__ __launch_bounds__(kWaves * 64, kWaves <= 4 ? 2 : 1) void dequant_skinny_split_epi_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep, SkinnySplit sp) {
+  dequant_skinny_body<kWaves, TPW, MROWS, NT, kW4, kEpi, kBatches, true>(wq, meta, x, K, M, N, y, out_f32, scales8, ep, sp);
 }
 
 // LDS bytes of one workgroup of dequant_skinny_kernel<kWaves, TPW, MROWS, *>

@@ -474,6 +474,8 @@ class FusedDecoder(GraphDecoder):
         lib = _lib.load()
         self.attn_ws_bytes = int(lib.ajq_attn_step_workspace_bytes(batch, self.heads))
         self.attn_ws = torch.zeros(max(self.attn_ws_bytes, 16), dtype=torch.uint8, device=dev)
+        # lent to the library for the duration of each step (zeroed: its first 4 KiB are ticket words)
+        self.matmul_ws = torch.zeros(int(lib.ajq_matmul_workspace_bytes()), dtype=torch.uint8, device=dev)
 
     @torch.no_grad()
     def prefill(self, prompt: torch.Tensor, rows_per_pass: int | None = None, fused: bool = False) -> None:
@@ -585,8 +587,16 @@ class FusedDecoder(GraphDecoder):
     def _logits(self) -> torch.Tensor:
         """Logits ``[B, V]`` of the token whose embedding row is in ``self.embedded`` (``prefill`` and
         every step leave it there), at cache row ``cache.position``; the decoding state is untouched."""
-        if self.fuse_epilogue:
-            return self._logits_epilogue()
+        lib = _lib.load()
+        # the step's matmuls may exchange split-K partial sums through this decoder's buffer (batched steps: w2)
+        _lib.check(lib.ajq_matmul_workspace_set(self.matmul_ws.data_ptr(), self.matmul_ws.numel()), "matmul_workspace_set")
+        try:
+            return self._logits_epilogue() if self.fuse_epilogue else self._logits_prologue()
+        finally:
+            lib.ajq_matmul_workspace_set(None, 0)
+
+    def _logits_prologue(self) -> torch.Tensor:
+        """``_logits`` with the norms and the gate in front of the GEMVs (small batches) or as launches of their own."""
         lib, st = _lib.load(), _stream()
         b, d = self.batch, self.model.d_model
         pos = self.cache.position

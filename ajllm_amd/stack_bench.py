@@ -139,15 +139,21 @@ def bench_stack(device, log=print, config: dict | None = None, batch: int = BATC
           .to(torch.bfloat16) for name, w in (("qkv", dec.layers[0]["qkv"]), ("o", dec.layers[0]["o"]),
                                               ("w13", dec.layers[0]["w13"]), ("w2", dec.layers[0]["w2"]))}
 
-    def linears():
-        for w in dec.layers:
-            for name in ("qkv", "o", "w13", "w2"):
-                w[name](xs[name])
-        dec.head(xs["qkv"])
-
-    t_linear = _graph_seconds(linears, stream)
     from . import _lib
     lib = _lib.load()
+
+    def linears():
+        # (with the decoder's buffer for split-K partial sums lent, as during its steps)
+        _lib.check(lib.ajq_matmul_workspace_set(dec.matmul_ws.data_ptr(), dec.matmul_ws.numel()), "matmul_workspace_set")
+        try:
+            for w in dec.layers:
+                for name in ("qkv", "o", "w13", "w2"):
+                    w[name](xs[name])
+            dec.head(xs["qkv"])
+        finally:
+            lib.ajq_matmul_workspace_set(None, 0)
+
+    t_linear = _graph_seconds(linears, stream)
 
     qkv = torch.randn((batch, (dec.heads + 2 * dec.kv_heads) * 128), device=device)
 

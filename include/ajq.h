@@ -221,6 +221,22 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
+/* A device buffer lent to the matmul entry points called from THIS host thread (all of ajq_w*a16_gemm, _gemv_residual,
+ * _gemv_gated, _gemv_rowscale, _gemv_norm_sums), for the split-K form of the weight-streaming kernel: at 17 <= M <= 32
+ * with K >= 8192 and N <= 4096 (the down projection of a SwiGLU feed-forward in a batched decode step) four workgroups
+ * share four row tiles and a quarter of K each, exchange their partial sums through this buffer and the last one to
+ * arrive adds them in a fixed order (results are run-to-run identical; they differ from the unsplit kernel's in the
+ * last bits, the sum being associated differently).  No counterpart in the reference.
+ *   - ajq_matmul_workspace_bytes() bytes, 16-byte aligned; its first 4096 bytes must be ZERO when it is lent (the
+ *     kernels leave them zero) and the buffer must stay allocated while launches that were given it can still run
+ *     (HIP graphs recorded while it was set included);
+ *   - launches that share one buffer must not overlap in time (one stream, or streams that are ordered): a second
+ *     stream or host thread takes a buffer of its own;
+ *   - workspace == NULL ends the loan (the state is per host thread; nothing is set initially, and without a buffer
+ *     every shape runs the kernels that need none). */
+size_t ajq_matmul_workspace_bytes(void);
+int ajq_matmul_workspace_set(void* workspace, size_t bytes);
+
 /* ajq_w4a16_gemm for callers that cannot allocate device memory or pass a workspace (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the group sums live in
  * a 16 MiB array inside the library's code object, one copy per GPU, held until the process ends

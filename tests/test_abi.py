@@ -101,6 +101,12 @@ def test_shape_alignment_and_option_errors():
     assert lib.ajq_gemv_rowscale_supported(1, 2048) == 1 and lib.ajq_gemv_rowscale_supported(32, 4096) == 1
     assert lib.ajq_gemv_rowscale_supported(8, 5632) == 1 and lib.ajq_gemv_rowscale_supported(12, 5632) == 0
     assert lib.ajq_gemv_rowscale_supported(32, 8192) == 0 and lib.ajq_gemv_rowscale_supported(200, 14336) == 0
+    # the buffer lent for split-K partial sums: size query, alignment and size checks, NULL ends the loan
+    need = lib.ajq_matmul_workspace_bytes()
+    assert need == 4096 + 64 * 4 * 4 * 2048
+    assert lib.ajq_matmul_workspace_set(odd, need) == -3
+    assert lib.ajq_matmul_workspace_set(p, need - 1) == -6 and b"bytes needed" in lib.ajq_last_error()
+    assert lib.ajq_matmul_workspace_set(None, 0) == 0
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 352, 1e-5, 12, 5632, p, p, 16, p, 0, 0, None) == -4
     assert lib.ajq_w8a16_gemv_rowscale(p, p, 512, 1e-5, 32, 8192, p, p, 16, p, 0, 0, None) == -4
     assert lib.ajq_w4a16_gemv_rowscale(p, p, 64, 1e-5, 4, 2048, p, p, 16, p, 0, 0, None) == -2     # parts is not K / 16

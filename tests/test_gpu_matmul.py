@@ -244,6 +244,88 @@ def test_batched_decode_matmul_is_deterministic(cuda, scheme):
     assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
 
 
+class _LentWorkspace:
+    """A zeroed buffer lent to the library's matmuls for the duration of a ``with`` block."""
+
+    def __init__(self, cuda):
+        from ajllm_amd import _lib
+
+        self.lib = _lib.load()
+        self.buffer = torch.zeros(int(self.lib.ajq_matmul_workspace_bytes()), dtype=torch.uint8, device=cuda)
+
+    def __enter__(self):
+        from ajllm_amd import _lib
+
+        _lib.check(self.lib.ajq_matmul_workspace_set(self.buffer.data_ptr(), self.buffer.numel()), "matmul_workspace_set")
+        return self
+
+    def __exit__(self, *exc):
+        self.lib.ajq_matmul_workspace_set(None, 0)
+
+    def tickets(self) -> torch.Tensor:
+        return self.buffer[:4096]
+
+
+@pytest.mark.parametrize("m,n,k", [(32, 4096, 14336), (17, 4096, 14336), (32, 4000, 8192), (24, 1040, 16384),
+                                   (32, 64, 8704)])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_batched_decode_matmul_split_along_k(cuda, scheme, m, n, k):
+    """The weight-streaming kernel with four workgroups per group of four row tiles, a quarter of K each, and the
+    partial sums exchanged through a lent buffer (17 <= M <= 32, K >= 8192, N <= 4096): against the oracle like
+    every other kernel; against the unsplit kernel within fp32 reassociation; identical from run to run; the
+    buffer's ticket words zero again afterwards; no trace of the previous call's partial sums when calls on
+    different matrices alternate on one buffer.  K = 14336 and 16384 take the straight-line kernels (seven and eight
+    waves' runs of four groups), 8192 and 8704 the loop; N = 4000 and 1040 end in a group of fewer than four row
+    tiles."""
+    w_hat, wq, meta = _quantized(scheme, n, k, 31, cuda)
+    x = make_activations(m, k, 131, True).to(cuda)
+    plain = _run(scheme, x, wq, meta, torch.float32, "gemm")
+    with _LentWorkspace(cuda) as ws:
+        split = _check(scheme, "gemm", m, n, k, seed=31, cuda=cuda, outliers=True)
+        again = _run(scheme, x, wq, meta, torch.float32, "gemm")
+        # another matrix through the same buffer, then the first again
+        other_wq = torch.roll(wq, 1, 0)
+        other = _run(scheme, x, other_wq, meta, torch.float32, "gemm")
+        third = _run(scheme, x, wq, meta, torch.float32, "gemm")
+        torch.cuda.synchronize()
+        assert int(ws.tickets().max()) == 0
+    assert not torch.equal(plain, split)  # (the split form did run: its sums associate differently)
+    assert errors(split.cpu(), plain.cpu().double())[0] <= 1e-4
+    assert torch.equal(split, again) and torch.equal(split, third) and not torch.equal(split, other)
+    # without the buffer the unsplit kernel runs again
+    assert torch.equal(plain, _run(scheme, x, wq, meta, torch.float32, "gemm"))
+
+
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_split_along_k_with_the_residual_epilogue(cuda, scheme):
+    """ajq_w*a16_gemv_residual (w2 of a batched decode step: K = 14336) through the split form: the new residual
+    stream is the plain split matmul's output added to h_in bit for bit, its bf16 image and the sums of squares
+    follow from it."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    m, d, k = 32, 4096, 14336
+    w_hat, wq, meta = _quantized(scheme, d, k, 31, cuda)
+    g = torch.Generator().manual_seed(5)
+    x = make_activations(m, k, 17, True).to(cuda)
+    h_in = (torch.randn((m, d), generator=g) * 3.0).to(cuda)
+    gain = (torch.rand(d, generator=g) + 0.5).to(cuda)
+    h_out = torch.zeros((m, d), dtype=torch.float32, device=cuda)
+    xt = torch.zeros((m, d), dtype=torch.bfloat16, device=cuda)
+    ssq = torch.zeros((m, d // 16), dtype=torch.float32, device=cuda)
+    res_fn = lib.ajq_w4a16_gemv_residual if scheme == "w4" else lib.ajq_w8a16_gemv_residual
+    with _LentWorkspace(cuda) as ws:
+        y = _run(scheme, x, wq, meta, torch.float32, "gemm")
+        _lib.check(res_fn(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), d, h_in.data_ptr(), gain.data_ptr(),
+                          h_out.data_ptr(), xt.data_ptr(), ssq.data_ptr(), st), "gemv_residual")
+        torch.cuda.synchronize()
+        assert int(ws.tickets().max()) == 0
+    assert torch.equal(h_out, h_in + y)
+    assert torch.equal(xt, (h_out * gain).to(torch.bfloat16))
+    tiles = h_out.double().square().reshape(m, d // 16, 16).sum(-1)
+    assert float((ssq.double() - tiles).abs().max() / tiles.max()) <= 1e-6
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemv_and_gemm_agree(cuda, scheme):
     w_hat, wq, meta = _quantized(scheme, 2048, 2048, 41, cuda)
