@@ -286,7 +286,23 @@ __global__ __launch_bounds__(kGWThreads) void dequant_gemm256w_kernel(const uint
 #pragma unroll
           for (int t = 0; t < 2; ++t) bf[t][s] = lds_read128((uint32_t)(nxt * kGWStage) + b_rel[t] + (uint32_t)(s * 1024));
         }
-        __builtin_amdgcn_sched_barrier(0x2 | 0x4);  // VALU and SALU may cross
+        if constexpr (!kW4) {
+          // int8: the order a position's instructions issue in is pinned (an MFMA, a fragment read, up to six of the
+          // converts in flight, the piece's write or a request; twice): left alone the compiler bunches a piece's
+          // converts and then issues MFMAs back to back.  +2-5 % in a same-process comparison; the int4 form, whose
+          // unpack is three times as long, measures 1-4 % slower with it and keeps the free order.
+#pragma unroll
+          for (int g = 0; g < 2; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // one MFMA
+            if (g == 0 || p >= 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // a fragment read
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                        // converts in flight
+            if (g == 1 && (p == 1 || p == 3)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // the piece's write
+            if (g == 1 && (p == 0 || p == 2)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // a request
+          }
+          if (p == 3 || p == 7) __builtin_amdgcn_sched_barrier(0);
+        } else {
+          __builtin_amdgcn_sched_barrier(0x2 | 0x4);  // VALU and SALU may cross
+        }
       }
     }
   };
