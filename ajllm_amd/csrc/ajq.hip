@@ -475,6 +475,10 @@ int launch_skinny_split(const uint16_t* x, int M, int K, const uint32_t* wq, con
   return launch_skinny_split_kernel<kW4, kEpi, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
 }
 
+// from this many workgroups of four row tiles on, the kernel runs as four-wave workgroups, two to a CU
+#ifndef AJQ_SKINNY_FOUR_WAVE_MIN
+#define AJQ_SKINNY_FOUR_WAVE_MIN 512
+#endif
 #ifndef AJQ_SKINNY_FORCE_NT
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
@@ -494,7 +498,7 @@ int skinny_row_tiles(int M, int N) {
   long long best = 0;
   for (int c = 1; c <= 4; c *= 2) {
     const long long wgs = (long long)((ntiles + c - 1) / c) * mblocks;
-    const int slots = (c == 4 && (ntiles / 4) * mblocks >= 512) ? 512 : 256;  // four-wave workgroups share a CU
+    const int slots = (c == 4 && (ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN) ? 512 : 256;  // four-wave workgroups share a CU
     const long long cost = ((wgs + slots - 1) / slots) * (64 + (kW4 ? 8 : 16) * c);
     if (c == 1 || cost < best) {
       best = cost;
@@ -513,7 +517,7 @@ int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const
   const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
   if (nt == 1) return launch_skinny_epi_cfg<8, 2, 32, 1, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   if (nt == 2) return launch_skinny_epi_cfg<8, 1, 32, 2, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
-  if ((ntiles / 4) * mblocks >= 512)
+  if ((ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN)
     return launch_skinny_epi_cfg<4, 1, 32, 4, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   return launch_skinny_epi_cfg<8, 1, 32, 4, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
 }
@@ -529,7 +533,7 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
   long long best = 0;
   for (int c = 1; c <= 4; c *= 2) {
     const long long wgs = (long long)((ntiles + c - 1) / c) * mblocks;
-    const int slots = (c == 4 && (ntiles / 4) * mblocks >= 512) ? 512 : 256;  // four-wave workgroups share a CU
+    const int slots = (c == 4 && (ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN) ? 512 : 256;  // four-wave workgroups share a CU
     const long long cost = ((wgs + slots - 1) / slots) * (64 + (kW4 ? 8 : 16) * c);
     if (c == 1 || cost < best) {
       best = cost;
@@ -541,7 +545,7 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
   if (nt == 2) return launch_skinny_cfg<8, 1, 32, 2, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   // two workgroups of four waves per CU once there are that many: one's start-up and
   // reduction overlap the other's arithmetic (12-15 % faster than one of eight waves)
-  if ((ntiles / 4) * mblocks >= 512)
+  if ((ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN)
     return launch_skinny_cfg<4, 1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
   return launch_skinny_cfg<8, 1, 32, 4, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
