@@ -108,6 +108,19 @@ def test_gemv_wide_matrix_with_ragged_last_workgroup(cuda, scheme, m):
         assert torch.equal(_run(scheme, x, wq, meta, torch.float32, "gemv"), first)
 
 
+@pytest.mark.parametrize("m", [8, 13, 16])
+@pytest.mark.parametrize("n", [6144, 16 * 2001])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_gemv_wide_matrix_at_k_2048(cuda, scheme, m, n):
+    """More row tiles than CUs at K = 2048 (q|k|v and the head of the 12-layer model at batch 8 and up; N = 32016 is no
+    multiple of the CU count), 8 to 16 rows."""
+    _check(scheme, "gemv", m, n, 2048, seed=17, cuda=cuda)
+    w_hat, wq, meta = _quantized(scheme, n, 2048, 17, cuda)
+    x = make_activations(m, 2048, 8).to(cuda)
+    first = _run(scheme, x, wq, meta, torch.float32, "gemv")
+    assert torch.equal(_run(scheme, x, wq, meta, torch.float32, "gemv"), first)
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemv_is_deterministic(cuda, scheme):
     w_hat, wq, meta = _quantized(scheme, 4096, 4096, 11 if scheme == "w4" else 12, cuda)
