@@ -70,6 +70,11 @@ SIGNATURES: dict[str, tuple] = {
         [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
          c_void_p, c_void_p],
     ),
+    "ajq_sample_pick": (
+        c_int,
+        [c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+         c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "ajq_gemv_merge_max_splits": (c_int, [c_int, c_int]),
     "ajq_w4a16_gemv_merge": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),
     "ajq_w8a16_gemv_merge": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p]),

@@ -1,5 +1,6 @@
 // C ABI of libajq.so: argument validation, launch geometry, error reporting.
 #include <stdarg.h>
+#include <cmath>
 #include <atomic>
 #include <stdio.h>
 
@@ -1377,6 +1378,32 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
                      reinterpret_cast<long long*>(token), reinterpret_cast<long long*>(out), out_ld,
                      reinterpret_cast<const long long*>(step), reinterpret_cast<long long*>(advance), ticket);
   return check_launch("ajq_greedy_pick");
+}
+
+int ajq_sample_pick(const float* logits, int B, int V, int ld, float temperature, float top_p, const float* uniforms,
+                    int uniform_rows, const float* embedding, int D, float* hidden, int64_t* token, int64_t* out,
+                    int out_ld, const int64_t* step, int64_t* advance, uint32_t* ticket, int32_t* kept, void* stream) {
+  if (!logits || !token || !out || !step) return fail(AJQ_ERR_NULL, "ajq_sample_pick: null pointer argument");
+  if ((embedding != nullptr) != (hidden != nullptr))
+    return fail(AJQ_ERR_NULL, "ajq_sample_pick: embedding and hidden go together (both or neither)");
+  if ((advance != nullptr) != (ticket != nullptr))
+    return fail(AJQ_ERR_NULL, "ajq_sample_pick: advance and ticket go together (both or neither)");
+  if (B < 1 || V < 1 || ld < V || ld % 4 != 0 || out_ld < 1 || (embedding && (D < 4 || D % 4 != 0)))
+    return fail(AJQ_ERR_SHAPE, "ajq_sample_pick: unsupported shape (B=%d V=%d ld=%d D=%d out_ld=%d)", B, V, ld, D, out_ld);
+  if (!aligned16(logits)) return fail(AJQ_ERR_ALIGN, "ajq_sample_pick: logits must be 16-byte aligned");
+  if (V > kSampleMaxBlocks * 1024)
+    return fail(AJQ_ERR_UNSUPPORTED, "ajq_sample_pick: V=%d exceeds %d", V, kSampleMaxBlocks * 1024);
+  if (!(temperature > 0.f) || !std::isfinite(temperature))
+    return fail(AJQ_ERR_SHAPE, "ajq_sample_pick: temperature must be positive and finite (use ajq_greedy_pick for argmax)");
+  if (!(top_p > 0.f)) return fail(AJQ_ERR_SHAPE, "ajq_sample_pick: top_p must be in (0, 1] (1: no filter)");
+  if (!uniforms || uniform_rows < 1) return fail(AJQ_ERR_NULL, "ajq_sample_pick: uniforms [uniform_rows, B] are needed");
+  if (embedding && (!aligned16(embedding) || !aligned16(hidden)))
+    return fail(AJQ_ERR_ALIGN, "ajq_sample_pick: embedding and hidden must be 16-byte aligned");
+  hipLaunchKernelGGL(sample_pick_kernel, dim3(B), dim3(1024), 0, (hipStream_t)stream, logits, V, ld, 1.0f / temperature,
+                     top_p, uniforms, uniform_rows, embedding, D, hidden, reinterpret_cast<long long*>(token),
+                     reinterpret_cast<long long*>(out), out_ld, reinterpret_cast<const long long*>(step),
+                     reinterpret_cast<long long*>(advance), ticket, kept);
+  return check_launch("ajq_sample_pick");
 }
 
 int ajq_attn_prefill(const float* q, const void* kcache, const void* vcache, int cache_dtype, int B, int H, int Hkv,

@@ -600,6 +600,272 @@ __global__ __launch_bounds__(1024) void greedy_pick_kernel(const float* __restri
   for (int i = t; i < D / 4; i += 1024) h4[i] = e4[i];
 }
 
+// Temperature / nucleus sampling at the end of a decode step (sample_next_token,
+// src/ajllm/generation/sampling.py:8-22), one workgroup of 1024 threads per sequence; the tail (token, output column,
+// embedding row, the step's counters) is greedy_pick_kernel's.
+//   p = softmax(logits / temperature); with top_p < 1 the tokens are kept whose probability mass STRICTLY above them
+//   (in descending order) is below top_p -- the reference's `cumulative - sorted_probabilities >= top_p` removed --
+//   and the choice is drawn from the kept tokens in proportion to p.
+// The draw is the inverse CDF over the kept tokens IN INDEX ORDER at u = uniforms[min(*step, uniform_rows - 1), b]
+// (the reference draws with torch.multinomial from the sorted tokens: the same distribution from other random bits).
+// Probabilities are compared and added as 40-bit fixed-point integers, so no result depends on the order of a sum:
+// the same logits and the same u give the same token on every run.
+//   1. row maximum; 2. Z = sum exp((l - max) / T) (a fixed order); weight w = exp(..) * 2^40 / Z as an integer;
+//   3. top_p < 1: the float bits of exp(..) order the tokens; four radix passes (8 bits each, 256 bins of summed
+//      weight) find the key where the weight above it is below top_p * 2^40 and the weight from it on is not: the
+//      last kept token's key (equal keys are kept together);
+//   4. the kept weight of every block of 1024 consecutive tokens (a wave per block), a serial walk to the block the
+//      draw falls in, then the waves of that block and the lanes of that wave.
+// kept (optional, [B]): the number of kept tokens, for tests.  Every walk over bins, blocks and tokens is a workgroup
+// prefix sum: no thread loops over LDS words behind a branch.
+constexpr int kSampleMaxBlocks = 1024;  // V <= 1024 * 1024
+// exp for x <= 0 on the hardware's exp2 (a row is walked up to seven times by ONE workgroup, so the exponential's
+// instruction count is the kernel's time: the library routine's thirty-odd instructions made a pass over 32000
+// columns 6 us); the same value on every pass, which is all the radix passes need
+__device__ __forceinline__ float sample_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896341f); }
+__device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, int off) {
+  const unsigned lo = __shfl_up((unsigned)v, off), hi = __shfl_up((unsigned)(v >> 32), off);
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned lo = __shfl_xor((unsigned)v, off), hi = __shfl_xor((unsigned)(v >> 32), off);
+    v += ((unsigned long long)hi << 32) | lo;
+  }
+  return v;
+}
+// inclusive prefix sum of one value per thread over a workgroup of 16 waves, in thread order (two barriers; the
+// serial walks this replaces, one thread reading LDS word after word behind a branch, were most of the kernel's time)
+__device__ __forceinline__ unsigned long long block_prefix_u64(unsigned long long v, unsigned long long* wave_total,
+                                                              int lane, int wave) {
+  unsigned long long incl = v;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const unsigned long long up = shfl_up_u64(incl, off);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  unsigned long long base = 0ull;
+#pragma unroll
+  for (int w = 0; w < 15; ++w) base += w < wave ? wave_total[w] : 0ull;
+  __syncthreads();
+  return incl + base;
+}
+__global__ __launch_bounds__(1024) void sample_pick_kernel(const float* __restrict__ logits, int V, int ld,
+                                                           float inv_temperature, float top_p,
+                                                           const float* __restrict__ uniforms, int uniform_rows,
+                                                           const float* __restrict__ embedding, int D,
+                                                           float* __restrict__ hidden, long long* __restrict__ token,
+                                                           long long* __restrict__ out, int out_ld, const long long* step,
+                                                           long long* advance, unsigned* ticket, int* __restrict__ kept) {
+  const int b = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const float* row = logits + (size_t)b * ld;
+  // 256 bins in sixteen copies each, one per lane & 15: the keys of a row crowd into a few bins (the exponent byte),
+  // and lanes that add to one LDS word queue behind each other
+  __shared__ float red[16];
+  __shared__ unsigned long long bins[256 * 16];
+  __shared__ unsigned long long block_weight[kSampleMaxBlocks];
+  __shared__ unsigned long long wave_total[16];
+  __shared__ unsigned long long sh_above, sh_rest, sh_total;
+  __shared__ unsigned sh_byte;
+  __shared__ int sh_block, sh_kept, chosen;
+  __shared__ long long sh_at;
+  __shared__ float sh_u;
+
+  if (t == 0) {
+    // `step` may alias advance[0..1]: read it once, through a volatile access (see greedy_pick_kernel)
+    const long long at = *reinterpret_cast<const volatile long long*>(step);
+    sh_at = at;
+    sh_u = uniforms[(size_t)min(max(at, 0LL), (long long)uniform_rows - 1) * gridDim.x + b];
+    sh_kept = 0;
+  }
+
+  // every element of the row once, four 128-bit loads per thread in flight (ld % 4 == 0, 16-byte aligned rows)
+  const float4* row4 = reinterpret_cast<const float4*>(row);
+  const int nvec = V >> 2;
+  auto for_each = [&](auto&& fn) {
+    for (int base = 0; base < nvec; base += 4 * 1024) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int idx = base + u * 1024 + t;
+        v[u] = idx < nvec ? row4[idx] : float4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (base + u * 1024 + t < nvec) {
+          fn(v[u].x);
+          fn(v[u].y);
+          fn(v[u].z);
+          fn(v[u].w);
+        }
+      }
+    }
+    if (4 * nvec + t < V) fn(row[4 * nvec + t]);  // the last V % 4 columns
+  };
+
+  // ---- 1. row maximum
+  float m = -INFINITY;
+  for_each([&](float l) { m = fmaxf(m, l); });
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) m = fmaxf(m, red[w]);
+  __syncthreads();
+  // ---- 2. normaliser, summed in a fixed order (a thread's elements in sequence, a fixed tree, waves in order)
+  float z = 0.f;
+  for_each([&](float l) { z += sample_exp((l - m) * inv_temperature); });
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off);
+  if (lane == 0) red[wave] = z;
+  __syncthreads();
+  z = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) z += red[w];
+  const float to_fixed = 0x1p40f / z;
+  auto weight_of = [&](float e) -> unsigned long long { return (unsigned long long)(e * to_fixed); };
+
+  // ---- 3. the key of the last kept token
+  unsigned threshold = 0u;  // keep keys >= threshold
+  if (top_p < 1.0f) {
+    const unsigned long long want = (unsigned long long)((double)top_p * 0x1p40);
+    unsigned prefix = 0u, prefix_mask = 0u;
+    unsigned long long above = 0ull;  // weight of the keys whose leading bytes are above the prefix
+    unsigned long long* my_bins = bins + (lane & 15);
+    for (int pass = 0; pass < 4; ++pass) {
+      const int shift = 24 - 8 * pass;
+      for (int i = t; i < 256 * 16; i += 1024) bins[i] = 0ull;
+      __syncthreads();
+      for_each([&](float l) {
+        const float e = sample_exp((l - m) * inv_temperature);
+        const unsigned key = __float_as_uint(e);
+        if ((key & prefix_mask) == prefix) atomicAdd(&my_bins[((key >> shift) & 255u) << 4], weight_of(e));
+      });
+      __syncthreads();
+      // thread q' < 256 takes byte 255 - q' (descending), so a prefix sum in thread order is the weight from that
+      // byte up; the byte where it first reaches the wanted weight is the next digit of the key.  If it never does
+      // (rounding at top_p ~ 1), byte 0: everything is kept.
+      unsigned long long mine = 0ull;
+      if (t < 256) {
+#pragma unroll
+        for (int w = 0; w < 16; ++w) mine += bins[(255 - t) * 16 + w];
+      }
+      const unsigned long long from_here = above + block_prefix_u64(mine, wave_total, lane, wave);
+      if (t < 256) {
+        const unsigned long long over = from_here - mine;  // weight strictly above this byte
+        if ((over < want && from_here >= want) || (t == 255 && from_here < want)) {
+          sh_byte = (unsigned)(255 - t);
+          sh_above = over;
+        }
+      }
+      __syncthreads();
+      prefix |= sh_byte << shift;
+      prefix_mask |= 255u << shift;
+      above = sh_above;
+    }
+    threshold = prefix;
+  }
+
+  // ---- 4. kept weight per block of 1024 consecutive tokens (wave w: blocks w, w + 16, ...)
+  const int blocks = (V + 1023) >> 10;
+  int kept_here = 0;
+  for (int c = wave; c < blocks; c += 16) {
+    unsigned long long w_sum = 0ull;
+    auto take = [&](int j, float l) {
+      if (j < V) {
+        const float e = sample_exp((l - m) * inv_temperature);
+        if (__float_as_uint(e) >= threshold) {
+          w_sum += weight_of(e);
+          ++kept_here;
+        }
+      }
+    };
+    float4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = (c << 10) + (i * 64 + lane) * 4;
+      v[i] = j + 3 < 4 * nvec ? row4[j >> 2] : float4{j < V ? row[j] : 0.f, j + 1 < V ? row[j + 1] : 0.f,
+                                                        j + 2 < V ? row[j + 2] : 0.f, j + 3 < V ? row[j + 3] : 0.f};
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = (c << 10) + (i * 64 + lane) * 4;
+      take(j, v[i].x);
+      take(j + 1, v[i].y);
+      take(j + 2, v[i].z);
+      take(j + 3, v[i].w);
+    }
+    w_sum = wave_sum_u64(w_sum);
+    if (lane == 0) block_weight[c] = w_sum;
+  }
+  if (kept) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) kept_here += __shfl_xor(kept_here, off);
+    if (lane == 0) atomicAdd(&sh_kept, kept_here);
+  }
+  __syncthreads();
+  // ---- the block the draw falls in: thread c < blocks holds block c's weight; the draw is an integer in [0, total)
+  {
+    const unsigned long long mine = t < blocks ? block_weight[t] : 0ull;
+    const unsigned long long upto = block_prefix_u64(mine, wave_total, lane, wave);
+    if (t == 1023) sh_total = upto;
+    if (t == 0) {
+      sh_block = blocks - 1;
+      sh_rest = 0ull;
+      if (kept) kept[b] = sh_kept;
+    }
+    __syncthreads();
+    const unsigned long long total = sh_total;  // >= 1: the maximum's weight alone is 2^40 / Z >= 2^40 / V
+    unsigned long long draw = (unsigned long long)((double)fminf(fmaxf(sh_u, 0.f), 1.f) * (double)total);
+    if (draw >= total) draw = total - 1;
+    if (t < blocks && draw >= upto - mine && draw < upto) {
+      sh_block = t;
+      sh_rest = draw - (upto - mine);
+    }
+    __syncthreads();
+  }
+  // ---- the token inside the block, the same way: thread i holds token 1024 block + i
+  {
+    const int j = (sh_block << 10) + t;
+    unsigned long long mine = 0ull;
+    if (j < V) {
+      const float e = sample_exp((row[j] - m) * inv_temperature);
+      if (__float_as_uint(e) >= threshold) mine = weight_of(e);
+    }
+    const unsigned long long upto = block_prefix_u64(mine, wave_total, lane, wave);
+    const unsigned long long rest = sh_rest;
+    if (t == 0) chosen = min(sh_block << 10, V - 1);
+    __syncthreads();
+    if (rest >= upto - mine && rest < upto) chosen = j;
+    __syncthreads();
+  }
+  if (t == 0) {
+    const int bi = min(chosen, V - 1);
+    chosen = bi;
+    token[b] = bi;
+    out[(size_t)b * out_ld + min(max(sh_at, 0LL), (long long)out_ld - 1)] = bi;
+    if (advance) {
+      __threadfence();
+      if (atomicAdd(ticket, 1u) == gridDim.x - 1) {
+        advance[0] += 1;
+        advance[1] += 1;
+        *ticket = 0u;
+      }
+    }
+  }
+  __syncthreads();
+  if (embedding) {
+    const float4* e4 = reinterpret_cast<const float4*>(embedding + (size_t)chosen * D);
+    float4* h4 = reinterpret_cast<float4*>(hidden + (size_t)b * D);
+    for (int i = t; i < D / 4; i += 1024) h4[i] = e4[i];
+  }
+}
+
 // ab [B, 2F] fp32 (gate projection, then up projection) -> out[b, f] = bf16( silu(a) * u ),
 // silu(a) = a * sigmoid(a).  F % 2 == 0; one thread per pair.
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ ab, uint16_t* __restrict__ out, int B,

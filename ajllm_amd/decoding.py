@@ -42,6 +42,50 @@ class GraphDecoder:
         self.graph_many: torch.cuda.CUDAGraph | None = None
         self.graph_many_steps = 0
         self.stream = torch.cuda.Stream(device=device)
+        # greedy unless ``set_sampling`` says otherwise
+        self.temperature = 0.0
+        self.top_p: float | None = None
+        self.uniforms: torch.Tensor | None = None
+
+    def set_sampling(self, temperature: float, top_p: float | None = None, seed: int = 0) -> None:
+        """Choose tokens as the reference's ``sample_next_token`` does (src/ajllm/generation/sampling.py:8-22):
+        ``temperature <= 0`` is the greedy choice (the default), otherwise a draw from
+        ``softmax(logits / temperature)``, restricted by ``top_p`` to the most probable tokens whose mass reaches it.
+        Call it before ``prefill``; graphs recorded so far are dropped.  The random numbers are ``max_len x batch``
+        uniforms made once from ``seed`` on the device (one row per output column), so a recorded step replays with
+        fresh ones and equal seeds give equal tokens; the draw itself is the library's ``ajq_sample_pick``."""
+        if top_p is not None and not 0 < top_p <= 1:
+            raise ValueError("top_p must be in (0, 1]")
+        self.temperature, self.top_p = float(temperature), top_p
+        self.uniforms = None
+        if self.temperature > 0:
+            generator = torch.Generator(device=self.device).manual_seed(int(seed))
+            self.uniforms = torch.rand((self.max_len, self.batch), generator=generator, device=self.device)
+        self.graph = self.graph_many = None
+        self.graph_many_steps = 0
+
+    def _sample(self, logits: torch.Tensor, embedding: torch.Tensor | None = None, hidden: torch.Tensor | None = None,
+                counters: torch.Tensor | None = None, ticket: torch.Tensor | None = None, vocab: int | None = None) -> None:
+        """A draw per row of fp32 ``logits`` (row stride = its width; the first ``vocab`` columns count) into
+        ``self.token`` and ``self.out[:, step_index]``; with ``embedding`` the chosen rows go to ``hidden``, with
+        ``counters`` the step's two counters advance."""
+        _lib.check(_lib.load().ajq_sample_pick(
+            logits.data_ptr(), self.batch, vocab or logits.shape[1], logits.shape[1], self.temperature,
+            1.0 if self.top_p is None else float(self.top_p), self.uniforms.data_ptr(), self.uniforms.shape[0],
+            embedding.data_ptr() if embedding is not None else None, embedding.shape[1] if embedding is not None else 0,
+            hidden.data_ptr() if hidden is not None else None, self.token.data_ptr(), self.out.data_ptr(),
+            self.out.shape[1], self.step_index.data_ptr(), counters.data_ptr() if counters is not None else None,
+            ticket.data_ptr() if ticket is not None else None, None, _stream()), "sample_pick")
+
+    def _choose(self, logits: torch.Tensor) -> None:
+        """The next token of every row from ``logits`` ``[B, V]`` into ``self.token`` and ``self.out[:, step_index]``
+        (greedy: the first maximum; otherwise ``_sample``)."""
+        if self.temperature > 0:
+            self._sample(logits.float().contiguous())
+            return
+        nxt = torch.argmax(logits, dim=-1, keepdim=True)
+        self.out.index_copy_(1, self.step_index, nxt)
+        self.token.copy_(nxt)
 
     def _logits(self) -> torch.Tensor:
         """Logits ``[B, V]`` of the token in ``self.token`` at cache row ``cache.position``."""
@@ -49,10 +93,7 @@ class GraphDecoder:
 
     @torch.no_grad()
     def _step(self) -> None:
-        logits = self._logits()
-        nxt = torch.argmax(logits, dim=-1, keepdim=True)
-        self.out.index_copy_(1, self.step_index, nxt)
-        self.token.copy_(nxt)
+        self._choose(self._logits())
         self.cache.position.add_(1)
         self.step_index.add_(1)
 
@@ -74,9 +115,7 @@ class GraphDecoder:
         self.cache.static = True
         self.cache.position.fill_(prompt.shape[1])
         self.step_index.zero_()
-        nxt = torch.argmax(logits, dim=-1, keepdim=True)
-        self.out.index_copy_(1, self.step_index, nxt)
-        self.token.copy_(nxt)
+        self._choose(logits)
         self.step_index.add_(1)
         self.produced = 1
         self.prompt_len = prompt.shape[1]
@@ -494,9 +533,7 @@ class FusedDecoder(GraphDecoder):
             self.cache.static = True
             self.cache.position.fill_(prompt.shape[1])
             self.step_index.zero_()
-            nxt = torch.argmax(logits, dim=-1, keepdim=True)
-            self.out.index_copy_(1, self.step_index, nxt)
-            self.token.copy_(nxt)
+            self._choose(logits)
             self.step_index.add_(1)
             self.produced = 1
             self.prompt_len = prompt.shape[1]
@@ -552,6 +589,9 @@ class FusedDecoder(GraphDecoder):
         input) and the two counters in one launch."""
         self._logits()
         full = self.logits_full
+        if self.temperature > 0:
+            self._sample(full, self.embedding, self.embedded, self.counters, self.ticket, self.vocab)
+            return
         _lib.check(_lib.load().ajq_greedy_pick(full.data_ptr(), self.batch, self.vocab, full.shape[1],
                                                self.embedding.data_ptr(), self.model.d_model, self.embedded.data_ptr(),
                                                self.token.data_ptr(), self.out.data_ptr(), self.out.shape[1],

@@ -334,6 +334,21 @@ int ajq_greedy_pick(const float* logits, int B, int V, int ld, const float* embe
                     int64_t* token, int64_t* out, int out_ld, const int64_t* step, int64_t* advance, uint32_t* ticket,
                     void* stream);
 
+/* Temperature / nucleus sampling at the end of a decode step (sample_next_token,
+ * src/ajllm/generation/sampling.py:8-22: p = softmax(logits / temperature); with top_p < 1 the tokens whose
+ * probability mass strictly above them, in descending order, is below top_p are kept; the choice is drawn from the
+ * kept tokens in proportion to p) with ajq_greedy_pick's outputs.  temperature > 0 (the reference's
+ * temperature <= 0 is ajq_greedy_pick); top_p in (0, 1], 1 = no filter.  The draw is the inverse CDF over the kept
+ * tokens in INDEX order at u = uniforms[min(*step, uniform_rows - 1), b] (fp32 [uniform_rows, B], each in [0, 1):
+ * the caller's random numbers, so a recorded HIP graph replays with fresh ones per step); the reference draws with
+ * torch.multinomial, the same distribution from other random bits.  Probabilities are compared and added as
+ * 40-bit fixed-point integers: equal inputs give equal tokens.  embedding / hidden may both be NULL (no embedding row
+ * is fetched); kept (optional, int32 [B]) receives the number of tokens the filter kept.  V <= 1048576; ld % 4 == 0
+ * and logits 16-byte aligned. */
+int ajq_sample_pick(const float* logits, int B, int V, int ld, float temperature, float top_p, const float* uniforms,
+                    int uniform_rows, const float* embedding, int D, float* hidden, int64_t* token, int64_t* out,
+                    int out_ld, const int64_t* step, int64_t* advance, uint32_t* ticket, int32_t* kept, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
