@@ -129,8 +129,8 @@ __global__ __launch_bounds__(kGRThreads) void dequant_gemm256r_w8_kernel(const u
     a_lo[s] = (uint32_t)((wm * 128 + col) * 128 + (((2 * s + kh) ^ ((col >> 1) & 7)) << 4));
     a_hi[s] = a_lo[s] + 2u * kGRABytes;
   }
-  auto a_frag = [&](int stage, int p) -> u32x4_t {  // position p = 4 i + s of the sub-block in `stage`
-    const int i = p >> 2, s = p & 3;
+  auto a_frag = [&](int stage, int p) -> u32x4_t {  // position p = 4 s + i of the sub-block in `stage`
+    const int i = p & 3, s = p >> 2;
     return lds_read128((stage < 2 ? a_lo[s] : a_hi[s]) + (uint32_t)((stage & 1) * kGRABytes + i * 32 * 128));
   };
   // weights: lane (col, kh) of 32-column block t reads, from the private tile that holds its column,
@@ -175,25 +175,33 @@ __global__ __launch_bounds__(kGRThreads) void dequant_gemm256r_w8_kernel(const u
       u32x4_t bf_next[2];
 #pragma unroll
       for (int p = 0; p < kPos; ++p) {
-        const int i = p >> 2, s = p & 3;
+        // k-step-major order (position p = 4 s + i): the B fragments of k-step s + 1 are first used four positions
+        // on, so their unpacking spreads over two positions, one column block each, and the order the instructions of
+        // a position issue in is pinned (an MFMA, a fragment read, up to six converts, an MFMA, up to six converts).
+        // A compute wave has its SIMD to itself: converts bunched between two MFMAs (the row-block-major order unpacked
+        // both column blocks of a k-step in one position) stall the matrix pipe for their whole issue time.
+        // Same results bit for bit; +2-3.5 % over the row-block-major order in a same-process comparison (M = 2048,
+        // N = K = 4096: 1067 -> 1102 TFLOP/s); three, nine or twelve converts per group measure no better than none.
+        const int i = p & 3, s = p >> 2;
         if (p == kPos - kAhead) {
           // the next sub-block has landed (the loader waited for it), and every wave is done with
           // the sub-block before this one
+          __builtin_amdgcn_sched_barrier(0);
           __syncthreads();
           raw_next = read_raw((st + 1) & 3);
         }
         afr[(p + kAhead) & 7] = p + kAhead < kPos ? a_frag(st, p + kAhead) : a_frag((st + 1) & 3, p + kAhead - kPos);
-        if (i == 0 && s + 1 < 4) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t) bf[t][s + 1] = unpack(raw, t, s + 1);
-        }
-        if (p == kPos - 2) {
-#pragma unroll
-          for (int t = 0; t < 2; ++t) bf_next[t] = unpack(raw_next, t, 0);
-        }
+        if (i < 2 && s + 1 < 4) bf[i][s + 1] = unpack(raw, i, s + 1);
+        if (p >= kPos - 2) bf_next[p - (kPos - 2)] = unpack(raw_next, p - (kPos - 2), 0);  // the next sub-block's first ones
 #pragma unroll
         for (int t = 0; t < 2; ++t) acc[i][t] = mfma32(afr[p & 7], bf[t][s], acc[i][t]);
-        __builtin_amdgcn_sched_barrier(0x2 | 0x4);  // VALU and SALU may cross
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (g == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+        }
+        if (i == 3) __builtin_amdgcn_sched_barrier(0);
       }
       raw = raw_next;
 #pragma unroll
