@@ -1,6 +1,7 @@
 // C ABI of libajq.so: argument validation, launch geometry, error reporting.
 #include <stdarg.h>
 #include <cmath>
+#include <algorithm>
 #include <atomic>
 #include <stdio.h>
 
@@ -15,6 +16,7 @@
 #include "gemm_wide_kernels.h"
 #include "gemm128_kernels.h"
 #include "skinny_kernels.h"
+#include "skinny_resident_kernels.h"
 #include "decode_kernels.h"
 #include "prefill_attention.h"
 
@@ -487,6 +489,76 @@ int launch_skinny_split(const uint16_t* x, int M, int K, const uint32_t* wq, con
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
 
+// ---- resident-activation form of the weight-streaming kernel (skinny_resident_kernels.h): K = 2048 or 4096, a
+// run of T = 4, 7 or 8 row tiles per workgroup.  Both forms are priced in bytes a CU pulls over its rounds of
+// workgroups: rounds x workgroups per CU x (64 bytes of activations + 16 b T of weights) per unit of K; the
+// resident form is taken where it is cheaper (N = 28672 at 32 rows: 7 tiles x 256 workgroups, 31 -> 24 us for
+// int8; a 128256-row head: 8 tiles; N = 14336: 4 tiles; N <= 8192 stays with the other form).
+#ifndef AJQ_SKINNY_RESIDENT
+#define AJQ_SKINNY_RESIDENT 1
+#endif
+template <bool kW4>
+long long skinny_cost(int ntiles, int mblocks, int tiles_per_wg, int slots) {
+  const long long wgs = (long long)((ntiles + tiles_per_wg - 1) / tiles_per_wg) * mblocks;
+  return ((wgs + slots - 1) / slots) * (slots / 256) * (64 + (kW4 ? 8 : 16) * tiles_per_wg);
+}
+// row tiles per workgroup of the resident form for (M, N, K), or 0 where the other form is taken
+template <bool kW4>
+int skinny_resident_tiles(int M, int N, int K) {
+  if (!AJQ_SKINNY_RESIDENT || (K != 2048 && K != 4096)) return 0;
+  const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
+  long long other = skinny_cost<kW4>(ntiles, mblocks, 1, 256);
+  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 2, 256));
+  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 4, (ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN ? 512 : 256));
+  int best = 0;
+  long long cost = other;
+  for (int t : {4, 7, 8}) {
+    const long long c = skinny_cost<kW4>(ntiles, mblocks, t, 256);
+    if (c <= cost) {  // (ties go to the resident form and to the longer run: the better pattern for HBM)
+      cost = c;
+      best = t;
+    }
+  }
+  return best;
+}
+
+template <int TPW, int T, bool kW4, int kEpi>
+int launch_skinny_resident_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                               const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep,
+                               hipStream_t stream) {
+  const int ntiles = N / kTileN;
+  const int nruns = (ntiles + T - 1) / T, mblocks = (M + 31) / 32;
+  const dim3 grid(8 * ((nruns + 7) / 8) * mblocks), block(kResWaves * 64);
+  if constexpr (kEpi != 0) {
+    auto kernel = dequant_skinny_resident_epi_kernel<TPW, T, kW4, kEpi>;
+    if (int s = allow_big_lds(kernel, kResEpiLdsBytes)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, kResEpiLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+                       out_f32, scales8, ep);
+  } else {
+    auto kernel = dequant_skinny_resident_kernel<TPW, T, kW4>;
+    if (int s = allow_big_lds(kernel, kResLdsBytes)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, kResLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+                       out_f32, scales8);
+  }
+  return AJQ_OK;
+}
+
+template <bool kW4, int kEpi>
+int launch_skinny_resident(int T, const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                           const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+#define AJQ_RES(P, TT) \
+  if (K == 1024 * P && T == TT) \
+    return launch_skinny_resident_cfg<P, TT, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
+  AJQ_RES(4, 4);
+  AJQ_RES(4, 7);
+  AJQ_RES(4, 8);
+  AJQ_RES(2, 4);
+  AJQ_RES(2, 7);
+  AJQ_RES(2, 8);
+#undef AJQ_RES
+  return fail(AJQ_ERR_UNSUPPORTED, "no resident-activation configuration for K = %d, %d row tiles", K, T);
+}
+
 // M >= 17.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup.  A workgroup
 // moves K * (2 * 32 + bytes per weight * 16 * tiles) bytes (the activations come from L2 once per
 // workgroup, so more row tiles mean less traffic per output) and the CUs take the workgroups in
@@ -517,6 +589,8 @@ template <bool kW4, int kEpi>
 int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                       int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
   if (skinny_split_applies(M, N, K)) return launch_skinny_split<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if (const int T = skinny_resident_tiles<kW4>(M, N, K))
+    return launch_skinny_resident<kW4, kEpi>(T, x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   const int nt = skinny_row_tiles<kW4>(M, N);
   const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
   if (nt == 1) return launch_skinny_epi_cfg<8, 2, 32, 1, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
@@ -531,6 +605,8 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   if (skinny_split_applies(M, N, K))
     return launch_skinny_split<kW4, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
+  if (const int T = skinny_resident_tiles<kW4>(M, N, K))
+    return launch_skinny_resident<kW4, 0>(T, x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
   const int ntiles = N / kTileN;
   const int mblocks = (M + 31) / 32;
   int nt = 1;

@@ -51,6 +51,58 @@ struct SkinnySplit {
   int S;
 };
 
+// What becomes of one finished unit of a 32-row block that starts at row m0: row tile `tile` of N, 16-row block r;
+// lane (nl, kc) holds rows 4 kc + i of the block in component i, column nl of the tile.  Channel scale (int8),
+// the rows' norm factors, then the plain store, the residual form or the SwiGLU gate on interleaved rows.
+template <bool kW4, int kEpi>
+__device__ __forceinline__ void skinny_finish_unit(const f32x4_t& sum, int tile, int r, const float (&rstd)[4], int m0, int M,
+                                                   int N, int lane, void* __restrict__ y, int out_f32,
+                                                   const uint16_t* __restrict__ scales8, const GemvEpilogue& ep) {
+  const int nl = lane & 15, kc = lane >> 4;
+  const int ntiles = N / kTileN;
+  const int n = tile * kTileN + nl;
+  float cs = 1.0f;
+  if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
+  if (kEpi & kEpiResidual) {
+    const float gain_n = ep.gain[n];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * r + 4 * kc + i;
+      float v = sum[i] * cs * rstd[i];
+      asm volatile("" : "+v"(v));  // no fused multiply-add: bit for bit the plain output, then the add
+      const float h = (m < M ? ep.h_in[(size_t)m * N + n] : 0.f) + v;
+      if (m < M) {
+        ep.h_out[(size_t)m * N + n] = h;
+        if (ep.xt) ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
+      }
+      const float sq = team_sum16(m < M ? h * h : 0.f);
+      if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + tile] = sq;
+    }
+  } else if (kEpi & kEpiGate) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * r + 4 * kc + i;
+      const float v = sum[i] * cs * rstd[i];
+      const float other = row_ror<8>(v);  // the lane 8 columns away
+      if (nl < 8 && m < M)
+        reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + tile * 8 + nl] =
+            f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + 16 * r + 4 * kc + i;
+      if (m < M) {
+        const float v = sum[i] * cs * rstd[i];
+        if (out_f32)
+          reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
+        else
+          reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
+      }
+    }
+  }
+}
+
 template <int kWaves, int TPW, int MROWS, int NT, bool kW4, int kEpi, int kBatches = 0, bool kSplitK = false>
 __device__ __forceinline__ void dequant_skinny_body(
     const u32x4_t* __restrict__ wq,
@@ -337,9 +389,6 @@ __device__ __forceinline__ void dequant_skinny_body(
     } else {
       sum = unit_sum(u);
     }
-    const int n = (nt0 + t) * kTileN + nl;
-    float cs = 1.0f;
-    if (!kW4) cs = f16_bits_to_f32(scales8[n]);  // per-output-channel scale, once
     float rstd[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     if (kEpi & kEpiRowScale) {
 #pragma unroll
@@ -350,44 +399,7 @@ __device__ __forceinline__ void dequant_skinny_body(
         rstd[i] = rsqrtf(total * ep.inv_k + ep.eps);
       }
     }
-    if (kEpi & kEpiResidual) {
-      const float gain_n = ep.gain[n];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m0 + 16 * r + 4 * kc + i;
-        float v = sum[i] * cs * rstd[i];
-        asm volatile("" : "+v"(v));  // no fused multiply-add: bit for bit the plain output, then the add
-        const float h = (m < M ? ep.h_in[(size_t)m * N + n] : 0.f) + v;
-        if (m < M) {
-          ep.h_out[(size_t)m * N + n] = h;
-          if (ep.xt) ep.xt[(size_t)m * N + n] = f32_to_bf16_rne(h * gain_n);
-        }
-        const float sq = team_sum16(m < M ? h * h : 0.f);
-        if (nl == 0 && m < M) ep.ssq_out[(size_t)m * ntiles + nt0 + t] = sq;
-      }
-    } else if (kEpi & kEpiGate) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m0 + 16 * r + 4 * kc + i;
-        const float v = sum[i] * cs * rstd[i];
-        const float other = row_ror<8>(v);  // the lane 8 columns away
-        if (nl < 8 && m < M)
-          reinterpret_cast<uint16_t*>(y)[(size_t)m * (N >> 1) + (nt0 + t) * 8 + nl] =
-              f32_to_bf16_rne(v * (1.0f / (1.0f + expf(-v))) * other);
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int m = m0 + 16 * r + 4 * kc + i;
-        if (m < M) {
-          const float v = sum[i] * cs * rstd[i];
-          if (out_f32)
-            reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
-          else
-            reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
-        }
-      }
-    }
+    skinny_finish_unit<kW4, kEpi>(sum, nt0 + t, r, rstd, m0, M, N, lane, y, out_f32, scales8, ep);
   }
 }
 

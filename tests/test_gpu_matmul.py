@@ -339,6 +339,36 @@ def test_split_along_k_with_the_residual_epilogue(cuda, scheme):
     assert float((ssq.double() - tiles).abs().max() / tiles.max()) <= 1e-6
 
 
+@pytest.mark.parametrize("m,n,k", [(32, 28672, 4096), (17, 14336, 4096), (64, 16 * 1001, 4096), (33, 16 * 513, 2048),
+                                   (100, 8192, 2048), (127, 16 * 131, 4096)])
+@pytest.mark.parametrize("scheme", ["w4", "w8"])
+def test_batched_decode_matmul_many_row_tiles(cuda, scheme, m, n, k):
+    """Several 16-row tiles of N per CU at K = 2048 / 4096: the weight-streaming form that keeps a workgroup's
+    activation block resident in registers and walks a run of 4, 7 or 8 row tiles past it (w1 | w3 of config 5 at
+    32 rows, a run count that does not divide the tiles, several row blocks, the last one ragged).  The plain
+    product against the oracle, then ajq_w*a16_gemv_gated on the same operands: bf16(silu(a) * u) over tiles of
+    8 gate rows and 8 up rows, from the same fp32 values."""
+    from ajllm_amd import _lib
+    lib = _lib.load()
+    y32 = _check(scheme, "gemm", m, n, k, seed=47, cuda=cuda, outliers=True, max_rows=48)
+    _, wq, meta = _quantized(scheme, n, k, 47, cuda)
+    x = make_activations(m, k, 147, True).to(cuda)
+    gated = torch.full((m, n // 2), 7.0, dtype=torch.bfloat16, device=cuda)
+    fn = lib.ajq_w4a16_gemv_gated if scheme == "w4" else lib.ajq_w8a16_gemv_gated
+    _lib.check(fn(x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, gated.data_ptr(),
+                  torch.cuda.current_stream().cuda_stream), "gemv_gated")
+    again = torch.empty_like(y32)
+    fn32 = lib.ajq_w4a16_gemm if scheme == "w4" else lib.ajq_w8a16_gemm
+    args = (x.data_ptr(), m, k, wq.data_ptr(), meta.data_ptr(), n, again.data_ptr(), _lib.AJQ_OUT_F32)
+    tail = (None, 0, torch.cuda.current_stream().cuda_stream) if scheme == "w4" else (torch.cuda.current_stream().cuda_stream,)
+    _lib.check(fn32(*args, *tail), "gemm")
+    torch.cuda.synchronize()
+    assert torch.equal(again, y32)  # run-to-run identical
+    pairs = y32.cpu().reshape(m, n // 16, 2, 8).double()
+    want = (torch.nn.functional.silu(pairs[:, :, 0]) * pairs[:, :, 1]).reshape(m, n // 2)
+    assert bf16_rounding_excess(gated.cpu(), want, 4e-6 * float(want.abs().max())) <= 0
+
+
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_gemv_and_gemm_agree(cuda, scheme):
     w_hat, wq, meta = _quantized(scheme, 2048, 2048, 41, cuda)
