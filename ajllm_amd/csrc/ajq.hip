@@ -305,19 +305,98 @@ int launch_gemv_rows(const uint16_t* x, int M, int K, const uint32_t* wq, const 
   return launch_gemv_cfg<kWaves, TPW, MROWS, kW4, false>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
-// Wide matrices whose K one batch per wave covers exactly: T row tiles per workgroup
-// (the activations are staged once per workgroup instead of once per row tile).
-template <int kWaves, int TPW, int MROWS, bool kW4>
-int launch_gemv_mt(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
-                   const uint16_t* scales8, int N, void* y, int out_f32, int T, hipStream_t stream) {
-  constexpr size_t lds = gemv_mt_lds_bytes(kWaves, TPW, MROWS);
-  static_assert(lds <= 160 * 1024, "GEMV configuration exceeds the 160 KiB LDS of a CU");
-  auto kernel = dequant_gemv_mt_kernel<kWaves, TPW, MROWS, kW4>;
-  if (int s = allow_big_lds(kernel, lds)) return s;
+// ---- resident-activation form of the weight-streaming kernel (skinny_resident_kernels.h): K = 2048 or 4096, a
+// run of T row tiles per workgroup, row blocks of 16 MB rows (MB = 1 for the GEMV's M <= 16, 2 above).  T is the
+// shortest run that fits the workgroups into one round of the chip (256: one workgroup per CU); where the longest
+// run still leaves more than one round, both forms are priced in bytes a CU pulls over its rounds (rounds x
+// workgroups per CU x (32 MB bytes of activations + 16 b T of weights) per unit of K) and the cheaper one runs.
+// Measured at 32 rows, K = 4096, int8 / int4, against the other form: N = 4096 (T = 1) 8.3 -> 7.6 / 8.2 -> 6.6 us;
+// N = 6144 (T = 2) 10.1 -> 9.4 / 8.7 -> 7.5; N = 28672 (T = 8) 31 -> 24 / 23 -> 19; a 128256-row head (T = 8, four
+// rounds) 103 -> 99 / 83 -> 72.
+#ifndef AJQ_SKINNY_RESIDENT
+#define AJQ_SKINNY_RESIDENT 1
+#endif
+// from this many workgroups of four row tiles on, the other form runs as four-wave workgroups, two to a CU
+#ifndef AJQ_SKINNY_FOUR_WAVE_MIN
+#define AJQ_SKINNY_FOUR_WAVE_MIN 512
+#endif
+template <bool kW4>
+long long skinny_cost(int ntiles, int mblocks, int tiles_per_wg, int slots, int mb = 2) {
+  const long long wgs = (long long)((ntiles + tiles_per_wg - 1) / tiles_per_wg) * mblocks;
+  return ((wgs + slots - 1) / slots) * (slots / 256) * (32 * mb + (kW4 ? 8 : 16) * tiles_per_wg);
+}
+// row tiles per workgroup of the resident form for (M, N, K), or 0 where the other form is taken (MB = 2 only: with
+// a 16-row block the caller has already decided)
+template <bool kW4, int MB>
+int skinny_resident_tiles(int M, int N, int K) {
+  if (!AJQ_SKINNY_RESIDENT || (K != 2048 && K != 4096)) return 0;
+  const int ntiles = N / kTileN, mblocks = (M + 16 * MB - 1) / (16 * MB);
+  if (MB == 1) {
+    for (int t : {2, 3, 4, 6, 8, 16})
+      if ((ntiles + t - 1) / t <= 256) return t;
+    return 16;
+  }
+  for (int t : {1, 2, 3, 4, 6, 8})
+    if ((long long)((ntiles + t - 1) / t) * mblocks <= 256) return t;
+  long long other = skinny_cost<kW4>(ntiles, mblocks, 1, 256);
+  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 2, 256));
+  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 4, (ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN ? 512 : 256));
+  int best = 0;
+  long long cost = other;
+  for (int t : {4, 6, 8}) {
+    const long long c = skinny_cost<kW4>(ntiles, mblocks, t, 256);
+    if (c <= cost) {  // (ties go to the resident form and to the longer run: the better pattern for HBM)
+      cost = c;
+      best = t;
+    }
+  }
+  return best;
+}
+// whether a GEMV (M <= 16) runs as the resident form with one 16-row block
+bool gemv_takes_resident(int M, int N, int K) {
+  return AJQ_SKINNY_RESIDENT && M >= 8 && M <= 16 && (K == 2048 || K == 4096) && N / kTileN > 256;
+}
+
+template <int TPW, int T, bool kW4, int kEpi, int MB>
+int launch_skinny_resident_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                               const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep,
+                               hipStream_t stream) {
   const int ntiles = N / kTileN;
-  hipLaunchKernelGGL(kernel, dim3((ntiles + T - 1) / T), dim3(kWaves * 64), lds, stream,
-                     reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M | (out_f32 << 8), N, y, scales8, T);
+  const int nruns = (ntiles + T - 1) / T, mblocks = (M + 16 * MB - 1) / (16 * MB);
+  const dim3 grid(8 * ((nruns + 7) / 8) * mblocks), block(kResWaves * 64);
+  if constexpr (kEpi != 0) {
+    auto kernel = dequant_skinny_resident_epi_kernel<TPW, T, kW4, kEpi, MB>;
+    if (int s = allow_big_lds(kernel, kResEpiLdsBytes)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, kResEpiLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+                       out_f32, scales8, ep);
+  } else {
+    auto kernel = dequant_skinny_resident_kernel<TPW, T, kW4, MB>;
+    if (int s = allow_big_lds(kernel, kResLdsBytes)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, kResLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+                       out_f32, scales8);
+  }
   return AJQ_OK;
+}
+
+template <bool kW4, int kEpi, int MB>
+int launch_skinny_resident(int T, const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
+                           const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+#define AJQ_RES(P, TT)                \
+  if (K == 1024 * P && T == TT)       \
+    return launch_skinny_resident_cfg<P, TT, kW4, kEpi, MB>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
+#define AJQ_RES_K(P)                  \
+  if constexpr (MB == 2) AJQ_RES(P, 1); \
+  AJQ_RES(P, 2);                      \
+  AJQ_RES(P, 3);                      \
+  AJQ_RES(P, 4);                      \
+  AJQ_RES(P, 6);                      \
+  AJQ_RES(P, 8);                      \
+  if constexpr (MB == 1) AJQ_RES(P, 16)
+  AJQ_RES_K(4);
+  AJQ_RES_K(2);
+#undef AJQ_RES_K
+#undef AJQ_RES
+  return fail(AJQ_ERR_UNSUPPORTED, "no resident-activation configuration for K = %d, %d row tiles", K, T);
 }
 
 // Row bound MROWS is the next power of two >= M; above 4 rows a wave stages two
@@ -326,18 +405,13 @@ int launch_gemv_mt(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 template <bool kW4>
 int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
                 const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
-  // 8 < = M, K = 4096 and more row tiles than CUs: several row tiles per workgroup, at most one
-  // workgroup per CU (measured on 14336 x 4096: 9.9 us against 16.5 us at M = 16; below
-  // M = 8 the single-tile kernel is the faster one)
-  const int ntiles = N / kTileN;
-  if (K == 8 * 4 * kGroup && ntiles > 256 && M >= 8) {
-    const int T = (ntiles + 255) / 256;
-    if (M <= 8) return launch_gemv_mt<8, 4, 8, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, T, stream);
-    return launch_gemv_mt<8, 4, 16, kW4>(x, M, K, wq, meta, scales8, N, y, out_f32, T, stream);
-  }
-  // (the same form at K = 2048 was measured on the 12-layer model's q|k|v and head at batch 8 and is slower: the
-  // linears of a step 0.226 against 0.215 ms; a workgroup's T row tiles in sequence cost more than the activation
-  // traffic they save when a tile is only 16 KiB)
+  // 8 <= M, K = 2048 or 4096 and more row tiles than CUs: the resident-activation form of the weight-streaming
+  // kernel with a 16-row block (a workgroup keeps its activations in registers and walks a run of row tiles past
+  // them; W4, M = 16: 14336 x 4096 10.4 -> 8.5 us, a 32000 x 2048 head 15.4 -> 9.1; below M = 8 and up to 256 row
+  // tiles the single-tile kernel is the faster one)
+  if (gemv_takes_resident(M, N, K))
+    return launch_skinny_resident<kW4, 0, 1>(skinny_resident_tiles<kW4, 1>(M, N, K), x, M, K, wq, meta, scales8, N, y, out_f32,
+                                             GemvEpilogue{}, stream);
   if (K == 8 * 2 * kGroup) {  // K = 2048: one batch of two groups per wave, straight-line kernel
     if (M <= 1) return launch_gemv_cfg<8, 2, 1, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
     if (M <= 2) return launch_gemv_cfg<8, 2, 2, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
@@ -481,83 +555,9 @@ int launch_skinny_split(const uint16_t* x, int M, int K, const uint32_t* wq, con
   return launch_skinny_split_kernel<kW4, kEpi, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
 }
 
-// from this many workgroups of four row tiles on, the kernel runs as four-wave workgroups, two to a CU
-#ifndef AJQ_SKINNY_FOUR_WAVE_MIN
-#define AJQ_SKINNY_FOUR_WAVE_MIN 512
-#endif
 #ifndef AJQ_SKINNY_FORCE_NT
 #define AJQ_SKINNY_FORCE_NT 0
 #endif
-
-// ---- resident-activation form of the weight-streaming kernel (skinny_resident_kernels.h): K = 2048 or 4096, a
-// run of T = 4, 7 or 8 row tiles per workgroup.  Both forms are priced in bytes a CU pulls over its rounds of
-// workgroups: rounds x workgroups per CU x (64 bytes of activations + 16 b T of weights) per unit of K; the
-// resident form is taken where it is cheaper (N = 28672 at 32 rows: 7 tiles x 256 workgroups, 31 -> 24 us for
-// int8; a 128256-row head: 8 tiles; N = 14336: 4 tiles; N <= 8192 stays with the other form).
-#ifndef AJQ_SKINNY_RESIDENT
-#define AJQ_SKINNY_RESIDENT 1
-#endif
-template <bool kW4>
-long long skinny_cost(int ntiles, int mblocks, int tiles_per_wg, int slots) {
-  const long long wgs = (long long)((ntiles + tiles_per_wg - 1) / tiles_per_wg) * mblocks;
-  return ((wgs + slots - 1) / slots) * (slots / 256) * (64 + (kW4 ? 8 : 16) * tiles_per_wg);
-}
-// row tiles per workgroup of the resident form for (M, N, K), or 0 where the other form is taken
-template <bool kW4>
-int skinny_resident_tiles(int M, int N, int K) {
-  if (!AJQ_SKINNY_RESIDENT || (K != 2048 && K != 4096)) return 0;
-  const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
-  long long other = skinny_cost<kW4>(ntiles, mblocks, 1, 256);
-  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 2, 256));
-  other = std::min(other, skinny_cost<kW4>(ntiles, mblocks, 4, (ntiles / 4) * mblocks >= AJQ_SKINNY_FOUR_WAVE_MIN ? 512 : 256));
-  int best = 0;
-  long long cost = other;
-  for (int t : {4, 7, 8}) {
-    const long long c = skinny_cost<kW4>(ntiles, mblocks, t, 256);
-    if (c <= cost) {  // (ties go to the resident form and to the longer run: the better pattern for HBM)
-      cost = c;
-      best = t;
-    }
-  }
-  return best;
-}
-
-template <int TPW, int T, bool kW4, int kEpi>
-int launch_skinny_resident_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
-                               const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep,
-                               hipStream_t stream) {
-  const int ntiles = N / kTileN;
-  const int nruns = (ntiles + T - 1) / T, mblocks = (M + 31) / 32;
-  const dim3 grid(8 * ((nruns + 7) / 8) * mblocks), block(kResWaves * 64);
-  if constexpr (kEpi != 0) {
-    auto kernel = dequant_skinny_resident_epi_kernel<TPW, T, kW4, kEpi>;
-    if (int s = allow_big_lds(kernel, kResEpiLdsBytes)) return s;
-    hipLaunchKernelGGL(kernel, grid, block, kResEpiLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
-                       out_f32, scales8, ep);
-  } else {
-    auto kernel = dequant_skinny_resident_kernel<TPW, T, kW4>;
-    if (int s = allow_big_lds(kernel, kResLdsBytes)) return s;
-    hipLaunchKernelGGL(kernel, grid, block, kResLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
-                       out_f32, scales8);
-  }
-  return AJQ_OK;
-}
-
-template <bool kW4, int kEpi>
-int launch_skinny_resident(int T, const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta,
-                           const uint16_t* scales8, int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
-#define AJQ_RES(P, TT) \
-  if (K == 1024 * P && T == TT) \
-    return launch_skinny_resident_cfg<P, TT, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
-  AJQ_RES(4, 4);
-  AJQ_RES(4, 7);
-  AJQ_RES(4, 8);
-  AJQ_RES(2, 4);
-  AJQ_RES(2, 7);
-  AJQ_RES(2, 8);
-#undef AJQ_RES
-  return fail(AJQ_ERR_UNSUPPORTED, "no resident-activation configuration for K = %d, %d row tiles", K, T);
-}
 
 // M >= 17.  Row blocks of 32 rows of M and 1, 2 or 4 row tiles of N per workgroup.  A workgroup
 // moves K * (2 * 32 + bytes per weight * 16 * tiles) bytes (the activations come from L2 once per
@@ -589,8 +589,8 @@ template <bool kW4, int kEpi>
 int launch_skinny_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                       int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
   if (skinny_split_applies(M, N, K)) return launch_skinny_split<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
-  if (const int T = skinny_resident_tiles<kW4>(M, N, K))
-    return launch_skinny_resident<kW4, kEpi>(T, x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if (const int T = skinny_resident_tiles<kW4, 2>(M, N, K))
+    return launch_skinny_resident<kW4, kEpi, 2>(T, x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   const int nt = skinny_row_tiles<kW4>(M, N);
   const int ntiles = N / kTileN, mblocks = (M + 31) / 32;
   if (nt == 1) return launch_skinny_epi_cfg<8, 2, 32, 1, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
@@ -605,8 +605,8 @@ int launch_skinny(const uint16_t* x, int M, int K, const uint32_t* wq, const uin
                   const uint16_t* scales8, int N, void* y, int out_f32, hipStream_t stream) {
   if (skinny_split_applies(M, N, K))
     return launch_skinny_split<kW4, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
-  if (const int T = skinny_resident_tiles<kW4>(M, N, K))
-    return launch_skinny_resident<kW4, 0>(T, x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
+  if (const int T = skinny_resident_tiles<kW4, 2>(M, N, K))
+    return launch_skinny_resident<kW4, 0, 2>(T, x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
   const int ntiles = N / kTileN;
   const int mblocks = (M + 31) / 32;
   int nt = 1;
@@ -661,6 +661,9 @@ template <bool kW4, int kEpi>
 int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                     int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
   if (!gemv_epi_straight(M, K)) return launch_skinny_epi<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
+  if (gemv_takes_resident(M, N, K))
+    return launch_skinny_resident<kW4, kEpi, 1>(skinny_resident_tiles<kW4, 1>(M, N, K), x, M, K, wq, meta, scales8, N, y, out_f32, ep,
+                                                stream);
 #define AJQ_EPI(W, T, R) return launch_gemv_epi_cfg<W, T, R, kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream)
   if (K == 2048) {
     if (M <= 1) AJQ_EPI(8, 2, 1);

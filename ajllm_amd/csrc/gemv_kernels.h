@@ -407,182 +407,6 @@ __global__ __launch_bounds__(kWaves * 64) void dequant_gemv_epi_kernel(
   dequant_gemv_body<kWaves, TPW, MROWS, kW4, kSingle, kEpi, kFrags>(wq, meta, x, K, m_flags, N, y, scales8, ep);
 }
 
-// ---------------------------------------------------------------------------
-// Multi-tile variant for wide matrices (N / 16 well above the CU count) with
-// K == kWaves * TPW * 128: a workgroup walks T consecutive 16-row tiles of N.
-// A wave stages its k-slice of the activations ONCE (and forms the group sums
-// once) and then streams the weight tiles of one row tile after the other, the
-// next row tile's loads in flight while the current one is computed.  For M = 16
-// this cuts the activation traffic out of L2 by T (every workgroup otherwise
-// re-stages all of x for a single row tile).  The waves' partial sums of a row
-// tile meet in one of two LDS buffers; wave (tile index mod kWaves) adds them in
-// wave order and stores, so one barrier per row tile suffices and the result is
-// as deterministic as the single-tile kernel's.
-// ---------------------------------------------------------------------------
-template <int kWaves, int TPW, int MROWS, bool kW4>
-__global__ __launch_bounds__(kWaves * 64) void dequant_gemv_mt_kernel(
-    const u32x4_t* __restrict__ wq,
-    const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
-    const uint16_t* __restrict__ x, int K,
-    int m_flags,  // M | out_f32 << 8
-    int N, void* __restrict__ y,
-    const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
-    int T) {                               // row tiles per workgroup
-  const int M = m_flags & 0xFF;
-  const bool out_f32 = (m_flags >> 8) != 0;
-  constexpr int kSlice = TPW * kGroup;
-  constexpr int kStride = kSlice + 8;
-  constexpr int kVecPerRow = kSlice / 8;
-  constexpr int kVecs = MROWS * kVecPerRow;
-  constexpr int kXLoads = (kVecs + 63) / 64;
-  constexpr int kLoadsPerGroup = kW4 ? 1 : 2;
-  constexpr int kRowQuads = (MROWS + 3) / 4;
-  constexpr int kLive = MROWS < 4 ? MROWS : 4;
-  typedef float live_t __attribute__((ext_vector_type(kLive == 3 ? 4 : kLive)));
-
-  extern __shared__ u32x4_t smem_raw[];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int nl = lane & 15, kc = lane >> 4;
-  const int G = K >> 7;
-  const int ntiles = N / kTileN;
-  const int nt_begin = blockIdx.x * T;
-  const int nt_end = min(ntiles, nt_begin + T);
-  uint16_t* xs = reinterpret_cast<uint16_t*>(smem_raw) + wave * (MROWS * kStride);
-  live_t* redv = reinterpret_cast<live_t*>(reinterpret_cast<uint16_t*>(smem_raw) + kWaves * (MROWS * kStride));
-  constexpr int kRedStride = kWaves * 16 * kRowQuads;  // live_t elements of one reduction buffer
-  const int g0 = wave * TPW;
-
-  struct Tile {
-    u32x4_t w[TPW][kLoadsPerGroup];
-    uint32_t m[TPW];
-  };
-  auto load = [&](Tile& b, int nt) {
-    __builtin_amdgcn_sched_barrier(0);
-    const u32x4_t* wtile = wq + ((size_t)nt * G + g0) * kLoadsPerGroup * 64 + lane;
-#pragma unroll
-    for (int p = 0; p < TPW; ++p)
-#pragma unroll
-      for (int h = 0; h < kLoadsPerGroup; ++h)
-        b.w[p][h] = __builtin_nontemporal_load(wtile + (p * kLoadsPerGroup + h) * 64);
-    if (kW4) {
-      const uint32_t* mtile = meta + ((size_t)nt * G + g0) * 16 + nl;
-#pragma unroll
-      for (int p = 0; p < TPW; ++p) b.m[p] = mtile[p * 16];
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  Tile t0, t1;
-  load(t0, nt_begin);
-  // ---- the wave's slice of the activations, once: global -> registers -> its own LDS rows
-  {
-    u32x4_t xv[kXLoads];
-#pragma unroll
-    for (int i = 0; i < kXLoads; ++i) {
-      const int v = min(lane + 64 * i, kVecs - 1);
-      const int m = min(v / kVecPerRow, M - 1), c = v % kVecPerRow;
-      xv[i] = *reinterpret_cast<const u32x4_t*>(x + (size_t)m * K + g0 * kGroup + 8 * c);
-    }
-#pragma unroll
-    for (int i = 0; i < kXLoads; ++i) {
-      const int v = lane + 64 * i;
-      if ((i + 1) * 64 <= kVecs || v < kVecs)
-        *reinterpret_cast<u32x4_t*>(xs + (v / kVecPerRow) * kStride + 8 * (v % kVecPerRow)) = xv[i];
-    }
-  }
-  const W4Consts w4c = w4_consts();
-  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-  const uint16_t* xrow = xs + min(nl, M - 1) * kStride + 8 * kc;
-  // group sums of the activations (zero-point term), once for all row tiles
-  f32x4_t asum[TPW];
-  if (kW4) {
-#pragma unroll
-    for (int p = 0; p < TPW; ++p) {
-      asum[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        asum[p] = mfma16(*reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j), ones, asum[p]);
-    }
-  }
-
-  auto compute = [&](Tile& b, int nt, int slot) {
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    if (kW4) {
-      float sc[TPW], zc[TPW];
-#pragma unroll
-      for (int p = 0; p < TPW; ++p) {
-        sc[p] = f16_bits_to_f32(b.m[p] & 0xFFFFu);
-        zc[p] = f16_bits_to_f32(b.m[p] >> 16);
-      }
-#pragma unroll
-      for (int p = 0; p < TPW; ++p) {
-        f32x4_t part = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-          part = mfma16(a, w4_unpack(b.w[p][0][j], w4c), part);
-        }
-#pragma unroll
-        for (int i = 0; i < kLive; ++i) acc[i] += sc[p] * (part[i] - zc[p] * asum[p][i]);
-      }
-    } else {
-#pragma unroll
-      for (int p = 0; p < TPW; ++p)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(xrow + p * kGroup + 32 * j);
-          const u32x2_t lo = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1)]);
-          const u32x2_t hi = w8_to_bf16(b.w[p][j >> 1][2 * (j & 1) + 1]);
-          acc = mfma16(a, u32x4_t{lo.x, lo.y, hi.x, hi.y}, acc);
-        }
-    }
-    asm volatile("" : "+v"(acc));
-    live_t mine;
-#pragma unroll
-    for (int i = 0; i < kLive; ++i) mine[i] = acc[i];
-    live_t* buf = redv + slot * kRedStride;
-    if (kc < kRowQuads) buf[wave * (16 * kRowQuads) + lane] = mine;
-    __syncthreads();
-    // the buffer is written again two row tiles later, after another barrier that the
-    // adding wave only reaches once it is through here
-    if (wave == (nt - nt_begin) % kWaves && kc < kRowQuads) {
-      live_t part[kWaves];
-#pragma unroll
-      for (int w = 0; w < kWaves; ++w) part[w] = buf[w * (16 * kRowQuads) + lane];
-      live_t sum = part[0];
-#pragma unroll
-      for (int w = 1; w < kWaves; ++w) sum += part[w];
-      const int n = nt * kTileN + nl;
-      float cs = 1.0f;
-      if (!kW4) cs = f16_bits_to_f32(scales8[n]);
-#pragma unroll
-      for (int i = 0; i < kLive; ++i) {
-        const int m = 4 * kc + i;
-        if (m < M) {
-          const float v = sum[i] * cs;
-          if (out_f32)
-            reinterpret_cast<float*>(y)[(size_t)m * N + n] = v;
-          else
-            reinterpret_cast<uint16_t*>(y)[(size_t)m * N + n] = f32_to_bf16_rne(v);
-        }
-      }
-    }
-  };
-
-  for (int nt = nt_begin; nt < nt_end; nt += 2) {
-    const bool has1 = nt + 1 < nt_end;
-    if (has1) load(t1, nt + 1);
-    compute(t0, nt, 0);
-    if (nt + 2 < nt_end) load(t0, nt + 2);
-    if (has1) compute(t1, nt + 1, 1);
-  }
-}
-
-constexpr size_t gemv_mt_lds_bytes(int waves, int tpw, int mrows) {
-  return (size_t)waves * mrows * (tpw * kGroup + 8) * 2 + (size_t)2 * waves * 64 * 16;
-}
-
 // LDS bytes of one workgroup of dequant_gemv_kernel<kWaves, TPW, MROWS, *>
 constexpr size_t gemv_lds_bytes(int waves, int tpw, int mrows) {
   return (size_t)waves * mrows * (tpw * kGroup + 8) * 2 + (size_t)waves * 64 * 16;

@@ -9,8 +9,8 @@
 //    row tile of the workgroup.  It loads its slice of the 32 activation rows once (row-major, through a
 //    wave-private LDS region, no barrier), and keeps it as MFMA A fragments in registers: 32 TPW registers;
 //  * W4: the slice's group sums (for the zero-point term) are formed once, not once per row tile;
-//  * then the row tiles one after the other: the wave's 2 or 1 KiB x TPW of tile t + 1 travel while tile t is
-//    computed (two register sets, asm loads with exact waits); the eight waves together read a tile's 16 K bytes
+//  * then the row tiles one after the other: the wave's 2 or 1 KiB x TPW of tiles t + 1 and (once tile t is done)
+//    t + 2 travel while tile t is computed (two register sets, asm loads with exact waits); the eight waves together read a tile's 16 K bytes
 //    as one contiguous run and the workgroup its T tiles as one contiguous sweep, which HBM serves much better than
 //    one 64 KiB stream per wave (measured: 4.8 against 6 TB/s and more);
 //  * a wave parks each finished tile's partial sums in its LDS region; at the end the (row tile, 16-row block)
@@ -24,8 +24,8 @@
 namespace ajq {
 
 constexpr int kResWaves = 8;
-constexpr int kResMaxTiles = 8;                               // row tiles per workgroup, at most
-constexpr int kResRegionBytes = kResMaxTiles * 2 * 1024;      // a wave's LDS region: 2 KiB of partial sums per tile
+constexpr int kResMaxUnits = 16;                              // (row tile, 16-row block) units per workgroup, at most
+constexpr int kResRegionBytes = kResMaxUnits * 1024;          // a wave's LDS region: 1 KiB of partial sums per unit
 constexpr int kResStride = kGroup + 8;                        // staging: one group of a row, padded, bf16 elements
 static_assert(32 * kResStride * 2 <= kResRegionBytes, "the staging of one group fits the wave's region");
 constexpr size_t kResLdsBytes = (size_t)kResWaves * kResRegionBytes;                    // 128 KiB
@@ -60,15 +60,19 @@ __device__ __forceinline__ void wait_rows(u32x4_t (&r)[8]) {
                : "n"(kLeft)
                : "memory");
 }
+template <int kLeft>
+__device__ __forceinline__ void wait_rows(u32x4_t (&r)[4]) {
+  asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(kLeft) : "memory");
+}
 
-template <int TPW, int T, bool kW4, int kEpi>
+template <int TPW, int T, bool kW4, int kEpi, int MB = 2>
 __device__ __forceinline__ void dequant_skinny_resident_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
     const GemvEpilogue& ep) {
-  static_assert(T >= 1 && T <= kResMaxTiles, "a wave's region holds the partial sums of T row tiles");
+  static_assert(T >= 1 && T * MB <= kResMaxUnits, "a wave's region holds the partial sums of T row tiles");
   constexpr int kWaves = kResWaves;
   constexpr int kLPG = kW4 ? 1 : 2;              // 1 KiB weight tiles per group
   constexpr int kWL = TPW * (kLPG + (kW4 ? 1 : 0));  // loads per wave and row tile
@@ -81,12 +85,13 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   // workgroup -> (run of T row tiles, row block): the row blocks of one run share an XCD (see dequant_skinny_kernel)
   const int ntiles = N / kTileN;
   const int nruns = (ntiles + T - 1) / T;
-  const int mblocks = (M + 31) / 32;
+  constexpr int kRows = 16 * MB;  // rows of a row block
+  const int mblocks = (M + kRows - 1) / kRows;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int run = xcd + 8 * (slot / mblocks);
   if (run >= nruns) return;  // padding of the last round (whole workgroup: no barrier is left waiting)
   const int mblock = slot % mblocks;
-  const int m0 = mblock * 32;
+  const int m0 = mblock * kRows;
   const int nt0 = run * T;
   const int tiles = min(T, ntiles - nt0);  // >= 1; past the matrix the last row tile is computed again, not stored
   const int G = K >> 7;                    // = kWaves * TPW (checked by the host)
@@ -111,44 +116,47 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   // ---- the activation slice: one group at a time, row-major into the wave's region (rows padded by 16 B so the
   // 16 rows of an A fragment fall in distinct banks), back as A fragments; LDS operations of one wave execute in
   // order, so no barrier is needed
-  u32x4_t frag[TPW][4][2];
-  f32x4_t asum[TPW][2];
+  u32x4_t frag[TPW][4][MB];
+  f32x4_t asum[TPW][MB];
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   Tile set[2];
   {
     // all requests of the prologue are asm, so that every wait is exact: the activations (L2 hits) come back while
     // the first row tile's weights are still on their way from memory
-    u32x4_t raw[TPW][8];
-    uint32_t xoff[8];
+    constexpr int kXL = 4 * MB;  // 16-byte vectors per lane and group
+    u32x4_t raw[TPW][kXL];
+    uint32_t xoff[kXL];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kXL; ++i) {
       const int v = lane + 64 * i;  // 16-byte vector v of a 32 x 128 block: row v / 16, vector v % 16
       xoff[i] = (uint32_t)((min(m0 + (v >> 4), M - 1) * K + 8 * (v & 15)) * 2);
     }
 #pragma unroll
     for (int p = 0; p < TPW; ++p)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) load16_async(raw[p][i], reinterpret_cast<const char*>(x) + (g0 + p) * (kGroup * 2), xoff[i]);
+      for (int i = 0; i < kXL; ++i) load16_async(raw[p][i], reinterpret_cast<const char*>(x) + (g0 + p) * (kGroup * 2), xoff[i]);
     request(set[0], 0);
+    if (T > 1) request(set[1], 1);  // two row tiles' weights travel while the activations are staged
+    constexpr int kAhead = (T > 1 ? 2 : 1) * kWL;
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
-      if (p == 0) wait_rows<kWL + 8 * (TPW - 1)>(raw[0]);
-      if (p == 1) wait_rows<kWL + 8 * (TPW > 1 ? TPW - 2 : 0)>(raw[TPW > 1 ? 1 : 0]);
-      if (p == 2) wait_rows<kWL + 8 * (TPW > 2 ? TPW - 3 : 0)>(raw[TPW > 2 ? 2 : 0]);
-      if (p == 3) wait_rows<kWL>(raw[TPW > 3 ? 3 : 0]);
+      if (p == 0) wait_rows<kAhead + kXL * (TPW - 1)>(raw[0]);
+      if (p == 1) wait_rows<kAhead + kXL * (TPW > 1 ? TPW - 2 : 0)>(raw[TPW > 1 ? 1 : 0]);
+      if (p == 2) wait_rows<kAhead + kXL * (TPW > 2 ? TPW - 3 : 0)>(raw[TPW > 2 ? 2 : 0]);
+      if (p == 3) wait_rows<kAhead>(raw[TPW > 3 ? 3 : 0]);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kXL; ++i) {
         const int v = lane + 64 * i;
         *reinterpret_cast<u32x4_t*>(xs + (v >> 4) * kResStride + 8 * (v & 15)) = raw[p][i];
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+        for (int r = 0; r < MB; ++r)
           frag[p][j][r] = *reinterpret_cast<const u32x4_t*>(xs + (16 * r + nl) * kResStride + 32 * j + 8 * kc);
       if (kW4) {
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
+        for (int r = 0; r < MB; ++r) {
           asum[p][r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int j = 0; j < 4; ++j) asum[p][r] = mfma16(frag[p][j][r], ones, asum[p][r]);
@@ -167,7 +175,7 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
 #pragma unroll
     for (int u = 0; u < kShareLoads; ++u) {
       const int j = wave * 2 + half + u * kWaves * 2;
-      const bool live = 4 * j < ep.parts && m < M;  // (idle lanes re-read the first 16 bytes)
+      const bool live = 4 * j < ep.parts && m < M && (lane & 31) < kRows;  // (idle lanes re-read the first 16 bytes)
       const float4 t = *reinterpret_cast<const float4*>(ep.ssq_in + (live ? (size_t)m * ep.parts + 4 * j : 0));
       ssq_share[u] = live ? t : float4{0.f, 0.f, 0.f, 0.f};
     }
@@ -176,21 +184,25 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   const W4Consts w4c = w4_consts();
   f32x4_t* mine = reinterpret_cast<f32x4_t*>(region);  // [tile][16-row block][lane]
   auto compute = [&](Tile& set, int t) __attribute__((always_inline)) {
-    f32x4_t acc[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+    f32x4_t acc[MB];
+#pragma unroll
+    for (int r = 0; r < MB; ++r) acc[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       if (kW4) {
         const float sc = f16_bits_to_f32(set.m[p] & 0xFFFFu), zc = f16_bits_to_f32(set.m[p] >> 16);
-        f32x4_t part[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};
+        f32x4_t part[MB];
+#pragma unroll
+        for (int r = 0; r < MB; ++r) part[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const u32x4_t w = w4_unpack(set.w[p][0][j], w4c);
 #pragma unroll
-          for (int r = 0; r < 2; ++r) part[r] = mfma16(frag[p][j][r], w, part[r]);
+          for (int r = 0; r < MB; ++r) part[r] = mfma16(frag[p][j][r], w, part[r]);
         }
         // (128+q) and (128+z) cancel in fp32 before the scale is applied
 #pragma unroll
-        for (int r = 0; r < 2; ++r)
+        for (int r = 0; r < MB; ++r)
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[r][i] += sc * (part[r][i] - zc * asum[p][r][i]);
       } else {
@@ -200,26 +212,26 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
           const u32x2_t hi = w8_to_bf16(set.w[p][j >> 1][2 * (j & 1) + 1]);
           const u32x4_t w = u32x4_t{lo.x, lo.y, hi.x, hi.y};
 #pragma unroll
-          for (int r = 0; r < 2; ++r) acc[r] = mfma16(frag[p][j][r], w, acc[r]);
+          for (int r = 0; r < MB; ++r) acc[r] = mfma16(frag[p][j][r], w, acc[r]);
         }
       }
     }
 #pragma unroll
-    for (int r = 0; r < 2; ++r) mine[(t * 2 + r) * 64 + lane] = acc[r];
+    for (int r = 0; r < MB; ++r) mine[(t * MB + r) * 64 + lane] = acc[r];
   };
 
-  // ---- the row tiles, two register sets in turn (the first tile's weights were requested in the prologue).
+  // ---- the row tiles, two register sets in turn (the first two tiles' weights were requested in the prologue;
+  // a set is requested again as soon as its tile is computed).
   // Straight-line code on purpose: with the sets carried around a loop the compiler may copy a set's registers
   // between the request and the wait, while the loads are still in flight.
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    if (t + 1 < T) {
-      request(set[(t + 1) & 1], t + 1);
+    if (t + 1 < T)
       wait_tile<kWL>(set[t & 1]);
-    } else {
+    else
       wait_tile<0>(set[t & 1]);
-    }
     compute(set[t & 1], t);
+    if (t + 2 < T) request(set[t & 1], t + 2);
   }
 
   if (kEpi & kEpiRowScale) {
@@ -231,8 +243,8 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   }
   __syncthreads();
   // ---- the (row tile, 16-row block) units, dealt round-robin to the waves: the waves' partial sums in wave order
-  for (int u = wave; u < 2 * tiles; u += kWaves) {
-    const int t = u >> 1, r = u & 1;
+  for (int u = wave; u < MB * tiles; u += kWaves) {
+    const int t = u / MB, r = u % MB;
     f32x4_t part[kWaves];
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
@@ -254,18 +266,18 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   }
 }
 
-template <int TPW, int T, bool kW4>
+template <int TPW, int T, bool kW4, int MB = 2>
 __global__ __launch_bounds__(kResWaves * 64, 1) void dequant_skinny_resident_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8) {
-  dequant_skinny_resident_body<TPW, T, kW4, 0>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
+  dequant_skinny_resident_body<TPW, T, kW4, 0, MB>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
 }
 
-template <int TPW, int T, bool kW4, int kEpi>
+template <int TPW, int T, bool kW4, int kEpi, int MB = 2>
 __global__ __launch_bounds__(kResWaves * 64, 1) void dequant_skinny_resident_epi_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
-  dequant_skinny_resident_body<TPW, T, kW4, kEpi>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
+  dequant_skinny_resident_body<TPW, T, kW4, kEpi, MB>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
 }
 
 }  // namespace ajq
