@@ -79,7 +79,7 @@ int allow_big_lds(Kernel kernel, size_t bytes) {
     const void* kernel;
     size_t bytes[16];
   };
-  static thread_local Grant grants[64] = {};
+  static thread_local Grant grants[192] = {};
   if (bytes <= 64 * 1024) return AJQ_OK;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = 0;
@@ -366,13 +366,15 @@ int launch_skinny_resident_cfg(const uint16_t* x, int M, int K, const uint32_t* 
   const dim3 grid(8 * ((nruns + 7) / 8) * mblocks), block(kResWaves * 64);
   if constexpr (kEpi != 0) {
     auto kernel = dequant_skinny_resident_epi_kernel<TPW, T, kW4, kEpi, MB>;
-    if (int s = allow_big_lds(kernel, kResEpiLdsBytes)) return s;
-    hipLaunchKernelGGL(kernel, grid, block, kResEpiLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+    constexpr size_t lds = res_lds_bytes(T, MB, true);
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
                        out_f32, scales8, ep);
   } else {
     auto kernel = dequant_skinny_resident_kernel<TPW, T, kW4, MB>;
-    if (int s = allow_big_lds(kernel, kResLdsBytes)) return s;
-    hipLaunchKernelGGL(kernel, grid, block, kResLdsBytes, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
+    constexpr size_t lds = res_lds_bytes(T, MB, false);
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y,
                        out_f32, scales8);
   }
   return AJQ_OK;

@@ -25,11 +25,15 @@ namespace ajq {
 
 constexpr int kResWaves = 8;
 constexpr int kResMaxUnits = 16;                              // (row tile, 16-row block) units per workgroup, at most
-constexpr int kResRegionBytes = kResMaxUnits * 1024;          // a wave's LDS region: 1 KiB of partial sums per unit
 constexpr int kResStride = kGroup + 8;                        // staging: one group of a row, padded, bf16 elements
-static_assert(32 * kResStride * 2 <= kResRegionBytes, "the staging of one group fits the wave's region");
-constexpr size_t kResLdsBytes = (size_t)kResWaves * kResRegionBytes;                    // 128 KiB
-constexpr size_t kResEpiLdsBytes = kResLdsBytes + (size_t)32 * kResWaves * 4;           // + the rows' sums of squares
+// a wave's LDS region: the staging of one group of its 16 MB rows, later 1 KiB of partial sums per unit
+constexpr int res_region_bytes(int tiles, int mb) {
+  return 16 * mb * kResStride * 2 > tiles * mb * 1024 ? 16 * mb * kResStride * 2 : tiles * mb * 1024;
+}
+// LDS bytes of one workgroup; the epilogue forms add the rows' sums of squares, one share per wave
+constexpr size_t res_lds_bytes(int tiles, int mb, bool epi) {
+  return (size_t)kResWaves * res_region_bytes(tiles, mb) + (epi ? (size_t)32 * kResWaves * 4 : 0);
+}
 
 __device__ __forceinline__ void load16_async_nt(u32x4_t& dst, const void* base, uint32_t voff) {
   asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(dst) : "v"(voff), "s"(base) : "memory");
@@ -96,7 +100,8 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   const int tiles = min(T, ntiles - nt0);  // >= 1; past the matrix the last row tile is computed again, not stored
   const int G = K >> 7;                    // = kWaves * TPW (checked by the host)
   const int g0 = wave * TPW;
-  char* region = reinterpret_cast<char*>(smem_raw) + wave * kResRegionBytes;
+  constexpr int kRegionBytes = res_region_bytes(T, MB);
+  char* region = reinterpret_cast<char*>(smem_raw) + wave * kRegionBytes;
   uint16_t* xs = reinterpret_cast<uint16_t*>(region);
 
   // ---- this wave's slice of the weights of row tile nt0 + t: TPW * kLPG KiB, contiguous
@@ -169,7 +174,7 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   // half-waves take alternate 16-byte pieces), used at the end
   constexpr int kShareLoads = 32 / kWaves;
   float4 ssq_share[kShareLoads];
-  float* red2 = reinterpret_cast<float*>(reinterpret_cast<char*>(smem_raw) + kResLdsBytes);  // [32][kWaves]
+  float* red2 = reinterpret_cast<float*>(reinterpret_cast<char*>(smem_raw) + kWaves * kRegionBytes);  // [32][kWaves]
   if (kEpi & kEpiRowScale) {
     const int m = m0 + (lane & 31), half = lane >> 5;
 #pragma unroll
@@ -248,7 +253,7 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
     f32x4_t part[kWaves];
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
-      part[w] = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const char*>(smem_raw) + w * kResRegionBytes)[u * 64 + lane];
+      part[w] = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const char*>(smem_raw) + w * kRegionBytes)[u * 64 + lane];
     f32x4_t sum = part[0];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w) sum += part[w];
@@ -267,14 +272,14 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
 }
 
 template <int TPW, int T, bool kW4, int MB = 2>
-__global__ __launch_bounds__(kResWaves * 64, 1) void dequant_skinny_resident_kernel(
+__global__ __launch_bounds__(kResWaves * 64, 2) void dequant_skinny_resident_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8) {
   dequant_skinny_resident_body<TPW, T, kW4, 0, MB>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{});
 }
 
 template <int TPW, int T, bool kW4, int kEpi, int MB = 2>
-__global__ __launch_bounds__(kResWaves * 64, 1) void dequant_skinny_resident_epi_kernel(
+__global__ __launch_bounds__(kResWaves * 64, 2) void dequant_skinny_resident_epi_kernel(
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
   dequant_skinny_resident_body<TPW, T, kW4, kEpi, MB>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
