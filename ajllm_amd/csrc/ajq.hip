@@ -305,6 +305,52 @@ int launch_gemv_rows(const uint16_t* x, int M, int K, const uint32_t* wq, const 
   return launch_gemv_cfg<kWaves, TPW, MROWS, kW4, false>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
 }
 
+// ---- split-K form of the weight-streaming kernel (see kSplitK in skinny_kernels.h): only with a buffer the caller
+// has lent to this host thread's calls (ajq_matmul_workspace_set), which holds the ticket words and the partial sums
+constexpr int kSplitTiles = 4, kSplitWays = 4;          // row tiles per workgroup, workgroups per row-tile group
+constexpr size_t kSplitTicketBytes = 4096;              // one word per (row-tile group, row block), zeroed
+constexpr int kSplitMaxCells = 64;                      // 256 workgroups: one round of the chip
+constexpr size_t kSplitCellBytes = (size_t)kSplitWays * kSplitTiles * 2 * 1024;
+constexpr size_t kSplitWorkspaceBytes = kSplitTicketBytes + kSplitMaxCells * kSplitCellBytes;
+struct SplitWorkspace {
+  void* base = nullptr;
+  size_t bytes = 0;
+};
+thread_local SplitWorkspace g_split_ws;
+
+// The split-K resident form for 9 <= M <= 16 at K = 14336 (four workgroups of seven waves share a run of four row
+// tiles and take 28 groups of K each; skinny_resident_kernels.h): the GEMV's workgroups each pull their whole
+// activation block out of L2, 459 KB at this K for 115 KB of int4 weights.  Measured at M = 16, N = 4096, int8 / int4:
+// 17.8 -> 14.7 / 13.4 -> 10.9 us; at M = 8 the int8 GEMV is the faster one, at 32 rows the 32-row split form is level.
+bool gemv_split_applies(int M, int N, int K) {
+  if (!g_split_ws.base || g_split_ws.bytes < kSplitWorkspaceBytes) return false;
+  const int ntiles = N / kTileN;
+  return M >= 9 && M <= kMaxGemvM && K == 14336 && ntiles >= kSplitTiles && (ntiles + kSplitTiles - 1) / kSplitTiles <= kSplitMaxCells;
+}
+template <bool kW4, int kEpi>
+int launch_gemv_split(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
+                      int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  constexpr int T = kSplitTiles, kWaves = 7, TPW = 4;
+  const int S = K / kGroup / (kWaves * TPW);
+  const int nruns = (N / kTileN + T - 1) / T;
+  const dim3 grid(8 * ((nruns + 7) / 8) * S), block(kWaves * 64);
+  SkinnySplit sp{reinterpret_cast<float*>(static_cast<char*>(g_split_ws.base) + kSplitTicketBytes),
+                 static_cast<unsigned*>(g_split_ws.base), S};
+  constexpr size_t lds = res_lds_bytes(T, 1, kEpi != 0);
+  if constexpr (kEpi != 0) {
+    auto kernel = dequant_skinny_resident_split_epi_kernel<TPW, T, kW4, kEpi, 1, kWaves>;
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32,
+                       scales8, ep, sp);
+  } else {
+    auto kernel = dequant_skinny_resident_split_kernel<TPW, T, kW4, 1, kWaves>;
+    if (int s = allow_big_lds(kernel, lds)) return s;
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32,
+                       scales8, sp);
+  }
+  return AJQ_OK;
+}
+
 // ---- resident-activation form of the weight-streaming kernel (skinny_resident_kernels.h): K = 2048 or 4096, a
 // run of T row tiles per workgroup, row blocks of 16 MB rows (MB = 1 for the GEMV's M <= 16, 2 above).  T is the
 // shortest run that fits the workgroups into one round of the chip (256: one workgroup per CU); where the longest
@@ -414,6 +460,8 @@ int launch_gemv(const uint16_t* x, int M, int K, const uint32_t* wq, const uint3
   if (gemv_takes_resident(M, N, K))
     return launch_skinny_resident<kW4, 0, 1>(skinny_resident_tiles<kW4, 1>(M, N, K), x, M, K, wq, meta, scales8, N, y, out_f32,
                                              GemvEpilogue{}, stream);
+  if (gemv_split_applies(M, N, K))
+    return launch_gemv_split<kW4, 0>(x, M, K, wq, meta, scales8, N, y, out_f32, GemvEpilogue{}, stream);
   if (K == 8 * 2 * kGroup) {  // K = 2048: one batch of two groups per wave, straight-line kernel
     if (M <= 1) return launch_gemv_cfg<8, 2, 1, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
     if (M <= 2) return launch_gemv_cfg<8, 2, 2, kW4, true>(x, M, K, wq, meta, scales8, N, y, out_f32, stream);
@@ -498,19 +546,6 @@ int launch_skinny_epi_cfg(const uint16_t* x, int M, int K, const uint32_t* wq, c
                      reinterpret_cast<const u32x4_t*>(wq), meta, x, K, M, N, y, out_f32, scales8, ep);
   return AJQ_OK;
 }
-
-// ---- split-K form of the weight-streaming kernel (see kSplitK in skinny_kernels.h): only with a buffer the caller
-// has lent to this host thread's calls (ajq_matmul_workspace_set), which holds the ticket words and the partial sums
-constexpr int kSplitTiles = 4, kSplitWays = 4;          // row tiles per workgroup, workgroups per row-tile group
-constexpr size_t kSplitTicketBytes = 4096;              // one word per (row-tile group, row block), zeroed
-constexpr int kSplitMaxCells = 64;                      // 256 workgroups: one round of the chip
-constexpr size_t kSplitCellBytes = (size_t)kSplitWays * kSplitTiles * 2 * 1024;
-constexpr size_t kSplitWorkspaceBytes = kSplitTicketBytes + kSplitMaxCells * kSplitCellBytes;
-struct SplitWorkspace {
-  void* base = nullptr;
-  size_t bytes = 0;
-};
-thread_local SplitWorkspace g_split_ws;
 
 // Whether the split-K form takes (M, N, K): a lent buffer, one round of workgroups, a K that four workgroups share
 // evenly, and enough of it that the activation traffic saved (each row-tile group of four reads the block once
@@ -662,6 +697,7 @@ bool gemv_rowscale_supported(int M, int K) { return gemv_epi_supported(M, K) && 
 template <bool kW4, int kEpi>
 int launch_gemv_epi(const uint16_t* x, int M, int K, const uint32_t* wq, const uint32_t* meta, const uint16_t* scales8,
                     int N, void* y, int out_f32, const GemvEpilogue& ep, hipStream_t stream) {
+  if (gemv_split_applies(M, N, K)) return launch_gemv_split<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   if (!gemv_epi_straight(M, K)) return launch_skinny_epi<kW4, kEpi>(x, M, K, wq, meta, scales8, N, y, out_f32, ep, stream);
   if (gemv_takes_resident(M, N, K))
     return launch_skinny_resident<kW4, kEpi, 1>(skinny_resident_tiles<kW4, 1>(M, N, K), x, M, K, wq, meta, scales8, N, y, out_f32, ep,

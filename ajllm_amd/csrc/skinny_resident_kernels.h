@@ -69,15 +69,15 @@ __device__ __forceinline__ void wait_rows(u32x4_t (&r)[4]) {
   asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]) : "n"(kLeft) : "memory");
 }
 
-template <int TPW, int T, bool kW4, int kEpi, int MB = 2>
+template <int TPW, int T, bool kW4, int kEpi, int MB = 2, int kWaves = kResWaves, bool kSplitK = false>
 __device__ __forceinline__ void dequant_skinny_resident_body(
     const u32x4_t* __restrict__ wq,
     const uint32_t* __restrict__ meta,     // W4: private meta; W8: unused
     const uint16_t* __restrict__ x, int K, int M, int N, void* __restrict__ y, int out_f32,
     const uint16_t* __restrict__ scales8,  // W8: fp16 [N]; W4: unused
-    const GemvEpilogue& ep) {
+    const GemvEpilogue& ep, const SkinnySplit& sp = SkinnySplit{}) {
+  static_assert(kWaves <= kResWaves, "the LDS regions are laid out for at most eight waves");
   static_assert(T >= 1 && T * MB <= kResMaxUnits, "a wave's region holds the partial sums of T row tiles");
-  constexpr int kWaves = kResWaves;
   constexpr int kLPG = kW4 ? 1 : 2;              // 1 KiB weight tiles per group
   constexpr int kWL = TPW * (kLPG + (kW4 ? 1 : 0));  // loads per wave and row tile
   using Tile = ResidentTile<TPW, kW4>;
@@ -92,14 +92,16 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   constexpr int kRows = 16 * MB;  // rows of a row block
   const int mblocks = (M + kRows - 1) / kRows;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int run = xcd + 8 * (slot / mblocks);
+  // split-K: S workgroups share a run and take 1 / S of K each (consecutive slots of the run's XCD)
+  const int S = kSplitK ? sp.S : 1;
+  const int run = xcd + 8 * (slot / (mblocks * S));
   if (run >= nruns) return;  // padding of the last round (whole workgroup: no barrier is left waiting)
-  const int mblock = slot % mblocks;
+  const int mblock = (slot / S) % mblocks, split = slot % S;
   const int m0 = mblock * kRows;
   const int nt0 = run * T;
   const int tiles = min(T, ntiles - nt0);  // >= 1; past the matrix the last row tile is computed again, not stored
-  const int G = K >> 7;                    // = kWaves * TPW (checked by the host)
-  const int g0 = wave * TPW;
+  const int G = K >> 7;                    // = S * kWaves * TPW (checked by the host)
+  const int g0 = (split * kWaves + wave) * TPW;
   constexpr int kRegionBytes = res_region_bytes(T, MB);
   char* region = reinterpret_cast<char*>(smem_raw) + wave * kRegionBytes;
   uint16_t* xs = reinterpret_cast<uint16_t*>(region);
@@ -124,7 +126,11 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   u32x4_t frag[TPW][4][MB];
   f32x4_t asum[TPW][MB];
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-  Tile set[2];
+  // row tiles in flight: two register sets (four were measured: 3 % faster at K = 2048, 2-4 % slower at K = 4096,
+  // and with 32 rows they do not fit the register file)
+  constexpr int kSets = T < 2 ? T : 2;
+  static_assert(kSets >= 1 && kSets <= 4, "the waits below count up to three tiles behind the current one");
+  Tile set[kSets];
   {
     // all requests of the prologue are asm, so that every wait is exact: the activations (L2 hits) come back while
     // the first row tile's weights are still on their way from memory
@@ -140,9 +146,9 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
     for (int p = 0; p < TPW; ++p)
 #pragma unroll
       for (int i = 0; i < kXL; ++i) load16_async(raw[p][i], reinterpret_cast<const char*>(x) + (g0 + p) * (kGroup * 2), xoff[i]);
-    request(set[0], 0);
-    if (T > 1) request(set[1], 1);  // two row tiles' weights travel while the activations are staged
-    constexpr int kAhead = (T > 1 ? 2 : 1) * kWL;
+#pragma unroll
+    for (int t = 0; t < kSets; ++t) request(set[t], t);  // the first row tiles' weights travel while the activations are staged
+    constexpr int kAhead = kSets * kWL;
 #pragma unroll
     for (int p = 0; p < TPW; ++p) {
       if (p == 0) wait_rows<kAhead + kXL * (TPW - 1)>(raw[0]);
@@ -172,7 +178,7 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
 
   // ---- row scale: this wave's share of the sums of squares of the block's 32 rows (lane -> row lane & 31, the two
   // half-waves take alternate 16-byte pieces), used at the end
-  constexpr int kShareLoads = 32 / kWaves;
+  constexpr int kShareLoads = (32 + kWaves - 1) / kWaves;
   float4 ssq_share[kShareLoads];
   float* red2 = reinterpret_cast<float*>(reinterpret_cast<char*>(smem_raw) + kWaves * kRegionBytes);  // [32][kWaves]
   if (kEpi & kEpiRowScale) {
@@ -231,12 +237,14 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   // between the request and the wait, while the loads are still in flight.
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    if (t + 1 < T)
-      wait_tile<kWL>(set[t & 1]);
-    else
-      wait_tile<0>(set[t & 1]);
-    compute(set[t & 1], t);
-    if (t + 2 < T) request(set[t & 1], t + 2);
+    // in flight behind tile t: the tiles up to t + kSets - 1 that exist
+    const int behind = t + kSets - 1 < T ? kSets - 1 : T - 1 - t;  // (a constant once the loop is unrolled)
+    if (behind == 0) wait_tile<0>(set[t % kSets]);
+    if (behind == 1) wait_tile<kWL>(set[t % kSets]);
+    if (behind == 2) wait_tile<2 * kWL>(set[t % kSets]);
+    if (behind == 3) wait_tile<3 * kWL>(set[t % kSets]);
+    compute(set[t % kSets], t);
+    if (t + kSets < T) request(set[t % kSets], t + kSets);
   }
 
   if (kEpi & kEpiRowScale) {
@@ -248,8 +256,7 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
   }
   __syncthreads();
   // ---- the (row tile, 16-row block) units, dealt round-robin to the waves: the waves' partial sums in wave order
-  for (int u = wave; u < MB * tiles; u += kWaves) {
-    const int t = u / MB, r = u % MB;
+  auto unit_sum = [&](int u) -> f32x4_t {
     f32x4_t part[kWaves];
 #pragma unroll
     for (int w = 0; w < kWaves; ++w)
@@ -257,6 +264,49 @@ __device__ __forceinline__ void dequant_skinny_resident_body(
     f32x4_t sum = part[0];
 #pragma unroll
     for (int w = 1; w < kWaves; ++w) sum += part[w];
+    return sum;
+  };
+  const unsigned long long* cell_partial = nullptr;  // split-K: [S][T * MB][64] f32x4 of this (run, row block)
+  if constexpr (kSplitK) {
+    // the exchange of dequant_skinny_kernel's split-K form: partial sums as device-scope relaxed atomic stores
+    // (written through the L2, which is not coherent across XCDs), complete at the workgroup barrier; a ticket;
+    // the workgroup that draws the last one adds the S partial results in split order and leaves the ticket zero
+    __shared__ unsigned drawn;
+    const int cell = run * mblocks + mblock;
+    unsigned long long* mine_out = reinterpret_cast<unsigned long long*>(sp.partial) + (size_t)cell * S * (T * MB * 128);
+    cell_partial = mine_out;
+    for (int u = wave; u < MB * tiles; u += kWaves) {
+      const f32x4_t v = unit_sum(u);
+      unsigned long long* dst = mine_out + (((size_t)split * T * MB + u) * 64 + lane) * 2;
+      __hip_atomic_store(dst, (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 1, (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32),
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) drawn = __hip_atomic_fetch_add(sp.tickets + cell, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (drawn != (unsigned)(S - 1)) return;
+    if (threadIdx.x == 0) __hip_atomic_store(sp.tickets + cell, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (int u = wave; u < MB * tiles; u += kWaves) {
+    const int t = u / MB, r = u % MB;
+    f32x4_t sum;
+    if constexpr (kSplitK) {
+      const unsigned long long* src = cell_partial + ((size_t)u * 64 + lane) * 2;
+      auto fetch = [&](int q) -> f32x4_t {
+        const unsigned long long* at = src + (size_t)q * T * MB * 128;
+        const unsigned long long lo = __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi = __hip_atomic_load(at + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return f32x4_t{__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)), __uint_as_float((uint32_t)hi),
+                       __uint_as_float((uint32_t)(hi >> 32))};
+      };
+      sum = fetch(0);
+      for (int q = 1; q < S; ++q) sum += fetch(q);
+    } else {
+      sum = unit_sum(u);
+    }
     float rstd[4] = {1.0f, 1.0f, 1.0f, 1.0f};
     if (kEpi & kEpiRowScale) {
 #pragma unroll
@@ -283,6 +333,21 @@ __global__ __launch_bounds__(kResWaves * 64, 2) void dequant_skinny_resident_epi
     const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
     void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep) {
   dequant_skinny_resident_body<TPW, T, kW4, kEpi, MB>(wq, meta, x, K, M, N, y, out_f32, scales8, ep);
+}
+
+// the split-K forms: seven waves of TPW groups per workgroup and K-part (K = 14336: four parts of 28 groups)
+template <int TPW, int T, bool kW4, int MB, int kWaves>
+__global__ __launch_bounds__(kWaves * 64, 2) void dequant_skinny_resident_split_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, SkinnySplit sp) {
+  dequant_skinny_resident_body<TPW, T, kW4, 0, MB, kWaves, true>(wq, meta, x, K, M, N, y, out_f32, scales8, GemvEpilogue{}, sp);
+}
+
+template <int TPW, int T, bool kW4, int kEpi, int MB, int kWaves>
+__global__ __launch_bounds__(kWaves * 64, 2) void dequant_skinny_resident_split_epi_kernel(
+    const u32x4_t* __restrict__ wq, const uint32_t* __restrict__ meta, const uint16_t* __restrict__ x, int K, int M, int N,
+    void* __restrict__ y, int out_f32, const uint16_t* __restrict__ scales8, GemvEpilogue ep, SkinnySplit sp) {
+  dequant_skinny_resident_body<TPW, T, kW4, kEpi, MB, kWaves, true>(wq, meta, x, K, M, N, y, out_f32, scales8, ep, sp);
 }
 
 }  // namespace ajq

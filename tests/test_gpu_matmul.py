@@ -280,7 +280,7 @@ class _LentWorkspace:
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 4096, 14336), (17, 4096, 14336), (32, 4000, 8192), (24, 1040, 16384),
-                                   (32, 64, 8704)])
+                                   (32, 64, 8704), (16, 4096, 14336), (9, 4000, 14336), (13, 64, 14336)])
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_batched_decode_matmul_split_along_k(cuda, scheme, m, n, k):
     """The weight-streaming kernel with four workgroups per group of four row tiles, a quarter of K each, and the
@@ -289,7 +289,8 @@ def test_batched_decode_matmul_split_along_k(cuda, scheme, m, n, k):
     buffer's ticket words zero again afterwards; no trace of the previous call's partial sums when calls on
     different matrices alternate on one buffer.  K = 14336 and 16384 take the straight-line kernels (seven and eight
     waves' runs of four groups), 8192 and 8704 the loop; N = 4000 and 1040 end in a group of fewer than four row
-    tiles."""
+    tiles.  With 9 <= M <= 16 at K = 14336 the same exchange runs behind the resident-activation form with one
+    16-row block (in place of the GEMV)."""
     w_hat, wq, meta = _quantized(scheme, n, k, 31, cuda)
     x = make_activations(m, k, 131, True).to(cuda)
     plain = _run(scheme, x, wq, meta, torch.float32, "gemm")
@@ -309,15 +310,16 @@ def test_batched_decode_matmul_split_along_k(cuda, scheme, m, n, k):
     assert torch.equal(plain, _run(scheme, x, wq, meta, torch.float32, "gemm"))
 
 
+@pytest.mark.parametrize("m", [32, 16, 11])
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
-def test_split_along_k_with_the_residual_epilogue(cuda, scheme):
+def test_split_along_k_with_the_residual_epilogue(cuda, scheme, m):
     """ajq_w*a16_gemv_residual (w2 of a batched decode step: K = 14336) through the split form: the new residual
     stream is the plain split matmul's output added to h_in bit for bit, its bf16 image and the sums of squares
     follow from it."""
     from ajllm_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
-    m, d, k = 32, 4096, 14336
+    d, k = 4096, 14336
     w_hat, wq, meta = _quantized(scheme, d, k, 31, cuda)
     g = torch.Generator().manual_seed(5)
     x = make_activations(m, k, 17, True).to(cuda)
