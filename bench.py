@@ -120,8 +120,12 @@ def time_graph_steps(step_fn, steps: int, warmup: int) -> float:
     return start.elapsed_time(stop) / 1e3
 
 
-def bench_gemv(scheme: str, m: int, n: int, k: int, copies: int, steps: int, warmup: int, device) -> dict:
-    from ajllm_amd import w4a16_matmul, w8a16_matmul
+def bench_gemv(scheme: str, m: int, n: int, k: int, copies: int, steps: int, warmup: int, device,
+               lend_workspace: bool = False) -> dict:
+    """One launch per matrix through the C ABI, `copies` distinct matrices per step.  lend_workspace: with the
+    caller-lent buffer of ajq_matmul_workspace_set in place (as the decoders run), which lets shapes with a long K
+    split K over workgroups."""
+    from ajllm_amd import _lib, w4a16_matmul, w8a16_matmul
 
     weights = make_w4(n, k, copies, device, 1234) if scheme == "w4" else make_w8(n, k, copies, device, 1234)
     x = make_x(m, k, device, 99)
@@ -134,13 +138,24 @@ def bench_gemv(scheme: str, m: int, n: int, k: int, copies: int, steps: int, war
         for a, b in weights:
             outs.append(fn(x, a, b, torch.bfloat16, kernel="gemv"))
 
-    seconds = time_graph_steps(step, steps, warmup)
+    lib = _lib.load()
+    lent = torch.zeros(int(lib.ajq_matmul_workspace_bytes()), dtype=torch.uint8, device=device) if lend_workspace else None
+    if lent is not None:
+        _lib.check(lib.ajq_matmul_workspace_set(lent.data_ptr(), lent.numel()), "matmul_workspace_set")
+    try:
+        seconds = time_graph_steps(step, steps, warmup)
+    finally:
+        if lent is not None:
+            lib.ajq_matmul_workspace_set(None, 0)
     launches = steps * copies
     us = seconds / launches * 1e6
     gbs = nbytes / (seconds / launches) / 1e9
-    return {"scheme": scheme, "M": m, "N": n, "K": k, "launches": launches, "us_per_launch": us,
-            "bytes_per_launch": nbytes, "GB/s": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-            "ms_per_step": seconds / steps * 1e3}
+    row = {"scheme": scheme, "M": m, "N": n, "K": k, "launches": launches, "us_per_launch": us,
+           "bytes_per_launch": nbytes, "GB/s": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+           "ms_per_step": seconds / steps * 1e3}
+    if lend_workspace:
+        row["matmul_workspace"] = "lent (ajq_matmul_workspace_set)"
+    return row
 
 
 def bench_gemm(scheme: str, m: int, n: int, k: int, steps: int, warmup: int, device, copies: int = 4) -> dict:
@@ -451,6 +466,13 @@ def main() -> int:
                     log("sweep", json.dumps(r))
                     sweep.append(r)
         extras["decode_sweep"] = sweep
+        # the rows that change when the caller lends the matmul workspace (K = 14336 at 9 to 16 rows)
+        lent_rows = []
+        for scheme in ("w4", "w8"):
+            r = bench_gemv(scheme, 16, 4096, 14336, 10, max(5, args.steps // 5), 2, device, lend_workspace=True)
+            log("sweep, workspace lent", json.dumps(r))
+            lent_rows.append(r)
+        extras["decode_sweep_workspace_lent"] = lent_rows
         gemm = []
         for scheme in ("w4", "w8"):
             for sm in (256, 2048, 8192):

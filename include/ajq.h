@@ -221,11 +221,11 @@ int ajq_w4a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const ui
 int ajq_w8a16_gemm(const uint16_t* x, int M, int K, const uint32_t* wq, const uint16_t* scales, int N,
                    void* y, int out_dtype, void* stream);
 
-/* A device buffer lent to the matmul entry points called from THIS host thread (all of ajq_w*a16_gemm, _gemv_residual,
- * _gemv_gated, _gemv_rowscale, _gemv_norm_sums), for the split-K form of the weight-streaming kernel: at 17 <= M <= 32
- * with K >= 8192 and N <= 4096 (the down projection of a SwiGLU feed-forward in a batched decode step) four workgroups
- * share four row tiles and a quarter of K each, exchange their partial sums through this buffer and the last one to
- * arrive adds them in a fixed order (results are run-to-run identical; they differ from the unsplit kernel's in the
+/* A device buffer lent to the matmul entry points called from THIS host thread (all of ajq_w*a16_gemm, _gemv, _gemv_residual,
+ * _gemv_gated, _gemv_rowscale, _gemv_norm_sums), for the split-K forms of the weight-streaming kernels: at 17 <= M <= 32
+ * with K >= 8192, and at 9 <= M <= 16 with K = 14336, both with N <= 4096 (the down projection of a SwiGLU feed-forward
+ * in a batched decode step), four workgroups share four row tiles and a quarter of K each, exchange their partial sums
+ * through this buffer and the last one to arrive adds them in a fixed order (results are run-to-run identical; they differ from the unsplit kernel's in the
  * last bits, the sum being associated differently).  No counterpart in the reference.
  *   - ajq_matmul_workspace_bytes() bytes, 16-byte aligned; its first 4096 bytes must be ZERO when it is lent (the
  *     kernels leave them zero) and the buffer must stay allocated while launches that were given it can still run
