@@ -342,12 +342,15 @@ def test_split_along_k_with_the_residual_epilogue(cuda, scheme, m):
 
 
 @pytest.mark.parametrize("m,n,k", [(32, 28672, 4096), (17, 14336, 4096), (64, 16 * 1001, 4096), (33, 16 * 513, 2048),
-                                   (100, 8192, 2048), (127, 16 * 131, 4096)])
+                                   (100, 8192, 2048), (127, 16 * 131, 4096), (17, 16, 2048), (31, 48, 4096),
+                                   (127, 4096 + 16, 4096), (16, 16 * 257, 2048), (9, 16 * 4100, 4096), (12, 16 * 700, 4096)])
 @pytest.mark.parametrize("scheme", ["w4", "w8"])
 def test_batched_decode_matmul_many_row_tiles(cuda, scheme, m, n, k):
     """Several 16-row tiles of N per CU at K = 2048 / 4096: the weight-streaming form that keeps a workgroup's
     activation block resident in registers and walks a run of 4, 7 or 8 row tiles past it (w1 | w3 of config 5 at
-    32 rows, a run count that does not divide the tiles, several row blocks, the last one ragged).  The plain
+    32 rows, a run count that does not divide the tiles, several row blocks, the last one ragged; a single row tile;
+    more workgroups than one round of the chip holds; with 9 to 16 rows the form with one 16-row block that takes the
+    GEMV's wide matrices, up to its longest run of 16 row tiles).  The plain
     product against the oracle, then ajq_w*a16_gemv_gated on the same operands: bf16(silu(a) * u) over tiles of
     8 gate rows and 8 up rows, from the same fp32 values."""
     from ajllm_amd import _lib
