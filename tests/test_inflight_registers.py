@@ -26,6 +26,24 @@ template __global__ void dequant_skinny_resident_split_epi_kernel<4, 4, false, 2
 """
 
 
+# the tile GEMMs keep asm-issued weight loads in flight around their main loops (one linear pass over each loop body)
+TILE_SOURCE = """
+#include <hip/hip_runtime.h>
+#include "ajq_common.h"
+#include "gemm_kernels.h"
+#include "gemm_ring_kernels.h"
+#include "gemm_split_kernels.h"
+#include "gemm_wide_kernels.h"
+namespace ajq {
+#define TILE const uint16_t*, int, int, const u32x4_t*, const uint32_t*, const uint16_t*, int, void*, int
+template __global__ void dequant_gemm256w_kernel<false, false>(TILE);
+template __global__ void dequant_gemm256w_kernel<true, true>(TILE);
+template __global__ void dequant_gemm256s_kernel<true, false>(TILE);
+template __global__ void dequant_gemm256r_w8_kernel<false>(const uint16_t*, int, int, const u32x4_t*, const uint16_t*, int, void*, int);
+}
+"""
+
+
 def test_the_scan_flags_a_copy_between_a_load_and_its_wait():
     listing = """
 _Z3badv:
@@ -56,5 +74,13 @@ _Z4goodv:
 def test_resident_kernels_leave_registers_of_loads_in_flight_alone():
     found = asm_check.scan(asm_check.compile_device_asm(SOURCE), "dequant_skinny_resident")
     assert len(found) == 8, sorted(found)
+    offending = {name: lines[:3] for name, lines in found.items() if lines}
+    assert not offending, offending
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_tile_gemm_kernels_leave_registers_of_loads_in_flight_alone():
+    found = asm_check.scan(asm_check.compile_device_asm(TILE_SOURCE), "dequant_gemm256")
+    assert len(found) == 4, sorted(found)
     offending = {name: lines[:3] for name, lines in found.items() if lines}
     assert not offending, offending
