@@ -1,4 +1,6 @@
 // Batched-decode dequant matmul, 17 <= M < 256:  y[M, N] = x[M, K] @ W_hat[N, K]^T.
+// The form for any K (K = 2048 and 4096 run skinny_resident_kernels.h, which keeps the activations in registers), the
+// 32-row split-K form, and the epilogue both forms share (skinny_finish_unit).
 //
 // Still bound by the weight stream (a 4096 x 4096 int8 matrix is 16 MB, 32 rows of
 // activations are 256 KB), so this is the decode GEMV's layout with more rows:
